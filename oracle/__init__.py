@@ -1,0 +1,232 @@
+"""ctypes front end of the CPU checker (oracle/nncv_oracle.c).
+
+TEST INFRASTRUCTURE ONLY.  May be imported by tests/, by __graft_entry__.smoke() and by the
+cpu_baseline leg of bench.py — never by nncv_amd/ (the product fails loudly without its HIP
+library instead of falling back to this).
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+_HWP = None
+_REF = None
+
+_f32p = np.ctypeslib.ndpointer(dtype=np.float32, flags="C_CONTIGUOUS")
+_f64p = np.ctypeslib.ndpointer(dtype=np.float64, flags="C_CONTIGUOUS")
+_int = ctypes.c_int
+_i64 = ctypes.c_int64
+
+
+def build(force=False):
+    """Compile the checker with the Makefile beside this file."""
+    if force or not os.path.exists(os.path.join(_HERE, "liboracle.so")) \
+            or not os.path.exists(os.path.join(_HERE, "libhostwparallel.so")):
+        subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s"])
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        build()
+        L = ctypes.CDLL(os.path.join(_HERE, "liboracle.so"))
+        L.orc_conv2d_nchw_fchw.argtypes = [_f32p, _f32p, _f32p] + [_int] * 9
+        L.orc_matmul.argtypes = [_f32p, _f32p, _f32p, _int, _int, _int]
+        L.orc_pad_nchw.argtypes = [_f32p, _f32p, _int, _int, _int, _int, _int, ctypes.c_float]
+        L.orc_batchnorm_nchw.argtypes = [_f32p] * 6 + [_int] * 3
+        L.orc_relu.argtypes = [_f32p, _f32p, _i64]
+        L.orc_add.argtypes = [_f32p, _f32p, _f32p, _i64]
+        L.orc_maxpool_nchw.argtypes = [_f32p, _f32p] + [_int] * 8
+        L.orc_global_avgpool_nchw.argtypes = [_f32p, _f32p] + [_int] * 4
+        L.orc_fc.argtypes = [_f32p] * 4 + [_int] * 3
+        L.orc_wino43_filter_transform.argtypes = [_f32p, _f64p, _int, _int]
+        L.orc_wino43_input_transform.argtypes = [_f32p, _f64p] + [_int] * 5
+        L.orc_wino43_batched_gemm.argtypes = [_f64p, _f64p, _f64p, _i64, _int, _int]
+        L.orc_wino43_output_transform.argtypes = [_f64p, _f32p] + [_int] * 4
+        L.orc_conv3x3_winograd43.argtypes = [_f32p, _f32p, _f32p] + [_int] * 6
+        L.orc_resnet18_forward.argtypes = [_f32p, _int, _int, _int, _f32p, _f32p, _int,
+                                           ctypes.c_void_p]
+        L.orc_resnet18_forward.restype = _int
+        L.orc_resnet18_num_params.restype = _i64
+        _LIB = L
+    return _LIB
+
+
+def _c(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def conv2d_nchw_fchw(x_padded, w, stride=1, out=None):
+    """out + conv(x_padded, w); x is already padded (linalg.conv_2d_nchw_fchw)."""
+    x_padded, w = _c(x_padded), _c(w)
+    N, C, H, W = x_padded.shape
+    F, C2, R, S = w.shape
+    assert C == C2
+    OH, OW = (H - R) // stride + 1, (W - S) // stride + 1
+    y = np.zeros((N, F, OH, OW), np.float32) if out is None else _c(out).copy()
+    assert y.shape == (N, F, OH, OW)
+    lib().orc_conv2d_nchw_fchw(x_padded, w, y, N, C, H, W, F, R, S, stride, stride)
+    return y
+
+
+def pad_nchw(x, pad, value=0.0):
+    x = _c(x)
+    N, C, H, W = x.shape
+    y = np.empty((N, C, H + 2 * pad, W + 2 * pad), np.float32)
+    lib().orc_pad_nchw(x, y, N, C, H, W, pad, value)
+    return y
+
+
+def matmul(a, b, c=None):
+    a, b = _c(a), _c(b)
+    M, K = a.shape
+    K2, N = b.shape
+    assert K == K2
+    y = np.zeros((M, N), np.float32) if c is None else _c(c).copy()
+    lib().orc_matmul(a, b, y, M, N, K)
+    return y
+
+
+def batchnorm(x, gamma, beta, mean, var):
+    x = _c(x)
+    N, C = x.shape[:2]
+    y = np.empty_like(x)
+    lib().orc_batchnorm_nchw(x, _c(gamma), _c(beta), _c(mean), _c(var), y, N, C,
+                             int(np.prod(x.shape[2:])))
+    return y
+
+
+def relu(x):
+    x = _c(x)
+    y = np.empty_like(x)
+    lib().orc_relu(x, y, x.size)
+    return y
+
+
+def maxpool3x3s2(x):
+    """-inf pad 1, 3x3 window, stride 2 (Res18.mlir:144-151)."""
+    xp = pad_nchw(x, 1, -np.inf)
+    N, C, H, W = xp.shape
+    OH, OW = (H - 3) // 2 + 1, (W - 3) // 2 + 1
+    y = np.full((N, C, OH, OW), -np.inf, np.float32)
+    lib().orc_maxpool_nchw(xp, y, N, C, H, W, 3, 3, 2, 2)
+    return y
+
+
+def global_avgpool(x):
+    x = _c(x)
+    N, C, H, W = x.shape
+    y = np.empty((N, C), np.float32)
+    lib().orc_global_avgpool_nchw(x, y, N, C, H, W)
+    return y
+
+
+def fc(x, w, b):
+    x, w, b = _c(x), _c(w), _c(b)
+    y = np.empty((x.shape[0], w.shape[0]), np.float32)
+    lib().orc_fc(x, w, b, y, x.shape[0], x.shape[1], w.shape[0])
+    return y
+
+
+def wino43_filter_transform(w):
+    w = _c(w)
+    F, C = w.shape[:2]
+    U = np.empty((36, F, C), np.float64)
+    lib().orc_wino43_filter_transform(w, U, F, C)
+    return U
+
+
+def wino43_input_transform(x, pad=1):
+    x = _c(x)
+    N, C, H, W = x.shape
+    OH, OW = H + 2 * pad - 2, W + 2 * pad - 2
+    tiles = N * ((OH + 3) // 4) * ((OW + 3) // 4)
+    V = np.empty((36, tiles, C), np.float64)
+    lib().orc_wino43_input_transform(x, V, N, C, H, W, pad)
+    return V
+
+
+def wino43_batched_gemm(V, U):
+    tiles, C = V.shape[1:]
+    F = U.shape[1]
+    M = np.empty((36, tiles, F), np.float64)
+    lib().orc_wino43_batched_gemm(np.ascontiguousarray(V), np.ascontiguousarray(U), M, tiles, C, F)
+    return M
+
+
+def wino43_output_transform(M, N, OH, OW, out=None):
+    F = M.shape[2]
+    y = np.zeros((N, F, OH, OW), np.float32) if out is None else _c(out).copy()
+    lib().orc_wino43_output_transform(np.ascontiguousarray(M), y, N, F, OH, OW)
+    return y
+
+
+def conv3x3_winograd43(x, w, pad=1):
+    x, w = _c(x), _c(w)
+    N, C, H, W = x.shape
+    F = w.shape[0]
+    y = np.zeros((N, F, H + 2 * pad - 2, W + 2 * pad - 2), np.float32)
+    lib().orc_conv3x3_winograd43(x, w, y, N, C, H, W, F, pad)
+    return y
+
+
+def resnet18_forward(x, params, tap_layer=-1):
+    """x [N,3,H,W] fp32, params flat fp32 blob (canonical order) -> logits [N,1000]
+    (and the tapped NCHW activation when tap_layer >= 0)."""
+    x, params = _c(x), _c(params)
+    N, C, H, W = x.shape
+    assert C == 3 and params.size == lib().orc_resnet18_num_params()
+    y = np.empty((N, 1000), np.float32)
+    tap = None
+    tp = None
+    if tap_layer >= 0:
+        ch = [64, 64, 128, 256, 512][tap_layer]
+        h = H // 4 if tap_layer == 0 else H // (4 * 2 ** (tap_layer - 1))
+        tap = np.empty((N, ch, h, h * W // H), np.float32)
+        tp = tap.ctypes.data_as(ctypes.c_void_p)
+    rc = lib().orc_resnet18_forward(x, N, H, W, params, y, tap_layer, tp)
+    assert rc == 0
+    return (y, tap) if tap_layer >= 0 else y
+
+
+# ---- reference-built model.bin reader/writer (oracle/_ref), present only where it was built ----
+def ref_lib():
+    global _REF
+    if _REF is None:
+        p = os.path.join(_HERE, "_ref", "libnncv_rt_ref.so")
+        if not os.path.exists(p):
+            return None
+        R = ctypes.CDLL(p)
+        R.ref_modelbin_read_f32.restype = ctypes.c_longlong
+        R.ref_modelbin_read_f32.argtypes = [ctypes.c_char_p, _f32p, ctypes.c_longlong]
+        R.ref_sizeof_descriptor.restype = ctypes.c_size_t
+        R.ref_sizeof_indexer.restype = ctypes.c_size_t
+        R.ref_sizeof_head.restype = ctypes.c_size_t
+        _REF = R
+    return _REF
+
+
+def ref_modelbin_write_f32(path, tensors):
+    """tensors: list of (name, ndarray fp32).  Uses the reference's own writer."""
+    R = ref_lib()
+    n = len(tensors)
+    names = (ctypes.c_char_p * n)(*[t[0].encode() for t in tensors])
+    dims = (ctypes.c_size_t * n)(*[t[1].ndim for t in tensors])
+    shapes = (ctypes.c_size_t * (8 * n))()
+    arrs = [np.ascontiguousarray(t[1], np.float32) for t in tensors]
+    for i, a in enumerate(arrs):
+        for d, s in enumerate(a.shape):
+            shapes[i * 8 + d] = s
+    ptrs = (ctypes.POINTER(ctypes.c_float) * n)(
+        *[a.ctypes.data_as(ctypes.POINTER(ctypes.c_float)) for a in arrs])
+    return R.ref_modelbin_write_f32(path.encode(), n, names, dims, shapes, ptrs)
+
+
+def ref_modelbin_read_f32(path, cap):
+    R = ref_lib()
+    out = np.zeros(cap, np.float32)
+    n = R.ref_modelbin_read_f32(path.encode(), out, cap)
+    return n, out

@@ -1,0 +1,100 @@
+"""model.bin byte format: the package's reader/writer against the README layout, against the
+reference's own compiled reader/writer (oracle/_ref, where it was built) and against a fixture
+that writer produced."""
+import os
+import struct
+
+import numpy as np
+import pytest
+
+import oracle
+from nncv_amd import modelbin, resnet18_spec as spec, synth
+
+
+def small_tensors():
+    return [("conv.weight", synth.normal(1, (2, 3, 3, 3))),
+            ("bn.weight", synth.uniform(2, (2,), 0.5, 1.5)),
+            ("fc.weight", synth.normal(3, (5, 4)))]
+
+
+def test_layout_by_hand(tmp_path):
+    p = str(tmp_path / "m.bin")
+    ts = small_tensors()
+    modelbin.write(p, ts)
+    raw = open(p, "rb").read()
+    assert struct.unpack_from("<qQQ", raw, 0) == (0x42, 24, 3)
+    assert len(raw) == 24 + 3 * 224 + 4 * (54 + 2 + 20)
+    # indexer 2: name @0, dims @128, shape @136, eleWidth @200, aligned @208, dataOffset @216
+    base = 24 + 2 * 224
+    assert raw[base:base + 9] == b"fc.weight"
+    assert struct.unpack_from("<Q", raw, base + 128)[0] == 2
+    assert struct.unpack_from("<2Q", raw, base + 136) == (5, 4)
+    assert struct.unpack_from("<Q", raw, base + 200)[0] == 4
+    assert struct.unpack_from("<Q", raw, base + 216)[0] == 24 + 3 * 224 + 4 * 56
+    data = np.frombuffer(raw, np.float32, offset=24 + 3 * 224)
+    assert np.array_equal(data[56:], ts[2][1].reshape(-1))
+
+
+def test_roundtrip_and_errors(tmp_path):
+    p = str(tmp_path / "m.bin")
+    ts = small_tensors()
+    modelbin.write(p, ts)
+    index, blob = modelbin.read(p)
+    assert [(n, s) for n, s, _ in index] == [(n, a.shape) for n, a in ts]
+    assert np.array_equal(blob, np.concatenate([a.reshape(-1) for _, a in ts]))
+    assert modelbin.read(str(tmp_path / "missing.bin")) is None
+    bad = bytearray(open(p, "rb").read())
+    bad[0] = 0x41
+    open(p, "wb").write(bad)
+    assert modelbin.read(p) is None  # bad magic -> the reference returns false
+
+
+def test_fp16_extension(tmp_path):
+    p = str(tmp_path / "h.bin")
+    ts = small_tensors()
+    modelbin.write(p, ts, np.float16)
+    index, blob = modelbin.read(p, np.float16)
+    assert all(w == 2 for _, _, w in index)
+    assert np.array_equal(blob, np.concatenate([a.reshape(-1) for _, a in ts]).astype(np.float16))
+
+
+def test_committed_fixture_from_reference_writer(golden_dir):
+    """tests/golden/ref_writer_small.bin was written by the reference's MemRefFlatArray::write
+    (see tests/golden/make_modelbin_fixture.py)."""
+    p = os.path.join(golden_dir, "ref_writer_small.bin")
+    index, blob = modelbin.read(p)
+    ts = small_tensors()
+    assert [(n, s, w) for n, s, w in index] == [(n, a.shape, 4) for n, a in ts]
+    assert np.array_equal(blob, np.concatenate([a.reshape(-1) for _, a in ts]))
+    # and this package's writer reproduces the file byte for byte
+    import tempfile
+    with tempfile.TemporaryDirectory() as d:
+        q = os.path.join(d, "mine.bin")
+        modelbin.write(q, ts)
+        assert open(q, "rb").read() == open(p, "rb").read()
+
+
+@pytest.mark.skipif(oracle.ref_lib() is None, reason="oracle/_ref not built (no reference tree)")
+def test_against_live_reference_reader_writer(tmp_path):
+    R = oracle.ref_lib()
+    assert R.ref_sizeof_head() == 24 and R.ref_sizeof_indexer() == 224
+    assert [R.ref_sizeof_descriptor(r) for r in (1, 2, 4)] == [40, 56, 88]
+    ts = small_tensors()
+    mine, theirs = str(tmp_path / "a.bin"), str(tmp_path / "b.bin")
+    modelbin.write(mine, ts)
+    assert oracle.ref_modelbin_write_f32(theirs, ts) == 0
+    assert open(mine, "rb").read() == open(theirs, "rb").read()
+    n, blob = oracle.ref_modelbin_read_f32(mine, 100)
+    assert n == 76 and np.array_equal(blob[:76], np.concatenate([a.reshape(-1) for _, a in ts]))
+
+
+def test_resnet18_table():
+    t = spec.tensor_table()
+    assert len(t) == spec.NUM_TENSORS == 102
+    assert sum(spec.numel(s) for _, s in t) == spec.NUM_ELEMENTS == 11699112
+    off = spec.offsets()
+    assert off["layer1.0.conv1.weight"][0] == 9664
+    assert off["layer4.1.conv2.weight"][0] == 8824768
+    assert off["fc.bias"][0] == 11698112
+    assert abs(spec.flops_per_image(224) / 1e9 - 3.628) < 1e-3
+    assert abs(spec.flops_per_image(256) / 1e9 - 4.738) < 1e-3

@@ -1,0 +1,122 @@
+/*
+ * nncv_hip.h — C ABI of libnncv_hip.so, the MI355X (gfx950) implementation of nncv's
+ * conv / GEMM / ResNet-18 hot path.
+ *
+ * Part 1 declares the symbols a program built against nncv already binds; replacing the object
+ * file nncv-c produced (libres18.o) by this library needs no source change.
+ * Part 2 declares device-resident forms of the same operations for callers that keep data in
+ * HBM (benchmarks, serving loops); they have no counterpart in the reference, whose object only
+ * knows host memory.
+ *
+ * All pointers are plain C; no C++ or framework types cross this boundary.
+ */
+#ifndef NNCV_HIP_H_
+#define NNCV_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* MLIR strided memref descriptors, byte-identical to nncv::rt::MemRefDescriptor<T,N>
+ * (include/libnncv/DataType.hpp:129-136): sizeof = 40 / 56 / 88 bytes for rank 1 / 2 / 4.
+ * Element i.. is aligned[offset + sum_k i_k * strides[k]]; strides are in elements. */
+typedef struct { void* allocated; void* aligned; intptr_t offset; intptr_t sizes[1]; intptr_t strides[1]; } nncv_memref1d;
+typedef struct { void* allocated; void* aligned; intptr_t offset; intptr_t sizes[2]; intptr_t strides[2]; } nncv_memref2d;
+typedef struct { void* allocated; void* aligned; intptr_t offset; intptr_t sizes[4]; intptr_t strides[4]; } nncv_memref4d;
+
+/* ---------------------------------------------------------------------------------------------
+ * Part 1 — the reference's ABI
+ * ------------------------------------------------------------------------------------------- */
+
+/* ResNet-18 forward, fp32, compiled with -split-params -wrap-c-interface.
+ * Replaces the symbol declared in examples/Res18/main.cpp:18-23 and called at :96.
+ *   dst    out: [N,1000]; the callee mallocs the buffer (64-byte aligned) and overwrites *dst,
+ *          as MLIR's C interface does; the caller owns it afterwards.
+ *   src    in : [N,3,H,W] NCHW host memory, any strides.
+ *   params nncv_memref1d* over the flat model.bin blob (MemRefFlatArray::get(),
+ *          src/libnncv/DataType.cpp:89-96), 11 699 112 fp32 elements in the canonical order
+ *          (torchvision state_dict order without num_batches_tracked).
+ * Errors (HIP failure, wrong parameter count, bad shape) print one "[ Erro ]" line to stderr and
+ * abort(), the reference's convention (DnnModelLowering.cpp:222-230). */
+void _mlir_ciface_forward(nncv_memref2d* dst, nncv_memref4d* src, void* params);
+
+/* Same network from tests/Nets/Res18-half.mlir: every element is an IEEE half (uint16_t bits,
+ * nncvFloat16 of DataType.hpp:127).  The reference object for it would carry the same symbol
+ * name as the fp32 one; one library cannot export both, hence the suffix. fp32 accumulation. */
+void _mlir_ciface_forward_f16(nncv_memref2d* dst, nncv_memref4d* src, void* params);
+
+/* linalg.matmul: res = c + a.b, fp32 row-major (tests/MatMulOptimization/MatMulDeafult.mlir:6-9).
+ * The product is accumulated into c's buffer in place and *res aliases it. */
+void _mlir_ciface_matmul(nncv_memref2d* res, nncv_memref2d* a, nncv_memref2d* b, nncv_memref2d* c);
+
+/* linalg.conv_2d_nchw_fchw: res = out + conv(in, filter), fp32, `in` already padded
+ * (tests/ConvOptimization/Conv2dNchwFchwManually.mlir:7-13).  The stride is a compile-time
+ * attribute in the reference; here it is recovered from the shapes:
+ * stride = (H - R) / (OH - 1) (1 when OH == 1), and the shapes must then be consistent.
+ * Accumulates into out's buffer in place; *res aliases it. */
+void _mlir_ciface_batch_nchw_conv(nncv_memref4d* res, nncv_memref4d* in, nncv_memref4d* filter, nncv_memref4d* out);
+
+/* ---------------------------------------------------------------------------------------------
+ * Part 2 — device-resident forms (no counterpart in the reference)
+ * Return 0 on success, non-zero on error; nncv_hip_last_error() then describes it.
+ * dtype: 1 = fp32, 2 = fp16 (numbering of nncv::rt::dataType, DataType.hpp:118-124).
+ * `stream` is a hipStream_t passed as void* (NULL = the library's own stream, after which the
+ * call synchronises; with a caller stream the call only enqueues).
+ * ------------------------------------------------------------------------------------------- */
+int nncv_hip_init(int device);            /* optional; device < 0 keeps the current device */
+const char* nncv_hip_last_error(void);
+const char* nncv_hip_device_arch(void);   /* e.g. "gfx950:sramecc+:xnack-" */
+
+/* conv algorithms for 3x3 stride-1 layers */
+#define NNCV_HIP_ALGO_AUTO 0
+#define NNCV_HIP_ALGO_WINOGRAD 1 /* F(4x4,3x3): input/filter/output transforms + 36 batched GEMMs */
+#define NNCV_HIP_ALGO_IGEMM 2    /* implicit GEMM on MFMA */
+
+typedef struct nncv_hip_model nncv_hip_model;
+/* params: HOST pointer to the flat blob (n_elems elements of `dtype`). Uploads, folds BN, re-lays
+ * and transforms the filters once. */
+nncv_hip_model* nncv_hip_resnet18_create(const void* params, int64_t n_elems, int dtype, int algo3x3);
+void nncv_hip_resnet18_destroy(nncv_hip_model* m);
+/* src: DEVICE NCHW [N,3,H,W] of the model's dtype; logits: DEVICE [N,1000] fp32. */
+int nncv_hip_resnet18_forward(nncv_hip_model* m, const void* src, int N, int H, int W, float* logits, void* stream);
+
+/* Same, and also copies the NHWC activation after `stage` (0: after the max-pool, 1..4: after
+ * layer1..layer4) of the model's dtype to DEVICE `tap` — for layer-by-layer parity checks. */
+int nncv_hip_resnet18_forward_tap(nncv_hip_model* m, const void* src, int N, int H, int W, float* logits, int stage,
+                                  void* tap, void* stream);
+
+typedef struct nncv_hip_conv nncv_hip_conv;
+/* One fused conv + BN + (residual) + ReLU layer. weights: HOST FCHW of `dtype`;
+ * bn: HOST gamma, beta, mean, var of `dtype`, each [F], or all NULL. */
+nncv_hip_conv* nncv_hip_conv_create(int dtype, const void* weights, int F, int C, int R, int S, int stride, int pad,
+                                    const void* gamma, const void* beta, const void* mean, const void* var, int relu,
+                                    int algo);
+void nncv_hip_conv_destroy(nncv_hip_conv* c);
+int nncv_hip_conv_algo(const nncv_hip_conv* c);
+/* layout: 0 = NCHW, 1 = NHWC for in, out and residual alike (DEVICE pointers of the layer's dtype);
+ * in is [N,C,H,W] UNPADDED, out [N,F,OH,OW]; residual may be NULL. NHWC is the native layout. */
+int nncv_hip_conv_forward(nncv_hip_conv* c, const void* in, int N, int H, int W, int layout, const void* residual,
+                          void* out, void* stream);
+
+/* C += A.B, fp32 row-major, DEVICE pointers (K and N multiples of 4). */
+int nncv_hip_matmul_f32(const float* A, const float* B, float* C, int M, int N, int K, void* stream);
+
+/* Winograd F(4x4,3x3) stages on DEVICE buffers (layouts: U[36][F][C], V[36][tiles][C], M[36][tiles][F],
+ * tiles = N*ceil(OH/4)*ceil(OW/4)); exposed so each stage can be checked and profiled alone. */
+int nncv_hip_wino43_filter(int dtype, const void* w_fchw, void* U, int F, int C, void* stream);
+int nncv_hip_wino43_input(int dtype, const void* in, int layout, void* V, int N, int C, int H, int W, int pad, void* stream);
+int nncv_hip_wino43_gemm(int dtype, const void* V, const void* U, void* M, int64_t tiles, int C, int F, void* stream);
+int nncv_hip_wino43_output(int dtype, const void* M, void* out, int layout, int N, int F, int OH, int OW,
+                           const float* scale, const float* shift, const void* residual, int relu, void* stream);
+
+/* pooling on DEVICE NHWC tensors */
+int nncv_hip_maxpool3x3s2(int dtype, const void* in, void* out, int N, int H, int W, int C, void* stream);
+int nncv_hip_global_avgpool(int dtype, const void* in, void* out, int N, int H, int W, int C, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NNCV_HIP_H_ */

@@ -1,0 +1,155 @@
+"""ctypes binding of libnncv_hip.so (include/nncv_hip.h) — the same structs and entry points a
+C or C++ caller of nncv uses, so tests read like calls into the reference's object.
+
+There is no fallback: if the library is missing or cannot be loaded this module raises.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libnncv_hip.so")
+
+F32, F16 = 1, 2
+NCHW, NHWC = 0, 1
+ALGO_AUTO, ALGO_WINOGRAD, ALGO_IGEMM = 0, 1, 2
+
+c_intptr = ctypes.c_ssize_t
+
+
+def _memref(rank):
+    class MemRef(ctypes.Structure):
+        _fields_ = [("allocated", ctypes.c_void_p), ("aligned", ctypes.c_void_p), ("offset", c_intptr),
+                    ("sizes", c_intptr * rank), ("strides", c_intptr * rank)]
+    MemRef.__name__ = "MemRef%dD" % rank
+    return MemRef
+
+
+MemRef1D, MemRef2D, MemRef4D = _memref(1), _memref(2), _memref(4)
+assert ctypes.sizeof(MemRef1D) == 40 and ctypes.sizeof(MemRef2D) == 56 and ctypes.sizeof(MemRef4D) == 88
+
+EXPORTS = [
+    "_mlir_ciface_forward", "_mlir_ciface_forward_f16", "_mlir_ciface_matmul", "_mlir_ciface_batch_nchw_conv",
+    "nncv_hip_init", "nncv_hip_last_error", "nncv_hip_device_arch",
+    "nncv_hip_resnet18_create", "nncv_hip_resnet18_destroy", "nncv_hip_resnet18_forward",
+    "nncv_hip_resnet18_forward_tap",
+    "nncv_hip_conv_create", "nncv_hip_conv_destroy", "nncv_hip_conv_algo", "nncv_hip_conv_forward",
+    "nncv_hip_matmul_f32", "nncv_hip_wino43_filter", "nncv_hip_wino43_input", "nncv_hip_wino43_gemm",
+    "nncv_hip_wino43_output", "nncv_hip_maxpool3x3s2", "nncv_hip_global_avgpool",
+]
+
+_lib = None
+
+
+def lib():
+    """Load the library (never builds, never falls back)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("%s is missing: run `python -m nncv_amd.build` (needs hipcc)" % LIB_PATH)
+        L = ctypes.CDLL(LIB_PATH)
+        vp, i, i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64
+        P = ctypes.POINTER
+        L._mlir_ciface_forward.argtypes = [P(MemRef2D), P(MemRef4D), vp]
+        L._mlir_ciface_forward.restype = None
+        L._mlir_ciface_forward_f16.argtypes = [P(MemRef2D), P(MemRef4D), vp]
+        L._mlir_ciface_forward_f16.restype = None
+        L._mlir_ciface_matmul.argtypes = [P(MemRef2D)] * 4
+        L._mlir_ciface_matmul.restype = None
+        L._mlir_ciface_batch_nchw_conv.argtypes = [P(MemRef4D)] * 4
+        L._mlir_ciface_batch_nchw_conv.restype = None
+        L.nncv_hip_init.argtypes = [i]
+        L.nncv_hip_last_error.restype = ctypes.c_char_p
+        L.nncv_hip_device_arch.restype = ctypes.c_char_p
+        L.nncv_hip_resnet18_create.argtypes = [vp, i64, i, i]
+        L.nncv_hip_resnet18_create.restype = vp
+        L.nncv_hip_resnet18_destroy.argtypes = [vp]
+        L.nncv_hip_resnet18_destroy.restype = None
+        L.nncv_hip_resnet18_forward.argtypes = [vp, vp, i, i, i, vp, vp]
+        L.nncv_hip_resnet18_forward_tap.argtypes = [vp, vp, i, i, i, vp, i, vp, vp]
+        L.nncv_hip_conv_create.argtypes = [i, vp, i, i, i, i, i, i, vp, vp, vp, vp, i, i]
+        L.nncv_hip_conv_create.restype = vp
+        L.nncv_hip_conv_destroy.argtypes = [vp]
+        L.nncv_hip_conv_destroy.restype = None
+        L.nncv_hip_conv_algo.argtypes = [vp]
+        L.nncv_hip_conv_forward.argtypes = [vp, vp, i, i, i, i, vp, vp, vp]
+        L.nncv_hip_matmul_f32.argtypes = [vp, vp, vp, i, i, i, vp]
+        L.nncv_hip_wino43_filter.argtypes = [i, vp, vp, i, i, vp]
+        L.nncv_hip_wino43_input.argtypes = [i, vp, i, vp, i, i, i, i, i, vp]
+        L.nncv_hip_wino43_gemm.argtypes = [i, vp, vp, vp, i64, i, i, vp]
+        L.nncv_hip_wino43_output.argtypes = [i, vp, vp, i, i, i, i, i, vp, vp, vp, i, vp]
+        L.nncv_hip_maxpool3x3s2.argtypes = [i, vp, vp, i, i, i, i, vp]
+        L.nncv_hip_global_avgpool.argtypes = [i, vp, vp, i, i, i, i, vp]
+        _lib = L
+    return _lib
+
+
+class NncvHipError(RuntimeError):
+    pass
+
+
+def check(rc):
+    if rc != 0:
+        raise NncvHipError(lib().nncv_hip_last_error().decode())
+
+
+def np_dtype(dt):
+    return np.float16 if dt == F16 else np.float32
+
+
+# ---- host memref helpers (for the reference ABI) ------------------------------------------------
+
+def memref_of(a):
+    """Descriptor over a numpy array (any strides); keeps no reference — keep `a` alive."""
+    cls = {1: MemRef1D, 2: MemRef2D, 4: MemRef4D}[a.ndim]
+    m = cls()
+    m.allocated = m.aligned = a.ctypes.data
+    m.offset = 0
+    for k in range(a.ndim):
+        m.sizes[k] = a.shape[k]
+        m.strides[k] = a.strides[k] // a.itemsize
+    return m
+
+
+def memref_to_numpy(m, dtype):
+    """View of a dense rank-2 result descriptor (the buffer was malloc'd by the callee)."""
+    n = m.sizes[0] * m.sizes[1]
+    buf = (ctypes.c_char * (n * np.dtype(dtype).itemsize)).from_address(m.aligned)
+    return np.frombuffer(buf, dtype=dtype).reshape(m.sizes[0], m.sizes[1])
+
+
+_libc = ctypes.CDLL(None)
+_libc.free.argtypes = [ctypes.c_void_p]
+
+
+def forward(x, params_blob):
+    """_mlir_ciface_forward / _f16 on host arrays: x [N,3,H,W], params flat blob -> logits [N,1000].
+    The element type (float32 / float16) selects the entry point."""
+    assert x.dtype == params_blob.dtype and x.dtype in (np.float32, np.float16)
+    src = memref_of(x)
+    par = memref_of(params_blob)
+    dst = MemRef2D()
+    fn = lib()._mlir_ciface_forward if x.dtype == np.float32 else lib()._mlir_ciface_forward_f16
+    fn(ctypes.byref(dst), ctypes.byref(src), ctypes.cast(ctypes.byref(par), ctypes.c_void_p))
+    out = memref_to_numpy(dst, x.dtype).copy()
+    _libc.free(dst.allocated)  # the caller owns the callee-allocated result
+    return out
+
+
+def matmul(a, b, c):
+    """_mlir_ciface_matmul: c += a @ b in place (fp32 host arrays); returns the aliasing result view."""
+    res = MemRef2D()
+    ma, mb, mc = memref_of(a), memref_of(b), memref_of(c)
+    lib()._mlir_ciface_matmul(ctypes.byref(res), ctypes.byref(ma), ctypes.byref(mb), ctypes.byref(mc))
+    assert res.aligned == mc.aligned
+    return c
+
+
+def batch_nchw_conv(x_padded, w, out):
+    """_mlir_ciface_batch_nchw_conv: out += conv(x_padded, w) in place (fp32 host arrays)."""
+    res = MemRef4D()
+    mi, mw, mo = memref_of(x_padded), memref_of(w), memref_of(out)
+    lib()._mlir_ciface_batch_nchw_conv(ctypes.byref(res), ctypes.byref(mi), ctypes.byref(mw), ctypes.byref(mo))
+    assert res.aligned == mo.aligned
+    return out

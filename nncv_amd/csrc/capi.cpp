@@ -1,0 +1,538 @@
+// extern "C" surface of libnncv_hip.so (declared in include/nncv_hip.h).
+#include <cstring>
+#include <functional>
+#include <memory>
+#include <mutex>
+#include <vector>
+
+#include "../../include/nncv_hip.h"
+#include "model.hpp"
+
+using namespace nncv_hip;
+
+namespace nncv_hip {
+
+Context& Context::get() {
+  static Context c;
+  return c;
+}
+
+void Context::init(int device) {
+  if (ready_ && (device < 0 || device == device_)) return;
+  int count = 0;
+  NNCV_HIP_CHECK(hipGetDeviceCount(&count));
+  NNCV_REQUIRE(count > 0, "no HIP device visible");
+  if (device < 0) NNCV_HIP_CHECK(hipGetDevice(&device));
+  NNCV_REQUIRE(device < count, "device index out of range");
+  NNCV_REQUIRE(!ready_ || device == device_, "nncv_hip is already initialised on another device");
+  NNCV_HIP_CHECK(hipSetDevice(device));
+  hipDeviceProp_t prop;
+  NNCV_HIP_CHECK(hipGetDeviceProperties(&prop, device));
+  arch_ = prop.gcnArchName;
+  // the code objects in this library exist for gfx950 only; anything else cannot run them
+  NNCV_REQUIRE(arch_.rfind("gfx950", 0) == 0, "this library is built for gfx950 (MI355X); found " + arch_);
+  NNCV_HIP_CHECK(hipStreamCreate(&stream_));  // default priority
+  device_ = device;
+  ready_ = true;
+}
+
+}  // namespace nncv_hip
+
+namespace {
+
+thread_local std::string g_last_error;
+
+// int-returning entry points: 0 / -1 + message.
+int guarded(const std::function<void()>& fn) {
+  try {
+    std::lock_guard<std::recursive_mutex> lk(Context::get().mu);
+    fn();
+    return 0;
+  } catch (const std::exception& e) {
+    g_last_error = e.what();
+    return -1;
+  }
+}
+
+// void entry points of the reference ABI: report like the reference does, then abort.
+void guarded_abort(const char* what, const std::function<void()>& fn) {
+  try {
+    std::lock_guard<std::recursive_mutex> lk(Context::get().mu);
+    fn();
+  } catch (const std::exception& e) {
+    fprintf(stderr, "[ Erro ] %s: %s\n", what, e.what());
+    fflush(stderr);
+    abort();
+  }
+}
+
+struct Sync {  // NULL stream -> library stream + synchronise on exit
+  hipStream_t s;
+  bool own;
+  explicit Sync(void* user) : s(user ? static_cast<hipStream_t>(user) : Context::get().stream()), own(user == nullptr) {}
+  void finish() {
+    if (own) NNCV_HIP_CHECK(hipStreamSynchronize(s));
+  }
+};
+
+// ---- host memref helpers ----------------------------------------------------------------
+template <int R>
+bool contiguous(const intptr_t* sizes, const intptr_t* strides) {
+  intptr_t expect = 1;
+  for (int i = R - 1; i >= 0; --i) {
+    if (sizes[i] != 1 && strides[i] != expect) return false;
+    expect *= sizes[i];
+  }
+  return true;
+}
+
+// copy a strided rank-R host tensor of `es`-byte elements to/from a dense buffer
+template <int R>
+void strided_copy(char* base, intptr_t offset, const intptr_t* sizes, const intptr_t* strides, size_t es, char* dense,
+                  bool to_dense) {
+  intptr_t idx[R] = {0};
+  long long total = 1;
+  for (int i = 0; i < R; ++i) total *= sizes[i];
+  for (long long lin = 0; lin < total; ++lin) {
+    intptr_t off = offset;
+    for (int i = 0; i < R; ++i) off += idx[i] * strides[i];
+    if (to_dense) memcpy(dense + lin * es, base + off * es, es);
+    else memcpy(base + off * es, dense + lin * es, es);
+    for (int i = R - 1; i >= 0; --i) {
+      if (++idx[i] < sizes[i]) break;
+      idx[i] = 0;
+    }
+  }
+}
+
+// upload a host memref to `dev` (dense, row-major)
+template <int R>
+void upload(const void* aligned, intptr_t offset, const intptr_t* sizes, const intptr_t* strides, size_t es, void* dev,
+            PinnedBuffer& pin, hipStream_t s) {
+  long long total = 1;
+  for (int i = 0; i < R; ++i) total *= sizes[i];
+  char* base = static_cast<char*>(const_cast<void*>(aligned));
+  if (contiguous<R>(sizes, strides)) {
+    NNCV_HIP_CHECK(hipMemcpyAsync(dev, base + offset * es, total * es, hipMemcpyHostToDevice, s));
+  } else {
+    char* p = static_cast<char*>(pin.ensure(total * es));
+    strided_copy<R>(base, offset, sizes, strides, es, p, true);
+    NNCV_HIP_CHECK(hipMemcpyAsync(dev, p, total * es, hipMemcpyHostToDevice, s));
+  }
+  NNCV_HIP_CHECK(hipStreamSynchronize(s));  // the pinned buffer / caller memory may be reused at once
+}
+
+template <int R>
+void download(void* aligned, intptr_t offset, const intptr_t* sizes, const intptr_t* strides, size_t es, const void* dev,
+              PinnedBuffer& pin, hipStream_t s) {
+  long long total = 1;
+  for (int i = 0; i < R; ++i) total *= sizes[i];
+  char* base = static_cast<char*>(aligned);
+  if (contiguous<R>(sizes, strides)) {
+    NNCV_HIP_CHECK(hipMemcpyAsync(base + offset * es, dev, total * es, hipMemcpyDeviceToHost, s));
+    NNCV_HIP_CHECK(hipStreamSynchronize(s));
+  } else {
+    char* p = static_cast<char*>(pin.ensure(total * es));
+    NNCV_HIP_CHECK(hipMemcpyAsync(p, dev, total * es, hipMemcpyDeviceToHost, s));
+    NNCV_HIP_CHECK(hipStreamSynchronize(s));
+    strided_copy<R>(base, offset, sizes, strides, es, p, false);
+  }
+}
+
+// ---- model cache for the handle-less reference ABI ---------------------------------------
+struct CachedModel {
+  const void* host_ptr;
+  long long n;
+  int dt;
+  uint64_t fingerprint;
+  std::unique_ptr<ResNet18> model;
+};
+std::vector<CachedModel>& model_cache() {
+  static std::vector<CachedModel> c;
+  return c;
+}
+
+// cheap change detector for a parameter blob that lives at the same address: 4096 strided samples
+uint64_t fingerprint(const void* p, long long n, size_t es) {
+  const unsigned char* b = static_cast<const unsigned char*>(p);
+  uint64_t h = 1469598103934665603ull ^ (uint64_t)n;
+  const long long step = std::max<long long>(1, n / 4096);
+  for (long long i = 0; i < n; i += step)
+    for (size_t k = 0; k < es; ++k) h = (h ^ b[i * es + k]) * 1099511628211ull;
+  for (size_t k = 0; k < es; ++k) h = (h ^ b[(n - 1) * es + k]) * 1099511628211ull;
+  return h;
+}
+
+std::unique_ptr<ResNet18> build_model(const void* host, long long n, int dt, int algo, hipStream_t s) {
+  DeviceBuffer blob((size_t)n * dtype_size(dt));
+  NNCV_HIP_CHECK(hipMemcpyAsync(blob.get(), host, blob.bytes(), hipMemcpyHostToDevice, s));
+  auto m = std::make_unique<ResNet18>(blob.get(), n, dt, algo, s);
+  NNCV_HIP_CHECK(hipStreamSynchronize(s));  // the staging blob dies here
+  return m;
+}
+
+ResNet18& cached_model(const void* host, long long n, int dt, hipStream_t s) {
+  const uint64_t fp = fingerprint(host, n, dtype_size(dt));
+  auto& cache = model_cache();
+  for (auto& e : cache)
+    if (e.host_ptr == host && e.n == n && e.dt == dt) {
+      if (e.fingerprint != fp) {  // same address, new contents: rebuild
+        e.model = build_model(host, n, dt, kAlgoAuto, s);
+        e.fingerprint = fp;
+      }
+      return *e.model;
+    }
+  if (cache.size() >= 4) cache.erase(cache.begin());
+  cache.push_back(CachedModel{host, n, dt, fp, build_model(host, n, dt, kAlgoAuto, s)});
+  return *cache.back().model;
+}
+
+void forward_abi(nncv_memref2d* dst, nncv_memref4d* src, void* params, int dt) {
+  NNCV_REQUIRE(dst && src && params, "null descriptor");
+  Context& ctx = Context::get();
+  ctx.init(-1);
+  hipStream_t s = ctx.stream();
+  const size_t es = dtype_size(dt);
+  const nncv_memref1d* p = static_cast<const nncv_memref1d*>(params);
+  NNCV_REQUIRE(p->aligned && p->strides[0] == 1, "params must be a dense rank-1 memref");
+  const int N = (int)src->sizes[0], C = (int)src->sizes[1], H = (int)src->sizes[2], W = (int)src->sizes[3];
+  NNCV_REQUIRE(C == 3, "forward: input must be [N,3,H,W]");
+  const char* blob = static_cast<const char*>(p->aligned) + p->offset * (intptr_t)es;
+  ResNet18& model = cached_model(blob, p->sizes[0], dt, s);
+
+  const size_t in_bytes = align256((size_t)N * 3 * H * W * es), out_bytes = align256((size_t)N * 1000 * 4);
+  const size_t ws_bytes = model.workspace_bytes(N, H, W);
+  ctx.arena.reserve(in_bytes + out_bytes + ws_bytes + 1024, s);
+  void* d_in = ctx.arena.take(in_bytes);
+  float* d_out = static_cast<float*>(ctx.arena.take(out_bytes));
+  void* ws = ctx.arena.take(ws_bytes);
+  // The reference object assumes identity layout and would misread a strided input
+  // (DnnModelLowering.cpp:107-108); strides are honoured here instead.
+  upload<4>(src->aligned, src->offset, src->sizes, src->strides, es, d_in, ctx.pin_in, s);
+  model.forward(d_in, N, H, W, d_out, ws, s);
+
+  // MLIR C-interface convention: the callee allocates the result and overwrites *dst.
+  void* result = nullptr;
+  NNCV_REQUIRE(posix_memalign(&result, 64, std::max<size_t>(64, (size_t)N * 1000 * es)) == 0, "out of host memory");
+  if (dt == kF32) {
+    NNCV_HIP_CHECK(hipMemcpyAsync(result, d_out, (size_t)N * 1000 * 4, hipMemcpyDeviceToHost, s));
+    NNCV_HIP_CHECK(hipStreamSynchronize(s));
+  } else {
+    float* tmp = static_cast<float*>(ctx.pin_out.ensure((size_t)N * 1000 * 4));
+    NNCV_HIP_CHECK(hipMemcpyAsync(tmp, d_out, (size_t)N * 1000 * 4, hipMemcpyDeviceToHost, s));
+    NNCV_HIP_CHECK(hipStreamSynchronize(s));
+    _Float16* h = static_cast<_Float16*>(result);
+    for (long long i = 0; i < (long long)N * 1000; ++i) h[i] = (_Float16)tmp[i];
+  }
+  dst->allocated = result;
+  dst->aligned = result;
+  dst->offset = 0;
+  dst->sizes[0] = N;
+  dst->sizes[1] = 1000;
+  dst->strides[0] = 1000;
+  dst->strides[1] = 1;
+}
+
+struct nncv_hip_model_impl {
+  std::unique_ptr<ResNet18> m;
+};
+struct nncv_hip_conv_impl {
+  std::unique_ptr<ConvLayer> c;
+};
+
+}  // namespace
+
+struct nncv_hip_model : nncv_hip_model_impl {};
+struct nncv_hip_conv : nncv_hip_conv_impl {};
+
+extern "C" {
+
+// ---------------------------------------------------------------------------------------------
+// Part 1 — reference ABI
+// ---------------------------------------------------------------------------------------------
+void _mlir_ciface_forward(nncv_memref2d* dst, nncv_memref4d* src, void* params) {
+  guarded_abort("_mlir_ciface_forward", [&] { forward_abi(dst, src, params, kF32); });
+}
+
+void _mlir_ciface_forward_f16(nncv_memref2d* dst, nncv_memref4d* src, void* params) {
+  guarded_abort("_mlir_ciface_forward_f16", [&] { forward_abi(dst, src, params, kF16); });
+}
+
+void _mlir_ciface_matmul(nncv_memref2d* res, nncv_memref2d* a, nncv_memref2d* b, nncv_memref2d* c) {
+  guarded_abort("_mlir_ciface_matmul", [&] {
+    NNCV_REQUIRE(res && a && b && c, "null descriptor");
+    Context& ctx = Context::get();
+    ctx.init(-1);
+    hipStream_t s = ctx.stream();
+    const int M = (int)a->sizes[0], K = (int)a->sizes[1], N = (int)b->sizes[1];
+    NNCV_REQUIRE(b->sizes[0] == K && c->sizes[0] == M && c->sizes[1] == N, "matmul: shapes do not agree");
+    const size_t ab = align256((size_t)M * K * 4), bb = align256((size_t)K * N * 4), cb = align256((size_t)M * N * 4);
+    ctx.arena.reserve(ab + bb + cb + 1024, s);
+    float* dA = static_cast<float*>(ctx.arena.take(ab));
+    float* dB = static_cast<float*>(ctx.arena.take(bb));
+    float* dC = static_cast<float*>(ctx.arena.take(cb));
+    upload<2>(a->aligned, a->offset, a->sizes, a->strides, 4, dA, ctx.pin_in, s);
+    upload<2>(b->aligned, b->offset, b->sizes, b->strides, 4, dB, ctx.pin_in, s);
+    upload<2>(c->aligned, c->offset, c->sizes, c->strides, 4, dC, ctx.pin_in, s);
+    launch_gemm_nn_f32(dA, dB, dC, M, N, K, s);
+    download<2>(c->aligned, c->offset, c->sizes, c->strides, 4, dC, ctx.pin_out, s);
+    *res = *c;  // in-place bufferization: the result aliases `outs`
+  });
+}
+
+void _mlir_ciface_batch_nchw_conv(nncv_memref4d* res, nncv_memref4d* in, nncv_memref4d* filter, nncv_memref4d* out) {
+  guarded_abort("_mlir_ciface_batch_nchw_conv", [&] {
+    NNCV_REQUIRE(res && in && filter && out, "null descriptor");
+    Context& ctx = Context::get();
+    ctx.init(-1);
+    hipStream_t s = ctx.stream();
+    const int N = (int)in->sizes[0], C = (int)in->sizes[1], H = (int)in->sizes[2], W = (int)in->sizes[3];
+    const int F = (int)filter->sizes[0], R = (int)filter->sizes[2], S = (int)filter->sizes[3];
+    const int OH = (int)out->sizes[2], OW = (int)out->sizes[3];
+    NNCV_REQUIRE(filter->sizes[1] == C && out->sizes[0] == N && out->sizes[1] == F, "conv: shapes do not agree");
+    NNCV_REQUIRE(H >= R && W >= S && OH >= 1 && OW >= 1, "conv: filter larger than input");
+    // stride is an attribute of the compiled op in the reference; recover it from the shapes
+    int stride = 1;
+    if (OH > 1) stride = (H - R) / (OH - 1);
+    else if (OW > 1) stride = (W - S) / (OW - 1);
+    NNCV_REQUIRE(stride >= 1 && (H - R) / stride + 1 == OH && (W - S) / stride + 1 == OW,
+                 "conv: output shape is not (in - filter)/stride + 1 for any stride");
+    const size_t ib = align256((size_t)N * C * H * W * 4), fb = align256((size_t)F * C * R * S * 4),
+                 ob = align256((size_t)N * F * OH * OW * 4);
+    ConvLayer::Desc d;
+    d.dt = kF32; d.C = C; d.F = F; d.R = R; d.S = S; d.stride = stride; d.pad = 0; d.relu = false; d.algo = kAlgoAuto;
+    DeviceBuffer dF(fb);
+    upload<4>(filter->aligned, filter->offset, filter->sizes, filter->strides, 4, dF.get(), ctx.pin_in, s);
+    ConvLayer layer(d, dF.get(), nullptr, nullptr, nullptr, nullptr, s);
+    const size_t wsb = layer.workspace_bytes(N, H, W, true);
+    ctx.arena.reserve(ib + ob + wsb + 1024, s);
+    void* dI = ctx.arena.take(ib);
+    void* dO = ctx.arena.take(ob);
+    void* ws = ctx.arena.take(wsb);
+    upload<4>(in->aligned, in->offset, in->sizes, in->strides, 4, dI, ctx.pin_in, s);
+    upload<4>(out->aligned, out->offset, out->sizes, out->strides, 4, dO, ctx.pin_in, s);
+    layer.forward_strided(dI, strides_of(kNCHW, C, H, W), N, H, W, nullptr, dO, strides_of(kNCHW, F, OH, OW), true, ws, s);
+    download<4>(out->aligned, out->offset, out->sizes, out->strides, 4, dO, ctx.pin_out, s);
+    *res = *out;
+  });
+}
+
+// ---------------------------------------------------------------------------------------------
+// Part 2 — device-resident forms
+// ---------------------------------------------------------------------------------------------
+int nncv_hip_init(int device) {
+  return guarded([&] { Context::get().init(device); });
+}
+
+const char* nncv_hip_last_error(void) { return g_last_error.c_str(); }
+
+const char* nncv_hip_device_arch(void) {
+  if (guarded([&] { Context::get().init(-1); }) != 0) return "";
+  return Context::get().arch().c_str();
+}
+
+nncv_hip_model* nncv_hip_resnet18_create(const void* params, int64_t n_elems, int dtype, int algo3x3) {
+  nncv_hip_model* h = nullptr;
+  const int rc = guarded([&] {
+    NNCV_REQUIRE(params, "null params");
+    NNCV_REQUIRE(dtype == kF32 || dtype == kF16, "dtype must be 1 (fp32) or 2 (fp16)");
+    Context& ctx = Context::get();
+    ctx.init(-1);
+    h = new nncv_hip_model();
+    try {
+      h->m = build_model(params, n_elems, dtype, algo3x3, ctx.stream());
+    } catch (...) {
+      delete h;
+      h = nullptr;
+      throw;
+    }
+  });
+  return rc == 0 ? h : nullptr;
+}
+
+void nncv_hip_resnet18_destroy(nncv_hip_model* m) {
+  if (!m) return;
+  guarded([&] {
+    (void)hipDeviceSynchronize();
+    delete m;
+  });
+}
+
+int nncv_hip_resnet18_forward(nncv_hip_model* m, const void* src, int N, int H, int W, float* logits, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(m && m->m && src && logits, "null argument");
+    Context& ctx = Context::get();
+    Sync sy(stream);
+    const size_t wsb = m->m->workspace_bytes(N, H, W);
+    ctx.arena.reserve(wsb + 1024, sy.s);
+    m->m->forward(src, N, H, W, logits, ctx.arena.take(wsb), sy.s);
+    sy.finish();
+  });
+}
+
+int nncv_hip_resnet18_forward_tap(nncv_hip_model* m, const void* src, int N, int H, int W, float* logits, int stage,
+                                  void* tap, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(m && m->m && src && logits && tap, "null argument");
+    NNCV_REQUIRE(stage >= 0 && stage <= 4, "stage must be 0..4");
+    Context& ctx = Context::get();
+    Sync sy(stream);
+    const size_t wsb = m->m->workspace_bytes(N, H, W);
+    ctx.arena.reserve(wsb + 1024, sy.s);
+    m->m->forward(src, N, H, W, logits, ctx.arena.take(wsb), sy.s, stage, tap);
+    sy.finish();
+  });
+}
+
+nncv_hip_conv* nncv_hip_conv_create(int dtype, const void* weights, int F, int C, int R, int S, int stride, int pad,
+                                    const void* gamma, const void* beta, const void* mean, const void* var, int relu,
+                                    int algo) {
+  nncv_hip_conv* h = nullptr;
+  const int rc = guarded([&] {
+    NNCV_REQUIRE(weights, "null weights");
+    NNCV_REQUIRE(dtype == kF32 || dtype == kF16, "dtype must be 1 (fp32) or 2 (fp16)");
+    NNCV_REQUIRE(F > 0 && C > 0 && R > 0 && S > 0, "conv: bad geometry");
+    Context& ctx = Context::get();
+    ctx.init(-1);
+    hipStream_t s = ctx.stream();
+    const size_t es = dtype_size(dtype);
+    DeviceBuffer w((size_t)F * C * R * S * es), bn;
+    NNCV_HIP_CHECK(hipMemcpyAsync(w.get(), weights, w.bytes(), hipMemcpyHostToDevice, s));
+    const char* g = nullptr;
+    if (gamma) {
+      NNCV_REQUIRE(beta && mean && var, "conv: BN needs gamma, beta, mean and var");
+      bn.reset((size_t)4 * F * es);
+      const void* srcs[4] = {gamma, beta, mean, var};
+      for (int i = 0; i < 4; ++i)
+        NNCV_HIP_CHECK(hipMemcpyAsync(bn.as<char>() + (size_t)i * F * es, srcs[i], (size_t)F * es, hipMemcpyHostToDevice, s));
+      g = bn.as<char>();
+    }
+    ConvLayer::Desc d;
+    d.dt = dtype; d.C = C; d.F = F; d.R = R; d.S = S; d.stride = stride; d.pad = pad; d.relu = relu != 0; d.algo = algo;
+    h = new nncv_hip_conv();
+    try {
+      h->c = std::make_unique<ConvLayer>(d, w.get(), g, g ? g + (size_t)F * es : nullptr, g ? g + (size_t)2 * F * es : nullptr,
+                                         g ? g + (size_t)3 * F * es : nullptr, s);
+      NNCV_HIP_CHECK(hipStreamSynchronize(s));
+    } catch (...) {
+      delete h;
+      h = nullptr;
+      throw;
+    }
+  });
+  return rc == 0 ? h : nullptr;
+}
+
+void nncv_hip_conv_destroy(nncv_hip_conv* c) {
+  if (!c) return;
+  guarded([&] {
+    (void)hipDeviceSynchronize();
+    delete c;
+  });
+}
+
+int nncv_hip_conv_algo(const nncv_hip_conv* c) { return (c && c->c) ? c->c->algo() : -1; }
+
+int nncv_hip_conv_forward(nncv_hip_conv* c, const void* in, int N, int H, int W, int layout, const void* residual, void* out,
+                          void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(c && c->c && in && out, "null argument");
+    NNCV_REQUIRE(layout == kNCHW || layout == kNHWC, "layout must be 0 (NCHW) or 1 (NHWC)");
+    Context& ctx = Context::get();
+    Sync sy(stream);
+    const ConvLayer& L = *c->c;
+    const size_t wsb = L.workspace_bytes(N, H, W, layout == kNCHW);
+    ctx.arena.reserve(wsb + 1024, sy.s);
+    void* ws = ctx.arena.take(wsb);
+    if (layout == kNHWC) {
+      L.forward(in, N, H, W, residual, out, ws, sy.s);
+    } else {
+      const int OH = L.out_h(H), OW = L.out_w(W);
+      L.forward_strided(in, strides_of(kNCHW, L.desc().C, H, W), N, H, W, residual, out, strides_of(kNCHW, L.desc().F, OH, OW),
+                        false, ws, sy.s);
+    }
+    sy.finish();
+  });
+}
+
+int nncv_hip_matmul_f32(const float* A, const float* B, float* C, int M, int N, int K, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(A && B && C, "null argument");
+    Context::get().init(-1);
+    Sync sy(stream);
+    launch_gemm_nn_f32(A, B, C, M, N, K, sy.s);
+    sy.finish();
+  });
+}
+
+int nncv_hip_wino43_filter(int dtype, const void* w, void* U, int F, int C, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(w && U, "null argument");
+    Context::get().init(-1);
+    Sync sy(stream);
+    launch_wino43_filter(w, dtype, U, dtype, F, C, sy.s);
+    sy.finish();
+  });
+}
+
+int nncv_hip_wino43_input(int dtype, const void* in, int layout, void* V, int N, int C, int H, int W, int pad, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(in && V, "null argument");
+    Context::get().init(-1);
+    Sync sy(stream);
+    launch_wino43_input(in, dtype, strides_of(layout, C, H, W), V, dtype, N, C, H, W, pad, sy.s);
+    sy.finish();
+  });
+}
+
+int nncv_hip_wino43_gemm(int dtype, const void* V, const void* U, void* M, int64_t tiles, int C, int F, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(V && U && M, "null argument");
+    NNCV_REQUIRE(tiles > 0 && tiles < (1ll << 31), "tiles out of range");
+    Context::get().init(-1);
+    Sync sy(stream);
+    IgemmArgs a{};
+    a.in = V; a.wt = U; a.out = M;
+    a.N = (int)tiles; a.H = 1; a.W = 1; a.C = C; a.F = F; a.R = 1; a.S = 1; a.OH = 1; a.OW = 1;
+    a.stride_h = a.stride_w = 1; a.ldo = F; a.batch = 36;
+    a.in_bs = tiles * C; a.wt_bs = (long long)F * C; a.out_bs = tiles * F;
+    launch_igemm(a, dtype, dtype, sy.s);
+    sy.finish();
+  });
+}
+
+int nncv_hip_wino43_output(int dtype, const void* M, void* out, int layout, int N, int F, int OH, int OW, const float* scale,
+                           const float* shift, const void* residual, int relu, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(M && out, "null argument");
+    Context::get().init(-1);
+    Sync sy(stream);
+    WinoOutArgs o{};
+    o.M = M; o.out = out; o.residual = residual; o.scale = scale; o.shift = shift;
+    o.st = strides_of(layout, F, OH, OW); o.N = N; o.F = F; o.OH = OH; o.OW = OW; o.relu = relu; o.accumulate = 0;
+    launch_wino43_output(o, dtype, dtype, sy.s);
+    sy.finish();
+  });
+}
+
+int nncv_hip_maxpool3x3s2(int dtype, const void* in, void* out, int N, int H, int W, int C, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(in && out, "null argument");
+    Context::get().init(-1);
+    Sync sy(stream);
+    launch_maxpool3x3s2_nhwc(in, out, dtype, N, H, W, C, sy.s);
+    sy.finish();
+  });
+}
+
+int nncv_hip_global_avgpool(int dtype, const void* in, void* out, int N, int H, int W, int C, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(in && out, "null argument");
+    Context::get().init(-1);
+    Sync sy(stream);
+    launch_global_avgpool_nhwc(in, out, dtype, N, H * W, C, sy.s);
+    sy.finish();
+  });
+}
+
+}  // extern "C"

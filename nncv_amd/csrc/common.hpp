@@ -1,0 +1,110 @@
+// Shared declarations of the gfx950 hot-path library: element types, error handling, kernel
+// argument blocks and the launcher prototypes each .hip file exports to the host layer.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <stdexcept>
+#include <string>
+
+namespace nncv_hip {
+
+typedef _Float16 half_t;
+
+enum DType : int { kF32 = 1, kF16 = 2 };  // numbering of nncv::rt::dataType (DataType.hpp:118-124)
+enum Layout : int { kNCHW = 0, kNHWC = 1 };
+
+inline size_t dtype_size(int dt) { return dt == kF16 ? 2 : 4; }
+
+struct Error : std::runtime_error {
+  using std::runtime_error::runtime_error;
+};
+
+[[noreturn]] inline void fail(const std::string& msg) { throw Error(msg); }
+
+#define NNCV_HIP_CHECK(expr)                                                              \
+  do {                                                                                    \
+    hipError_t _e = (expr);                                                               \
+    if (_e != hipSuccess)                                                                 \
+      ::nncv_hip::fail(std::string(#expr) + ": " + hipGetErrorString(_e) + " (" __FILE__ ":" + \
+                       std::to_string(__LINE__) + ")");                                   \
+  } while (0)
+
+#define NNCV_REQUIRE(cond, msg)                     \
+  do {                                              \
+    if (!(cond)) ::nncv_hip::fail(std::string(msg)); \
+  } while (0)
+
+// ---------------------------------------------------------------------------------------------
+// Implicit-GEMM convolution / batched GEMM on MFMA.
+//   out[b][p][f] = epilogue( sum_k  X[b][p][k] * Wt[b][f][k] )
+// p = output pixel (n, oy, ox) of an NHWC activation tensor, k = (r, s, c) with c fastest,
+// X gathered on the fly with zero fill outside the image (the reference materialises the halo
+// with tensor.pad; here it never exists).  With R = S = 1, stride 1, pad 0 this is a plain
+// K-contiguous GEMM, which is how the 36 transformed-domain GEMMs of Winograd and the FC use it.
+// ---------------------------------------------------------------------------------------------
+struct IgemmArgs {
+  const void* in;        // [batch][N][H][W][C]
+  const void* wt;        // [batch][F][R*S*C]   (K-contiguous rows)
+  void* out;             // [batch][P][ldo], channel f at out[p*ldo + f]
+  const float* scale;    // [F] or null (1)
+  const float* shift;    // [F] or null (0)
+  const void* residual;  // same indexing as out, or null
+  int N, H, W, C, F, R, S, OH, OW;
+  int stride_h, stride_w, pad_h, pad_w;
+  int relu;
+  int ldo;     // out/residual row pitch in elements
+  int batch;   // grid.z
+  long long in_bs, wt_bs, out_bs;  // batch strides in elements
+};
+// in_dt: element type of in/wt (kF32 | kF16); out_dt: element type of out/residual.
+void launch_igemm(const IgemmArgs& a, int in_dt, int out_dt, hipStream_t s);
+
+// fp32 row-major C += A.B  (linalg.matmul)
+void launch_gemm_nn_f32(const float* A, const float* B, float* C, int M, int N, int K, hipStream_t s);
+
+// ---------------------------------------------------------------------------------------------
+// Winograd F(4x4,3x3)
+// ---------------------------------------------------------------------------------------------
+struct Strides4 { long long n, c, h, w; };  // element strides of a logical [N][C][H][W] tensor
+inline Strides4 strides_of(int layout, int C, int H, int W) {
+  if (layout == kNHWC) return {(long long)H * W * C, 1, (long long)W * C, C};
+  return {(long long)C * H * W, (long long)H * W, W, 1};
+}
+
+// U[36][F][C] = G g G^T from w[F][C][3][3]; U stored as u_dt, optionally scaled by 2^u_shift.
+void launch_wino43_filter(const void* w, int w_dt, void* U, int u_dt, int F, int C, hipStream_t s);
+// V[36][tiles][C] = B^T d B; input addressed through `st` (any layout), zero halo of `pad`.
+void launch_wino43_input(const void* in, int in_dt, Strides4 st, void* V, int v_dt, int N, int C, int H,
+                         int W, int pad, hipStream_t s);
+// out = epilogue(A^T M A), M[36][tiles][F] of m_dt; out/residual addressed through `st`.
+struct WinoOutArgs {
+  const void* M; void* out; const void* residual; const float* scale; const float* shift;
+  Strides4 st; int N, F, OH, OW; int relu; int accumulate;  // accumulate: out += result (ABI conv form)
+};
+void launch_wino43_output(const WinoOutArgs& a, int m_dt, int out_dt, hipStream_t s);
+
+// ---------------------------------------------------------------------------------------------
+// Pooling, layout and parameter preparation
+// ---------------------------------------------------------------------------------------------
+void launch_maxpool3x3s2_nhwc(const void* in, void* out, int dt, int N, int H, int W, int C, hipStream_t s);
+void launch_global_avgpool_nhwc(const void* in, void* out, int dt, int N, int HW, int C, hipStream_t s);
+// generic strided copy/cast between layouts: dst[n,c,h,w] (+)= (c < Csrc ? src[n,c,h,w] : 0) for c < Cdst
+void launch_relayout(const void* src, int src_dt, Strides4 ss, void* dst, int dst_dt, Strides4 ds, int N,
+                     int Csrc, int Cdst, int H, int W, bool accumulate, hipStream_t s);
+// stem input: NCHW [N,3,H,W] -> zero-haloed pixel-pair image [N][H+6][(W+8)/2][8]
+void launch_stem_pack(const void* src, int src_dt, void* dst, int dst_dt, int N, int H, int W, hipStream_t s);
+// weights FCRS -> [F][R][S][Cp] (Cp >= C, zero filled), cast to dst_dt
+void launch_weight_frsc(const void* w, int w_dt, void* dst, int dst_dt, int F, int C, int R, int S, int Cp,
+                        hipStream_t s);
+// stem weights [64,3,7,7] -> [64][7][4][8] over (pixel-pair, channel4)
+void launch_stem_weight(const void* w, int w_dt, void* dst, int dst_dt, int F, hipStream_t s);
+// BN fold: scale = gamma / sqrt(var + eps), shift = beta - mean*scale (fp32 out)
+void launch_bn_fold(const void* gamma, const void* beta, const void* mean, const void* var, int dt, float* scale,
+                    float* shift, int C, hipStream_t s);
+void launch_cast(const void* src, int src_dt, void* dst, int dst_dt, long long n, hipStream_t s);
+void launch_fill_f32(float* dst, float v, long long n, hipStream_t s);
+
+}  // namespace nncv_hip

@@ -1,0 +1,274 @@
+#include "model.hpp"
+
+#include <cstring>
+
+namespace nncv_hip {
+
+static int env_algo3x3() {
+  const char* e = getenv("NNCV_HIP_CONV3X3");
+  if (!e) return kAlgoAuto;
+  if (!strcmp(e, "winograd")) return kAlgoWinograd;
+  if (!strcmp(e, "igemm")) return kAlgoIgemm;
+  return kAlgoAuto;
+}
+
+static int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+ConvLayer::ConvLayer(const Desc& d, const void* w, const void* gamma, const void* beta, const void* mean, const void* var,
+                     hipStream_t s)
+    : d_(d) {
+  NNCV_REQUIRE(d.dt == kF32 || d.dt == kF16, "conv: dtype must be f32 or f16");
+  NNCV_REQUIRE(d.C > 0 && d.F > 0 && d.R > 0 && d.S > 0 && d.stride > 0 && d.pad >= 0, "conv: bad geometry");
+  const int ce = d.dt == kF16 ? 8 : 4;
+  const size_t es = dtype_size(d.dt);
+  const bool wino_ok = !d.stem && d.R == 3 && d.S == 3 && d.stride == 1 && d.C % ce == 0 && d.F % 4 == 0;
+  int algo = d.algo;
+  if (algo == kAlgoAuto) algo = env_algo3x3();
+  // default: Winograd where it is exact enough to be free (fp32); direct implicit GEMM in fp16,
+  // where F(4,3) costs about 10x the rounding error of the direct form.
+  if (algo == kAlgoAuto) algo = (d.dt == kF32) ? kAlgoWinograd : kAlgoIgemm;
+  if (algo == kAlgoWinograd && !wino_ok) algo = kAlgoIgemm;
+  algo_ = algo;
+
+  if (d.stem) {
+    NNCV_REQUIRE(d.C == 3 && d.R == 7 && d.S == 7 && d.stride == 2 && d.pad == 3, "stem: must be 7x7 s2 p3 over 3 channels");
+    NNCV_REQUIRE(d.F % 4 == 0, "stem: F must be a multiple of 4");
+    wt_.reset((size_t)d.F * 224 * es);
+    launch_stem_weight(w, d.dt, wt_.get(), d.dt, d.F, s);
+  } else if (algo_ == kAlgoWinograd) {
+    U_.reset((size_t)36 * d.F * d.C * es);
+    launch_wino43_filter(w, d.dt, U_.get(), d.dt, d.F, d.C, s);
+  } else {
+    const int Cp = round_up(d.C, ce), Fp = round_up(d.F, 4);
+    wt_.reset((size_t)Fp * d.R * d.S * Cp * es);
+    NNCV_HIP_CHECK(hipMemsetAsync(wt_.get(), 0, wt_.bytes(), s));
+    launch_weight_frsc(w, d.dt, wt_.get(), d.dt, d.F, d.C, d.R, d.S, Cp, s);
+  }
+  if (gamma) {
+    NNCV_REQUIRE(beta && mean && var, "conv: BN needs gamma, beta, mean and var");
+    const int Fp = round_up(d.F, 4);
+    scale_.reset((size_t)Fp * 4);
+    shift_.reset((size_t)Fp * 4);
+    launch_fill_f32(scale_.as<float>(), 0.0f, Fp, s);
+    launch_fill_f32(shift_.as<float>(), 0.0f, Fp, s);
+    launch_bn_fold(gamma, beta, mean, var, d.dt, scale_.as<float>(), shift_.as<float>(), d.F, s);
+  }
+}
+
+size_t ConvLayer::workspace_bytes(int N, int H, int W, bool strided) const {
+  const size_t es = dtype_size(d_.dt);
+  const int ce = d_.dt == kF16 ? 8 : 4;
+  const int OH = out_h(H), OW = out_w(W);
+  size_t b = 0;
+  if (d_.stem) b += align256((size_t)N * (H + 6) * ((W + 9) / 2) * 8 * es);
+  if (algo_ == kAlgoWinograd) {
+    const size_t tiles = (size_t)N * ((OH + 3) / 4) * ((OW + 3) / 4);
+    b += align256(36 * tiles * d_.C * es) + align256(36 * tiles * d_.F * es);
+  }
+  // strided (operator-level) form of the igemm path stages NHWC copies of input and output
+  if (strided && !d_.stem && algo_ == kAlgoIgemm)
+    b += align256((size_t)N * H * W * round_up(d_.C, ce) * es) + 2 * align256((size_t)N * OH * OW * round_up(d_.F, 4) * es);
+  return b;
+}
+
+void ConvLayer::forward(const void* in, int N, int H, int W, const void* residual, void* out, void* ws, hipStream_t s) const {
+  const int OH = out_h(H), OW = out_w(W);
+  NNCV_REQUIRE(N > 0 && OH > 0 && OW > 0, "conv: empty tensor");
+  const size_t es = dtype_size(d_.dt);
+  char* wsp = static_cast<char*>(ws);
+  if (d_.stem) {
+    const int HP = H + 6, WP = (W + 9) / 2;
+    launch_stem_pack(in, d_.dt, wsp, d_.dt, N, H, W, s);
+    IgemmArgs a{};
+    a.in = wsp; a.wt = wt_.get(); a.out = out;
+    a.scale = scale_.as<float>(); a.shift = shift_.as<float>(); a.residual = residual;
+    a.N = N; a.H = HP; a.W = WP; a.C = 8; a.F = d_.F; a.R = 7; a.S = 4; a.OH = OH; a.OW = OW;
+    a.stride_h = 2; a.stride_w = 1; a.pad_h = 0; a.pad_w = 0;
+    a.relu = d_.relu; a.ldo = d_.F; a.batch = 1;
+    launch_igemm(a, d_.dt, d_.dt, s);
+    return;
+  }
+  if (algo_ == kAlgoWinograd) {
+    forward_strided(in, strides_of(kNHWC, d_.C, H, W), N, H, W, residual, out, strides_of(kNHWC, d_.F, OH, OW), false, ws, s);
+    return;
+  }
+  NNCV_REQUIRE(d_.C % (16 / (int)es) == 0 && d_.F % 4 == 0, "conv: NHWC igemm needs C %% chunk == 0 and F %% 4 == 0");
+  IgemmArgs a{};
+  a.in = in; a.wt = wt_.get(); a.out = out;
+  a.scale = scale_.as<float>(); a.shift = shift_.as<float>(); a.residual = residual;
+  a.N = N; a.H = H; a.W = W; a.C = d_.C; a.F = d_.F; a.R = d_.R; a.S = d_.S; a.OH = OH; a.OW = OW;
+  a.stride_h = a.stride_w = d_.stride; a.pad_h = a.pad_w = d_.pad;
+  a.relu = d_.relu; a.ldo = d_.F; a.batch = 1;
+  launch_igemm(a, d_.dt, d_.dt, s);
+}
+
+void ConvLayer::forward_strided(const void* in, Strides4 in_st, int N, int H, int W, const void* residual, void* out,
+                                Strides4 out_st, bool accumulate, void* ws, hipStream_t s) const {
+  NNCV_REQUIRE(!d_.stem, "conv: the stem has no strided form");
+  const int OH = out_h(H), OW = out_w(W);
+  NNCV_REQUIRE(N > 0 && OH > 0 && OW > 0, "conv: empty tensor");
+  const size_t es = dtype_size(d_.dt);
+  const int ce = d_.dt == kF16 ? 8 : 4;
+  char* wsp = static_cast<char*>(ws);
+  if (algo_ == kAlgoWinograd) {
+    const int TH = (OH + 3) / 4, TW = (OW + 3) / 4;
+    const long long tiles = (long long)N * TH * TW;
+    void* V = wsp;
+    void* M = wsp + align256((size_t)36 * tiles * d_.C * es);
+    launch_wino43_input(in, d_.dt, in_st, V, d_.dt, N, d_.C, H, W, d_.pad, s);
+    IgemmArgs a{};
+    a.in = V; a.wt = U_.get(); a.out = M;
+    NNCV_REQUIRE(tiles < (1ll << 31), "conv: too many Winograd tiles");
+    a.N = (int)tiles; a.H = 1; a.W = 1; a.C = d_.C; a.F = d_.F; a.R = 1; a.S = 1; a.OH = 1; a.OW = 1;
+    a.stride_h = a.stride_w = 1; a.ldo = d_.F; a.batch = 36;
+    a.in_bs = tiles * d_.C; a.wt_bs = (long long)d_.F * d_.C; a.out_bs = tiles * d_.F;
+    launch_igemm(a, d_.dt, d_.dt, s);
+    WinoOutArgs o{};
+    o.M = M; o.out = out; o.residual = residual; o.scale = scale_.as<float>(); o.shift = shift_.as<float>();
+    o.st = out_st; o.N = N; o.F = d_.F; o.OH = OH; o.OW = OW; o.relu = d_.relu; o.accumulate = accumulate;
+    launch_wino43_output(o, d_.dt, d_.dt, s);
+    return;
+  }
+  // implicit GEMM through NHWC staging copies (operator-level forms only; the network itself is
+  // NHWC end to end and never comes here)
+  const int Cp = round_up(d_.C, ce), Fp = round_up(d_.F, 4);
+  const size_t in_b = align256((size_t)N * H * W * Cp * es), out_b = align256((size_t)N * OH * OW * Fp * es);
+  void* xin = wsp;
+  void* yout = wsp + in_b;
+  void* rin = residual ? wsp + in_b + out_b : nullptr;
+  launch_relayout(in, d_.dt, in_st, xin, d_.dt, strides_of(kNHWC, Cp, H, W), N, d_.C, Cp, H, W, false, s);
+  if (residual)
+    launch_relayout(residual, d_.dt, out_st, rin, d_.dt, strides_of(kNHWC, Fp, OH, OW), N, d_.F, Fp, OH, OW, false, s);
+  IgemmArgs a{};
+  a.in = xin; a.wt = wt_.get(); a.out = yout; a.residual = rin;
+  a.scale = scale_.as<float>(); a.shift = shift_.as<float>();
+  a.N = N; a.H = H; a.W = W; a.C = Cp; a.F = Fp; a.R = d_.R; a.S = d_.S; a.OH = OH; a.OW = OW;
+  a.stride_h = a.stride_w = d_.stride; a.pad_h = a.pad_w = d_.pad;
+  a.relu = d_.relu; a.ldo = Fp; a.batch = 1;
+  NNCV_REQUIRE(!(accumulate && (d_.relu || residual)), "conv: accumulate form has no epilogue");
+  launch_igemm(a, d_.dt, d_.dt, s);
+  // out (+)= y : y is NHWC with Fp channels; only the first F are copied
+  launch_relayout(yout, d_.dt, strides_of(kNHWC, Fp, OH, OW), out, d_.dt, out_st, N, d_.F, d_.F, OH, OW, accumulate, s);
+}
+
+// ---------------------------------------------------------------------------------------------
+
+ResNet18::ResNet18(const void* params, long long n_elems, int dt, int algo3x3, hipStream_t s) : dt_(dt) {
+  NNCV_REQUIRE(n_elems == kResNet18Elems,
+               "ResNet-18 params: expected 11699112 elements in the canonical model.bin order, got " + std::to_string(n_elems));
+  const size_t es = dtype_size(dt);
+  const char* p = static_cast<const char*>(params);
+  auto take = [&](long long n) { const void* r = p; p += n * es; return r; };
+  auto make = [&](int C, int F, int R, int stride, int pad, bool relu, bool stem) {
+    ConvLayer::Desc d;
+    d.dt = dt; d.C = C; d.F = F; d.R = d.S = R; d.stride = stride; d.pad = pad; d.relu = relu; d.stem = stem;
+    d.algo = (R == 3 && stride == 1) ? algo3x3 : kAlgoIgemm;
+    const void* w = take((long long)F * C * R * R);
+    const void* g = take(F); const void* b = take(F); const void* m = take(F); const void* v = take(F);
+    return std::make_unique<ConvLayer>(d, w, g, b, m, v, s);
+  };
+  stem_ = make(3, 64, 7, 2, 3, true, true);
+  int cin = 64;
+  const int widths[4] = {64, 128, 256, 512};
+  for (int L = 0; L < 4; ++L)
+    for (int blk = 0; blk < 2; ++blk) {
+      const int F = widths[L], stride = (L > 0 && blk == 0) ? 2 : 1;
+      Block b;
+      b.c1 = make(cin, F, 3, stride, 1, true, false);
+      b.c2 = make(F, F, 3, 1, 1, true, false);  // ReLU after the residual add
+      if (stride != 1 || cin != F) b.ds = make(cin, F, 1, stride, 0, false, false);
+      blocks_.push_back(std::move(b));
+      cin = F;
+    }
+  const void* fw = take(1000 * 512);
+  const void* fb = take(1000);
+  fc_w_.reset((size_t)1000 * 512 * es);
+  NNCV_HIP_CHECK(hipMemcpyAsync(fc_w_.get(), fw, fc_w_.bytes(), hipMemcpyDeviceToDevice, s));
+  fc_b_.reset(1000 * 4);
+  launch_cast(fb, dt, fc_b_.get(), kF32, 1000, s);
+  NNCV_REQUIRE((p - static_cast<const char*>(params)) == (long long)(kResNet18Elems * es), "ResNet-18 params: table walk mismatch");
+}
+
+namespace {
+struct Plan {
+  int h1, w1, h2, w2;   // after stem, after maxpool
+  size_t stem_out, act, pooled, conv_ws, total;
+};
+}  // namespace
+
+static Plan make_plan(const ResNet18& m, const ConvLayer& stem, const std::vector<const ConvLayer*>& convs, int dt, int N,
+                      int H, int W) {
+  (void)m;
+  Plan p{};
+  const size_t es = dtype_size(dt);
+  p.h1 = stem.out_h(H); p.w1 = stem.out_w(W);
+  p.h2 = (p.h1 + 2 - 3) / 2 + 1; p.w2 = (p.w1 + 2 - 3) / 2 + 1;
+  p.stem_out = align256((size_t)N * p.h1 * p.w1 * 64 * es);
+  p.act = align256((size_t)N * p.h2 * p.w2 * 64 * es);  // largest activation after the pool
+  p.pooled = align256((size_t)N * 512 * es);
+  p.conv_ws = stem.workspace_bytes(N, H, W);
+  int h = p.h2, w = p.w2;
+  for (const ConvLayer* c : convs) {
+    // every conv sees at most the post-pool resolution; sizes only shrink afterwards
+    p.conv_ws = std::max(p.conv_ws, c->workspace_bytes(N, h, w));
+  }
+  p.total = p.stem_out + 4 * p.act + p.pooled + p.conv_ws + 4096;
+  return p;
+}
+
+size_t ResNet18::workspace_bytes(int N, int H, int W) const {
+  std::vector<const ConvLayer*> convs;
+  for (const Block& b : blocks_) { convs.push_back(b.c1.get()); convs.push_back(b.c2.get()); if (b.ds) convs.push_back(b.ds.get()); }
+  return make_plan(*this, *stem_, convs, dt_, N, H, W).total;
+}
+
+void ResNet18::forward(const void* src, int N, int H, int W, void* logits, void* ws, hipStream_t s, int tap_stage,
+                       void* tap) const {
+  NNCV_REQUIRE(N > 0 && H >= 32 && W >= 32, "ResNet-18: input must be at least 32x32");
+  std::vector<const ConvLayer*> convs;
+  for (const Block& b : blocks_) { convs.push_back(b.c1.get()); convs.push_back(b.c2.get()); if (b.ds) convs.push_back(b.ds.get()); }
+  const Plan p = make_plan(*this, *stem_, convs, dt_, N, H, W);
+  char* base = static_cast<char*>(ws);
+  char* stem_out = base; base += p.stem_out;
+  char* act[4];
+  for (int i = 0; i < 4; ++i) { act[i] = base; base += p.act; }
+  char* pooled = base; base += p.pooled;
+  char* cws = base;
+
+  // stem: conv7x7 s2 + BN + ReLU (Res18.mlir:118-142), then maxpool 3x3 s2 (:144-151)
+  stem_->forward(src, N, H, W, nullptr, stem_out, cws, s);
+  launch_maxpool3x3s2_nhwc(stem_out, act[0], dt_, N, p.h1, p.w1, 64, s);
+  int cur = 0, h = p.h2, w = p.w2, nblk = 0, ch = 64;
+  const size_t es = dtype_size(dt_);
+  if (tap_stage == 0) NNCV_HIP_CHECK(hipMemcpyAsync(tap, act[0], (size_t)N * h * w * 64 * es, hipMemcpyDeviceToDevice, s));
+  for (const Block& b : blocks_) {
+    // BasicBlock (Res18.mlir:152-203, :255-320): y = relu(bn2(conv2(relu(bn1(conv1(x))))) + shortcut(x))
+    char* x = act[cur];
+    char* y1 = act[(cur + 1) & 3];
+    char* idn = act[(cur + 2) & 3];
+    char* y2 = act[(cur + 3) & 3];
+    const int oh = b.c1->out_h(h), ow = b.c1->out_w(w);
+    b.c1->forward(x, N, h, w, nullptr, y1, cws, s);
+    const void* shortcut = x;
+    if (b.ds) {
+      b.ds->forward(x, N, h, w, nullptr, idn, cws, s);
+      shortcut = idn;
+    }
+    b.c2->forward(y1, N, oh, ow, shortcut, y2, cws, s);
+    cur = (cur + 3) & 3;
+    h = oh; w = ow;
+    ch = b.c2->desc().F;
+    ++nblk;
+    if (nblk % 2 == 0 && tap_stage == nblk / 2)
+      NNCV_HIP_CHECK(hipMemcpyAsync(tap, act[cur], (size_t)N * h * w * ch * es, hipMemcpyDeviceToDevice, s));
+  }
+  // head: global average pool (sum, one divide), FC with bias (Res18.mlir:609-628)
+  launch_global_avgpool_nhwc(act[cur], pooled, dt_, N, h * w, 512, s);
+  IgemmArgs a{};
+  a.in = pooled; a.wt = fc_w_.get(); a.out = logits; a.shift = fc_b_.as<float>();
+  a.N = N; a.H = 1; a.W = 1; a.C = 512; a.F = 1000; a.R = 1; a.S = 1; a.OH = 1; a.OW = 1;
+  a.stride_h = a.stride_w = 1; a.ldo = 1000; a.batch = 1;
+  launch_igemm(a, dt_, kF32, s);
+}
+
+}  // namespace nncv_hip

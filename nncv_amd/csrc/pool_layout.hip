@@ -1,0 +1,292 @@
+// Bandwidth-bound helpers of the ResNet-18 path: pooling, layout packing and one-time parameter
+// preparation.  Activations are NHWC inside the library (channels contiguous), so every kernel
+// here maps lanes to the channel axis and moves 16 bytes per lane where the shape allows.
+#include "common.hpp"
+
+namespace nncv_hip {
+
+template <typename T>
+struct Vec16;  // 16-byte vector of T
+template <>
+struct Vec16<float> {
+  typedef float type __attribute__((ext_vector_type(4)));
+  static constexpr int n = 4;
+};
+template <>
+struct Vec16<half_t> {
+  typedef half_t type __attribute__((ext_vector_type(8)));
+  static constexpr int n = 8;
+};
+
+// arith.maximumf (tests/Nets/Pool2DMax.mlir:24): NaN in either operand wins.
+__device__ __forceinline__ float max_nan(float m, float v) { return (v > m || v != v) ? v : m; }
+
+// ---------------------------------------------------------------------------------------------
+// linalg.pooling_nchw_max 3x3 stride 2 over a -inf halo of 1 (tests/Nets/Res18.mlir:144-151),
+// NHWC.  One thread = one output pixel x one 16-byte channel group; the halo is a predicate.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void maxpool3x3s2_kernel(const T* __restrict__ in, T* __restrict__ out, int N, int H,
+                                                           int W, int C, int OH, int OW) {
+  constexpr int VN = Vec16<T>::n;
+  typedef typename Vec16<T>::type V;
+  const int CG = C / VN;
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long long)N * OH * OW * CG) return;
+  const int cg = (int)(idx % CG);
+  long long p = idx / CG;
+  const int ox = (int)(p % OW);
+  p /= OW;
+  const int oy = (int)(p % OH);
+  const int n = (int)(p / OH);
+  float m[VN];
+#pragma unroll
+  for (int e = 0; e < VN; ++e) m[e] = -INFINITY;
+#pragma unroll
+  for (int r = 0; r < 3; ++r) {
+    const int iy = oy * 2 - 1 + r;
+    if ((unsigned)iy >= (unsigned)H) continue;
+#pragma unroll
+    for (int s = 0; s < 3; ++s) {
+      const int ix = ox * 2 - 1 + s;
+      if ((unsigned)ix >= (unsigned)W) continue;
+      const V v = *reinterpret_cast<const V*>(in + (((long long)n * H + iy) * W + ix) * C + cg * VN);
+#pragma unroll
+      for (int e = 0; e < VN; ++e) m[e] = max_nan(m[e], (float)v[e]);
+    }
+  }
+  V o;
+#pragma unroll
+  for (int e = 0; e < VN; ++e) o[e] = (T)m[e];
+  *reinterpret_cast<V*>(out + (((long long)n * OH + oy) * OW + ox) * C + cg * VN) = o;
+}
+
+void launch_maxpool3x3s2_nhwc(const void* in, void* out, int dt, int N, int H, int W, int C, hipStream_t s) {
+  const int OH = (H + 2 - 3) / 2 + 1, OW = (W + 2 - 3) / 2 + 1;
+  const int vn = dt == kF16 ? 8 : 4;
+  NNCV_REQUIRE(C % vn == 0, "maxpool: C must be a multiple of the 16-byte vector");
+  const long long work = (long long)N * OH * OW * (C / vn);
+  const long long grid = (work + 255) / 256;
+  NNCV_REQUIRE(grid < (1ll << 31), "maxpool: grid too large");
+  if (dt == kF16)
+    hipLaunchKernelGGL((maxpool3x3s2_kernel<half_t>), dim3((unsigned)grid), dim3(256), 0, s, (const half_t*)in, (half_t*)out, N, H, W, C, OH, OW);
+  else
+    hipLaunchKernelGGL((maxpool3x3s2_kernel<float>), dim3((unsigned)grid), dim3(256), 0, s, (const float*)in, (float*)out, N, H, W, C, OH, OW);
+  NNCV_HIP_CHECK(hipGetLastError());
+}
+
+// ---------------------------------------------------------------------------------------------
+// linalg.pooling_nchw_sum over the whole image followed by one divf by H*W
+// (tests/Nets/Res18.mlir:609-614).  NHWC [N][HW][C] -> [N][C].
+// A workgroup handles one image x 64 channels: each of its 4 waves sums a quarter of the pixels
+// with lanes along the channels (one contiguous 128/256-byte segment per wave per pixel), then
+// the four partial sums meet in LDS.  fp32 accumulation; sum first, one divide.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void global_avgpool_kernel(const T* __restrict__ in, T* __restrict__ out, int HW, int C) {
+  __shared__ float part[4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + lane, n = blockIdx.y;
+  float s = 0.0f;
+  if (c < C)
+    for (int p = wave; p < HW; p += 4) s += (float)in[((long long)n * HW + p) * C + c];
+  part[wave][lane] = s;
+  __syncthreads();
+  if (wave == 0 && c < C) {
+    const float tot = ((part[0][lane] + part[1][lane]) + part[2][lane]) + part[3][lane];
+    out[(long long)n * C + c] = (T)(tot / (float)HW);
+  }
+}
+
+void launch_global_avgpool_nhwc(const void* in, void* out, int dt, int N, int HW, int C, hipStream_t s) {
+  dim3 grid((C + 63) / 64, N);
+  if (dt == kF16)
+    hipLaunchKernelGGL((global_avgpool_kernel<half_t>), grid, dim3(256), 0, s, (const half_t*)in, (half_t*)out, HW, C);
+  else
+    hipLaunchKernelGGL((global_avgpool_kernel<float>), grid, dim3(256), 0, s, (const float*)in, (float*)out, HW, C);
+  NNCV_HIP_CHECK(hipGetLastError());
+}
+
+// ---------------------------------------------------------------------------------------------
+// generic strided relayout / cast, dst (+)= src (operator-level ABI only; not on the ResNet-18 path)
+// ---------------------------------------------------------------------------------------------
+template <typename Ts, typename Td>
+__global__ void relayout_kernel(const Ts* __restrict__ src, Strides4 ss, Td* __restrict__ dst, Strides4 ds, int N, int Cs,
+                                int Cd, int H, int W, int dst_c_fastest, int accumulate) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long long)N * Cd * H * W) return;
+  int n, c, h, w;
+  long long r = idx;
+  if (dst_c_fastest) {
+    c = (int)(r % Cd); r /= Cd; w = (int)(r % W); r /= W; h = (int)(r % H); n = (int)(r / H);
+  } else {
+    w = (int)(r % W); r /= W; h = (int)(r % H); r /= H; c = (int)(r % Cd); n = (int)(r / Cd);
+  }
+  const float v = c < Cs ? (float)src[n * ss.n + c * ss.c + h * ss.h + w * ss.w] : 0.0f;
+  Td* d = dst + (n * ds.n + c * ds.c + h * ds.h + w * ds.w);
+  *d = accumulate ? (Td)((float)*d + v) : (Td)v;
+}
+
+void launch_relayout(const void* src, int src_dt, Strides4 ss, void* dst, int dst_dt, Strides4 ds, int N, int Cs, int Cd,
+                     int H, int W, bool accumulate, hipStream_t s) {
+  const long long work = (long long)N * Cd * H * W;
+  if (work == 0) return;
+  const long long grid = (work + 255) / 256;
+  NNCV_REQUIRE(grid < (1ll << 31), "relayout: grid too large");
+  const int cf = ds.c == 1;
+#define LAUNCH(TS, TD) \
+  hipLaunchKernelGGL((relayout_kernel<TS, TD>), dim3((unsigned)grid), dim3(256), 0, s, (const TS*)src, ss, (TD*)dst, ds, N, Cs, Cd, H, W, cf, accumulate ? 1 : 0)
+  if (src_dt == kF32 && dst_dt == kF32) LAUNCH(float, float);
+  else if (src_dt == kF32 && dst_dt == kF16) LAUNCH(float, half_t);
+  else if (src_dt == kF16 && dst_dt == kF16) LAUNCH(half_t, half_t);
+  else if (src_dt == kF16 && dst_dt == kF32) LAUNCH(half_t, float);
+#undef LAUNCH
+  NNCV_HIP_CHECK(hipGetLastError());
+}
+
+// ---------------------------------------------------------------------------------------------
+// Stem input packing.  The 7x7 stride-2 pad-3 convolution over 3 channels
+// (tests/Nets/Res18.mlir:118-124) is run by the implicit-GEMM kernel as a 7x4 stride-(2,1)
+// convolution over "pixel pairs": the NCHW image becomes [N][H+6][Wp][8] where element
+// (y', xp, 4*p + c) = in[c][y'-3][2*xp + p - 3] (zero outside the image and for c = 3), so that
+// one 16-byte chunk holds two horizontally adjacent pixels and a stride-2 walk in x becomes a
+// stride-1 walk over pairs.  Wp = (W + 9) / 2.
+// ---------------------------------------------------------------------------------------------
+template <typename Ts, typename Td>
+__global__ __launch_bounds__(256) void stem_pack_kernel(const Ts* __restrict__ src, Td* __restrict__ dst, int N, int H, int W,
+                                                        int HP, int WP) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long long)N * HP * WP) return;
+  const int xp = (int)(idx % WP);
+  const int yp = (int)((idx / WP) % HP);
+  const int n = (int)(idx / ((long long)WP * HP));
+  const int iy = yp - 3;
+  Td v[8];
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const int ix = 2 * xp + p - 3;
+    const bool ok = (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
+#pragma unroll
+    for (int c = 0; c < 3; ++c) v[4 * p + c] = ok ? (Td)(float)src[(((long long)n * 3 + c) * H + iy) * W + ix] : (Td)0.0f;
+    v[4 * p + 3] = (Td)0.0f;
+  }
+  Td* d = dst + idx * 8;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) d[e] = v[e];
+}
+
+void launch_stem_pack(const void* src, int src_dt, void* dst, int dst_dt, int N, int H, int W, hipStream_t s) {
+  const int HP = H + 6, WP = (W + 9) / 2;
+  const long long work = (long long)N * HP * WP;
+  const long long grid = (work + 255) / 256;
+  NNCV_REQUIRE(grid < (1ll << 31), "stem_pack: grid too large");
+#define LAUNCH(TS, TD) \
+  hipLaunchKernelGGL((stem_pack_kernel<TS, TD>), dim3((unsigned)grid), dim3(256), 0, s, (const TS*)src, (TD*)dst, N, H, W, HP, WP)
+  if (src_dt == kF32 && dst_dt == kF32) LAUNCH(float, float);
+  else if (src_dt == kF16 && dst_dt == kF16) LAUNCH(half_t, half_t);
+  else if (src_dt == kF32 && dst_dt == kF16) LAUNCH(float, half_t);
+  else fail("stem_pack: unsupported dtype combination");
+#undef LAUNCH
+  NNCV_HIP_CHECK(hipGetLastError());
+}
+
+// ---------------------------------------------------------------------------------------------
+// one-time parameter preparation
+// ---------------------------------------------------------------------------------------------
+template <typename Ts, typename Td>
+__global__ void weight_frsc_kernel(const Ts* __restrict__ w, Td* __restrict__ dst, int F, int C, int R, int S, int Cp) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long long)F * R * S * Cp) return;
+  const int c = (int)(idx % Cp);
+  long long r = idx / Cp;
+  const int s = (int)(r % S); r /= S;
+  const int rr = (int)(r % R);
+  const int f = (int)(r / R);
+  dst[idx] = c < C ? (Td)(float)w[(((long long)f * C + c) * R + rr) * S + s] : (Td)0.0f;
+}
+
+void launch_weight_frsc(const void* w, int w_dt, void* dst, int dst_dt, int F, int C, int R, int S, int Cp, hipStream_t s) {
+  const long long work = (long long)F * R * S * Cp;
+  const unsigned grid = (unsigned)((work + 255) / 256);
+#define LAUNCH(TS, TD) hipLaunchKernelGGL((weight_frsc_kernel<TS, TD>), dim3(grid), dim3(256), 0, s, (const TS*)w, (TD*)dst, F, C, R, S, Cp)
+  if (w_dt == kF32 && dst_dt == kF32) LAUNCH(float, float);
+  else if (w_dt == kF16 && dst_dt == kF16) LAUNCH(half_t, half_t);
+  else if (w_dt == kF32 && dst_dt == kF16) LAUNCH(float, half_t);
+  else fail("weight_frsc: unsupported dtype combination");
+#undef LAUNCH
+  NNCV_HIP_CHECK(hipGetLastError());
+}
+
+template <typename Ts, typename Td>
+__global__ void stem_weight_kernel(const Ts* __restrict__ w, Td* __restrict__ dst, int F) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;  // over [F][7][4][8]
+  if (idx >= F * 7 * 4 * 8) return;
+  const int e = idx & 7, sp = (idx >> 3) & 3, r = (idx >> 5) % 7, f = idx / 224;
+  const int p = e >> 2, c = e & 3, s = 2 * sp + p;
+  dst[idx] = (c < 3 && s < 7) ? (Td)(float)w[((f * 3 + c) * 7 + r) * 7 + s] : (Td)0.0f;
+}
+
+void launch_stem_weight(const void* w, int w_dt, void* dst, int dst_dt, int F, hipStream_t s) {
+  const unsigned grid = (unsigned)((F * 224 + 255) / 256);
+#define LAUNCH(TS, TD) hipLaunchKernelGGL((stem_weight_kernel<TS, TD>), dim3(grid), dim3(256), 0, s, (const TS*)w, (TD*)dst, F)
+  if (w_dt == kF32 && dst_dt == kF32) LAUNCH(float, float);
+  else if (w_dt == kF16 && dst_dt == kF16) LAUNCH(half_t, half_t);
+  else if (w_dt == kF32 && dst_dt == kF16) LAUNCH(float, half_t);
+  else fail("stem_weight: unsupported dtype combination");
+#undef LAUNCH
+  NNCV_HIP_CHECK(hipGetLastError());
+}
+
+// BN (tests/Nets/Res18.mlir:127-136) folded to y = x*scale + shift:
+//   r = 1/sqrt(var + (float)1e-5) ; scale = gamma * r ; shift = beta - mean * scale
+// evaluated in fp64 and rounded once, so the fold adds less than one fp32 ulp to each factor.
+template <typename T>
+__global__ void bn_fold_kernel(const T* g, const T* b, const T* m, const T* v, float* scale, float* shift, int C) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const double eps = (double)(float)1e-5;
+  const double r = 1.0 / sqrt((double)(float)v[c] + eps);
+  const double sc = (double)(float)g[c] * r;
+  scale[c] = (float)sc;
+  shift[c] = (float)((double)(float)b[c] - (double)(float)m[c] * sc);
+}
+
+void launch_bn_fold(const void* g, const void* b, const void* m, const void* v, int dt, float* scale, float* shift, int C,
+                    hipStream_t s) {
+  const unsigned grid = (unsigned)((C + 255) / 256);
+  if (dt == kF16)
+    hipLaunchKernelGGL((bn_fold_kernel<half_t>), dim3(grid), dim3(256), 0, s, (const half_t*)g, (const half_t*)b, (const half_t*)m, (const half_t*)v, scale, shift, C);
+  else
+    hipLaunchKernelGGL((bn_fold_kernel<float>), dim3(grid), dim3(256), 0, s, (const float*)g, (const float*)b, (const float*)m, (const float*)v, scale, shift, C);
+  NNCV_HIP_CHECK(hipGetLastError());
+}
+
+template <typename Ts, typename Td>
+__global__ void cast_kernel(const Ts* __restrict__ src, Td* __restrict__ dst, long long n) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = (Td)(float)src[i];
+}
+
+void launch_cast(const void* src, int src_dt, void* dst, int dst_dt, long long n, hipStream_t s) {
+  if (n == 0) return;
+  const unsigned grid = (unsigned)((n + 255) / 256);
+#define LAUNCH(TS, TD) hipLaunchKernelGGL((cast_kernel<TS, TD>), dim3(grid), dim3(256), 0, s, (const TS*)src, (TD*)dst, n)
+  if (src_dt == kF32 && dst_dt == kF32) LAUNCH(float, float);
+  else if (src_dt == kF16 && dst_dt == kF16) LAUNCH(half_t, half_t);
+  else if (src_dt == kF32 && dst_dt == kF16) LAUNCH(float, half_t);
+  else LAUNCH(half_t, float);
+#undef LAUNCH
+  NNCV_HIP_CHECK(hipGetLastError());
+}
+
+__global__ void fill_f32_kernel(float* dst, float v, long long n) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = v;
+}
+void launch_fill_f32(float* dst, float v, long long n, hipStream_t s) {
+  if (n == 0) return;
+  hipLaunchKernelGGL(fill_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, dst, v, n);
+  NNCV_HIP_CHECK(hipGetLastError());
+}
+
+}  // namespace nncv_hip

@@ -1,0 +1,97 @@
+"""GPU parity of the convolution paths against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+
+import oracle
+from nncv_amd import abi, synth
+from gpu_util import (Conv, dev, host, nhwc, nchw, max_rel, rel_l2, FP32_MAX_REL, FP16_REL_L2)
+
+pytestmark = pytest.mark.gpu
+
+
+def oracle_layer(x, w, stride, pad, bn=None, residual=None, relu=False):
+    y = oracle.conv2d_nchw_fchw(oracle.pad_nchw(x, pad), w, stride=stride)
+    if bn is not None:
+        y = oracle.batchnorm(y, *bn)
+    if residual is not None:
+        y = y + residual
+    if relu:
+        y = oracle.relu(y)
+    return y
+
+
+def bn_params(seed, F):
+    return (synth.uniform(seed, (F,), 0.5, 1.5), synth.normal(seed + 1, (F,), 0.1),
+            synth.normal(seed + 2, (F,), 0.1), synth.uniform(seed + 3, (F,), 0.5, 1.5))
+
+
+CASES = [  # N, C, F, H, W, R, stride, pad
+    (2, 64, 64, 14, 14, 3, 1, 1),
+    (1, 64, 128, 28, 28, 3, 2, 1),
+    (3, 64, 128, 14, 14, 1, 2, 0),
+    (2, 128, 64, 9, 13, 3, 1, 1),     # ragged: odd, non-square
+    (1, 32, 200, 7, 7, 3, 1, 1),      # F not a multiple of the tile
+    (5, 16, 8, 6, 5, 3, 2, 1),        # tiny
+]
+
+
+@pytest.mark.parametrize("N,C,F,H,W,R,stride,pad", CASES)
+@pytest.mark.parametrize("dt", [abi.F32, abi.F16])
+@pytest.mark.parametrize("algo", [abi.ALGO_IGEMM, abi.ALGO_WINOGRAD])
+def test_conv_bn_relu_residual_nhwc(N, C, F, H, W, R, stride, pad, dt, algo):
+    if algo == abi.ALGO_WINOGRAD and not (R == 3 and stride == 1):
+        pytest.skip("Winograd F(4,3) covers 3x3 stride-1 only")
+    print("case", N, C, F, H, W, R, stride, pad, dt, algo, flush=True)
+    x = synth.normal(100, (N, C, H, W))
+    w = synth.normal(101, (F, C, R, R), std=float(np.sqrt(2.0 / (C * R * R))))
+    bn = bn_params(102, F)
+    OH, OW = (H + 2 * pad - R) // stride + 1, (W + 2 * pad - R) // stride + 1
+    res = synth.normal(106, (N, F, OH, OW))
+    if dt == abi.F16:
+        x, w, res = synth.round_fp16(x), synth.round_fp16(w), synth.round_fp16(res)
+        bn = tuple(synth.round_fp16(b) for b in bn)
+    want = oracle_layer(x, w, stride, pad, bn, res, relu=True)
+    layer = Conv(dt, w, stride, pad, bn=bn, relu=True, algo=algo)
+    assert layer.algo == algo
+    got = nchw(host(layer(dev(nhwc(x), dt), abi.NHWC, residual=dev(nhwc(res), dt))))
+    if dt == abi.F32:
+        assert max_rel(got, want) < FP32_MAX_REL
+    else:
+        assert rel_l2(got, want) < FP16_REL_L2
+    assert (got >= 0).all()
+
+
+@pytest.mark.parametrize("algo", [abi.ALGO_IGEMM, abi.ALGO_WINOGRAD])
+def test_conv_nchw_layout_plain(algo):
+    """NCHW in/out (the layout of the reference's ABI), no epilogue."""
+    x = synth.normal(110, (2, 16, 10, 11))
+    w = synth.normal(111, (12, 16, 3, 3), std=0.1)
+    want = oracle_layer(x, w, 1, 1)
+    layer = Conv(abi.F32, w, 1, 1, algo=algo)
+    got = host(layer(dev(x), abi.NCHW))
+    assert max_rel(got, want) < FP32_MAX_REL
+
+
+def test_relu_keeps_nan_and_conv_zero_halo():
+    """`ugt` ReLU keeps NaN (Res18.mlir:139-141); the halo contributes exact zeros."""
+    x = np.ones((1, 8, 4, 4), np.float32)
+    w = np.ones((4, 8, 3, 3), np.float32)
+    layer = Conv(abi.F32, w, 1, 1, relu=True, algo=abi.ALGO_IGEMM)
+    got = nchw(host(layer(dev(nhwc(x)), abi.NHWC)))
+    want = np.array([[32, 48, 48, 32], [48, 72, 72, 48], [48, 72, 72, 48], [32, 48, 48, 32]], np.float32)
+    assert np.array_equal(got[0, 0], want)
+    x[0, 0, 1, 1] = np.nan
+    got = nchw(host(layer(dev(nhwc(x)), abi.NHWC)))
+    assert np.isnan(got[0, :, 0:3, 0:3]).all() and not np.isnan(got[0, :, 3, 3]).any()
+
+
+def test_cfg2_single_conv_winograd_vs_direct():
+    """BASELINE config 2: 3x3 s1 p1 fp32, input [1,64,56,56], filter [64,64,3,3]."""
+    x, w = synth.cfg2_conv()
+    want = oracle_layer(x, w, 1, 1)
+    for algo in (abi.ALGO_WINOGRAD, abi.ALGO_IGEMM):
+        layer = Conv(abi.F32, w, 1, 1, algo=algo)
+        got = nchw(host(layer(dev(nhwc(x)), abi.NHWC)))
+        err = max_rel(got, want)
+        print("cfg2 algo", algo, "max_rel", err, flush=True)
+        assert err < FP32_MAX_REL

@@ -1,0 +1,67 @@
+"""Pooling kernels and the fp32 GEMM against the oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from nncv_amd import abi, synth
+from gpu_util import dev, empty, host, nhwc, nchw, max_rel, FP32_MAX_REL
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dt", [abi.F32, abi.F16])
+@pytest.mark.parametrize("N,C,H,W", [(2, 64, 16, 16), (1, 8, 9, 7), (3, 16, 5, 6)])
+def test_maxpool(dt, N, C, H, W):
+    x = synth.normal(300, (N, C, H, W))
+    if dt == abi.F16:
+        x = synth.round_fp16(x)
+    x[0, 1, 2, 2] = np.nan  # arith.maximumf propagates NaN
+    want = oracle.maxpool3x3s2(x)
+    OH, OW = want.shape[2:]
+    out = empty((N, OH, OW, C), dt)
+    abi.check(abi.lib().nncv_hip_maxpool3x3s2(dt, dev(nhwc(x), dt).data_ptr(), out.data_ptr(), N, H, W, C, None))
+    got = nchw(host(out))
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.array_equal(np.nan_to_num(got, nan=7.0), np.nan_to_num(want, nan=7.0))  # max is exact
+
+
+@pytest.mark.parametrize("dt", [abi.F32, abi.F16])
+@pytest.mark.parametrize("N,C,H,W", [(2, 512, 7, 7), (1, 512, 8, 8), (3, 96, 3, 5)])
+def test_global_avgpool(dt, N, C, H, W):
+    x = synth.normal(310, (N, C, H, W))
+    if dt == abi.F16:
+        x = synth.round_fp16(x)
+    want = oracle.global_avgpool(x)
+    out = empty((N, C), dt)
+    abi.check(abi.lib().nncv_hip_global_avgpool(dt, dev(nhwc(x), dt).data_ptr(), out.data_ptr(), N, H, W, C, None))
+    tol = 1e-6 if dt == abi.F32 else 1e-3  # fp16 result is rounded to half once
+    assert np.abs(host(out) - want).max() <= tol * max(1.0, np.abs(want).max())
+
+
+@pytest.mark.parametrize("M,N,K", [(1024, 1024, 1024), (130, 68, 36), (64, 64, 16), (257, 512, 1000), (1, 4, 4)])
+def test_matmul_device(M, N, K):
+    a = synth.uniform(320, (M, K), -1, 1)
+    b = synth.uniform(321, (K, N), -1, 1)
+    c0 = synth.uniform(322, (M, N), -1, 1)
+    want = oracle.matmul(a, b, c0)
+    c = dev(c0)
+    abi.check(abi.lib().nncv_hip_matmul_f32(dev(a).data_ptr(), dev(b).data_ptr(), c.data_ptr(), M, N, K, None))
+    err = max_rel(host(c), want)
+    print("matmul", M, N, K, "max_rel", err, flush=True)
+    assert err < FP32_MAX_REL
+
+
+def test_cfg1_matmul_through_reference_abi():
+    """BASELINE config 1 through _mlir_ciface_matmul: C (zeros) += A.B on host memrefs, plus a
+    strided (transposed-view) operand, which the descriptor semantics must honour."""
+    a, b = synth.cfg1_matmul()
+    c = np.zeros((1024, 1024), np.float32)
+    abi.matmul(a, b, c)
+    want = oracle.matmul(a, b)
+    assert max_rel(c, want) < FP32_MAX_REL
+    at = np.ascontiguousarray(a.T).T  # same values, column-major strides
+    assert at.strides != a.strides
+    c2 = np.zeros((1024, 1024), np.float32)
+    abi.matmul(at, b, c2)
+    assert np.array_equal(c, c2)

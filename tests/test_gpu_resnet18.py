@@ -1,0 +1,77 @@
+"""ResNet-18 forward on the GPU against the oracle: device API, taps, and the reference ABI."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from nncv_amd import abi, modelbin, synth
+from gpu_util import Model, dev, host, nchw, max_rel, rel_l2, FP32_MAX_REL, FP16_REL_L2
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def blob():
+    return synth.resnet18_params()
+
+
+@pytest.mark.parametrize("algo", [abi.ALGO_WINOGRAD, abi.ALGO_IGEMM])
+def test_fp32_small_image_with_taps(blob, algo):
+    x = synth.uniform(3001, (2, 3, 64, 64), 0.0, 1.0)
+    m = Model(blob, abi.F32, algo)
+    xd = dev(x)
+    for stage in (0, 1, 2, 3, 4):
+        want_logits, want_tap = oracle.resnet18_forward(x, blob, tap_layer=stage)
+        logits, tap = m(xd, tap_stage=stage)
+        err = max_rel(nchw(host(tap)), want_tap)
+        print("algo", algo, "stage", stage, "tap max_rel", err, flush=True)
+        assert err < FP32_MAX_REL
+    err = max_rel(host(logits), want_logits)
+    print("logits max_rel", err, flush=True)
+    assert err < FP32_MAX_REL
+    assert (host(logits).argmax(1) == want_logits.argmax(1)).all()
+
+
+def test_cfg3_fp32_256_through_reference_abi(blob, tmp_path):
+    """BASELINE config 3: [1,3,256,256] fp32, params read back from a -split-params style
+    model.bin, called through _mlir_ciface_forward like examples/Res18/main.cpp does."""
+    p = str(tmp_path / "model.bin")
+    modelbin.write_resnet18(p, blob)
+    index, params = modelbin.read(p)
+    assert len(index) == 102
+    params = np.array(params)  # own, writable copy like MemRefFlatArray's blob
+    x = synth.cfg3_input()
+    got = abi.forward(x, params)
+    want = oracle.resnet18_forward(x, blob)
+    err = max_rel(got, want)
+    print("cfg3 logits max_rel", err, "top1", got.argmax(1), want.argmax(1), flush=True)
+    assert got.shape == (1, 1000)
+    assert err < FP32_MAX_REL
+    assert (got.argmax(1) == want.argmax(1)).all()
+    # second call hits the cached device model; a strided input view must give the same answer
+    xs = np.zeros((1, 3, 256, 512), np.float32)[:, :, :, ::2]
+    xs[...] = x
+    assert not xs.flags["C_CONTIGUOUS"]
+    again = abi.forward(xs, params)
+    assert np.array_equal(again, got)
+    # same address, new contents: the cache must notice
+    params[-1000:] += 1.0  # fc.bias
+    shifted = abi.forward(x, params)
+    assert np.allclose(shifted, got + 1.0, atol=1e-5)
+
+
+def test_fp16_small_batch(blob):
+    """fp16 storage, fp32 accumulate vs the fp32 oracle on half-rounded weights and input."""
+    hb = synth.round_fp16(blob)
+    x = synth.round_fp16(synth.uniform(4001, (4, 3, 224, 224), 0.0, 1.0))
+    want = oracle.resnet18_forward(x, hb)
+    for algo in (abi.ALGO_IGEMM, abi.ALGO_WINOGRAD):
+        m = Model(hb, abi.F16, algo)
+        got = host(m(dev(x, abi.F16)))
+        err = rel_l2(got, want)
+        print("fp16 algo", algo, "rel_l2", err, "top1", got.argmax(1), want.argmax(1), flush=True)
+        assert err < FP16_REL_L2
+        if algo == abi.ALGO_IGEMM:
+            assert (got.argmax(1) == want.argmax(1)).all()

@@ -1,0 +1,168 @@
+#!/usr/bin/env python3
+"""ResNet-18 inference benchmark of libnncv_hip.so on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 32] [--algo auto|winograd|igemm]
+
+One step = one forward pass of BASELINE config 4 (ResNet-18, fp16 storage / fp32 accumulate,
+input [32,3,224,224], seeded synthetic input and random-init weights) with the input already
+resident in HBM and the logits left in HBM.  Prints ONE JSON line.
+
+Besides the headline images/s the line carries
+  roofline      the dominant kernel (the implicit-GEMM MFMA kernel instance that takes the most
+                time) : algorithmic flops per launch / average launch duration, measured live
+                with HIP events on the launch stream in a separate profiled pass of the same
+                workload, against the published dense fp16 MFMA peak;
+  kernels       the same event-timed breakdown for every kernel tag (ms per step, share);
+  batch1        images/s of the same network at batch 1;
+  cpu_baseline  the CPU checker (oracle/, fp32, OpenMP) timed on this box's host cores on a
+                bounded sample of the same workload — a reported baseline, not a target.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 matrix peak
+HBM_PEAK_GBS = 8000.0
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--batch", type=int, default=32)
+    ap.add_argument("--algo", default="auto", choices=["auto", "winograd", "igemm"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--profile-steps", type=int, default=5)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.stderr.write("bench.py: this build measures ONE GPU only (the path shards over the batch with no "
+                         "communication; see DESIGN.md). Run with --gpus 1.\n")
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from nncv_amd import abi, resnet18_spec as spec, synth
+
+    if not torch.cuda.is_available():
+        sys.stderr.write("bench.py: no GPU visible\n")
+        sys.exit(1)
+    L = abi.lib()  # raises if the HIP library is missing: there is no fallback path
+    algo = {"auto": abi.ALGO_AUTO, "winograd": abi.ALGO_WINOGRAD, "igemm": abi.ALGO_IGEMM}[args.algo]
+
+    N, H = args.batch, 224
+    blob32 = synth.resnet18_params()
+    blob = blob32.astype(np.float16)
+    x = synth.cfg4_input(N).astype(np.float16)
+    model = L.nncv_hip_resnet18_create(blob.ctypes.data, blob.size, abi.F16, algo)
+    if not model:
+        raise RuntimeError(L.nncv_hip_last_error().decode())
+    xd = torch.from_numpy(x).cuda()
+    logits = torch.empty((N, 1000), dtype=torch.float32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def step(xt, out, n):
+        abi.check(L.nncv_hip_resnet18_forward(model, xt.data_ptr(), n, H, H, out.data_ptr(), stream))
+
+    def timed(xt, out, n, warmup, steps):
+        for _ in range(warmup):
+            step(xt, out, n)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step(xt, out, n)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps
+
+    sec = timed(xd, logits, N, args.warmup, args.steps)
+    ips = N / sec
+    flops_step = spec.flops_per_image(H) * N
+
+    # batch 1 (the other half of the headline metric)
+    x1 = xd[:1].contiguous()
+    l1 = torch.empty((1, 1000), dtype=torch.float32, device="cuda")
+    sec1 = timed(x1, l1, 1, args.warmup, max(args.steps, 50))
+
+    # event-timed per-kernel pass (separate from the timed region above: the events serialise launches)
+    abi.profile_enable(True)
+    abi.profile_report()
+    for _ in range(args.profile_steps):
+        step(xd, logits, N)
+    torch.cuda.synchronize()
+    prof = abi.profile_report()
+    abi.profile_enable(False)
+    total_ms = sum(v["ms"] for v in prof.values()) or 1.0
+    kernels = {}
+    for tag, v in sorted(prof.items(), key=lambda kv: -kv[1]["ms"]):
+        per_launch_ms = v["ms"] / v["launches"]
+        kernels[tag] = {
+            "launches_per_step": v["launches"] / args.profile_steps,
+            "ms_per_step": round(v["ms"] / args.profile_steps, 5),
+            "share": round(v["ms"] / total_ms, 4),
+            "avg_launch_us": round(per_launch_ms * 1e3, 3),
+            "tflops": round(v["flops"] / (v["ms"] * 1e-3) / 1e12, 3) if v["flops"] else None,
+            "gbs": round(v["bytes"] / (v["ms"] * 1e-3) / 1e9, 2),
+        }
+    # dominant kernel: the igemm instance with the most time
+    dom = max((t for t in prof if t.startswith("igemm")), key=lambda t: prof[t]["ms"])
+    d = prof[dom]
+    achieved = d["flops"] / (d["ms"] * 1e-3) / 1e12
+    roofline = {"kernel": dom, "bound": "mfma", "achieved": round(achieved, 3), "peak": MFMA_F16_PEAK_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 5),
+                "flops_per_launch": d["flops"] / d["launches"],
+                "avg_launch_us": round(d["ms"] / d["launches"] * 1e3, 3), "launches": d["launches"],
+                "traffic": None}
+    conv3x3_flops = 13 * 2 * 56 * 56 * 64 * 64 * 9 * N  # the 13 stride-1 3x3 layers all cost the same per image
+    out = {
+        "metric": "resnet18_fp16_bs%d_images_per_s" % N, "value": round(ips, 2), "unit": "images/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 (fp32 accumulate)",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE config 4: ResNet-18 forward, fp16, input [%d,3,224,224], seeded U[0,1] input, "
+                               "random-init Kaiming/BN-folded weights from a model.bin-order blob" % N,
+                   "batch": N, "image": H, "algo3x3": args.algo, "input_resident_in_hbm": True},
+        "tflops_effective": round(flops_step / sec / 1e12, 3),
+        "frac_of_fp16_mfma_peak": round(flops_step / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 5),
+        "conv3x3s1_gflop_per_step": round(conv3x3_flops / 1e9, 2),
+        "batch1": {"images_per_s": round(1.0 / sec1, 2), "ms_per_image": round(sec1 * 1e3, 4)},
+        "roofline": roofline,
+        "kernels": kernels,
+        "device": L.nncv_hip_device_arch().decode(),
+    }
+
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(blob32, x)
+    L.nncv_hip_resnet18_destroy(model)
+    print(json.dumps(out))
+
+
+def cpu_baseline(blob32, x16):
+    """The CPU checker timed on this host: fp32 ResNet-18 forward of the first images of the same
+    batch (half-rounded weights and input, like the parity tests), OpenMP over all host cores the
+    process may use.  Bounded: one warm-up image, then as many single images as fit in ~15 s."""
+    import numpy as np
+    import oracle
+    from nncv_amd import synth
+    hb = synth.round_fp16(blob32)
+    x = x16.astype(np.float32)
+    cores = len(os.sched_getaffinity(0))
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    t0 = time.perf_counter()
+    oracle.resnet18_forward(x[:1], hb)
+    first = time.perf_counter() - t0
+    n = int(max(1, min(8, 15.0 / max(first, 1e-3))))
+    t0 = time.perf_counter()
+    oracle.resnet18_forward(x[:n], hb)
+    dt = time.perf_counter() - t0
+    return {"value": round(n / dt, 3), "unit": "images/s", "cores": cores, "kind": "port",
+            "sample": "%d image(s) of the same batch, fp32 scalar/OpenMP restatement of the path (oracle/nncv_oracle.c), "
+                      "fp64 accumulation" % n}
+
+
+if __name__ == "__main__":
+    main()

@@ -70,6 +70,14 @@ int nncv_hip_init(int device);            /* optional; device < 0 keeps the curr
 const char* nncv_hip_last_error(void);
 const char* nncv_hip_device_arch(void);   /* e.g. "gfx950:sramecc+:xnack-" */
 
+/* Per-kernel timing with HIP events on the launch stream. While enabled every kernel launch is
+ * bracketed by two events; nncv_hip_profile_report waits for them, writes a JSON object
+ * {tag: {"launches", "ms", "flops", "bytes"}} (algorithmic flops / bytes as declared by each
+ * launcher) into buf (at most cap bytes, NUL terminated), clears the records and returns the size
+ * the full text needs. */
+void nncv_hip_profile_enable(int on);
+size_t nncv_hip_profile_report(char* buf, size_t cap);
+
 /* conv algorithms for 3x3 stride-1 layers */
 #define NNCV_HIP_ALGO_AUTO 0
 #define NNCV_HIP_ALGO_WINOGRAD 1 /* F(4x4,3x3): input/filter/output transforms + 36 batched GEMMs */

@@ -32,6 +32,7 @@ assert ctypes.sizeof(MemRef1D) == 40 and ctypes.sizeof(MemRef2D) == 56 and ctype
 EXPORTS = [
     "_mlir_ciface_forward", "_mlir_ciface_forward_f16", "_mlir_ciface_matmul", "_mlir_ciface_batch_nchw_conv",
     "nncv_hip_init", "nncv_hip_last_error", "nncv_hip_device_arch",
+    "nncv_hip_profile_enable", "nncv_hip_profile_report",
     "nncv_hip_resnet18_create", "nncv_hip_resnet18_destroy", "nncv_hip_resnet18_forward",
     "nncv_hip_resnet18_forward_tap",
     "nncv_hip_conv_create", "nncv_hip_conv_destroy", "nncv_hip_conv_algo", "nncv_hip_conv_forward",
@@ -62,6 +63,10 @@ def lib():
         L.nncv_hip_init.argtypes = [i]
         L.nncv_hip_last_error.restype = ctypes.c_char_p
         L.nncv_hip_device_arch.restype = ctypes.c_char_p
+        L.nncv_hip_profile_enable.argtypes = [i]
+        L.nncv_hip_profile_enable.restype = None
+        L.nncv_hip_profile_report.argtypes = [ctypes.c_char_p, ctypes.c_size_t]
+        L.nncv_hip_profile_report.restype = ctypes.c_size_t
         L.nncv_hip_resnet18_create.argtypes = [vp, i64, i, i]
         L.nncv_hip_resnet18_create.restype = vp
         L.nncv_hip_resnet18_destroy.argtypes = [vp]
@@ -92,6 +97,18 @@ class NncvHipError(RuntimeError):
 def check(rc):
     if rc != 0:
         raise NncvHipError(lib().nncv_hip_last_error().decode())
+
+
+def profile_enable(on):
+    lib().nncv_hip_profile_enable(1 if on else 0)
+
+
+def profile_report():
+    """-> {tag: {"launches", "ms", "flops", "bytes"}} since the last report."""
+    import json
+    buf = ctypes.create_string_buffer(1 << 16)
+    lib().nncv_hip_profile_report(buf, len(buf))
+    return json.loads(buf.value.decode())
 
 
 def np_dtype(dt):

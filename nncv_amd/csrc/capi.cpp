@@ -326,6 +326,21 @@ int nncv_hip_init(int device) {
 
 const char* nncv_hip_last_error(void) { return g_last_error.c_str(); }
 
+void nncv_hip_profile_enable(int on) {
+  guarded([&] { profiler_enable(on != 0); });
+}
+
+size_t nncv_hip_profile_report(char* buf, size_t cap) {
+  std::string r;
+  if (guarded([&] { r = profiler_report(); }) != 0) r = "{}";
+  if (buf && cap) {
+    const size_t n = std::min(cap - 1, r.size());
+    memcpy(buf, r.data(), n);
+    buf[n] = 0;
+  }
+  return r.size() + 1;
+}
+
 const char* nncv_hip_device_arch(void) {
   if (guarded([&] { Context::get().init(-1); }) != 0) return "";
   return Context::get().arch().c_str();

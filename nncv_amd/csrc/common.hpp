@@ -38,6 +38,25 @@ struct Error : std::runtime_error {
   } while (0)
 
 // ---------------------------------------------------------------------------------------------
+// Optional event timing of every launch (profiler.cpp).  `name` must be a string literal or
+// otherwise outlive the scope; flops / bytes are the ALGORITHMIC work of the launch.
+// ---------------------------------------------------------------------------------------------
+bool profiler_enabled();
+void profiler_enable(bool on);
+std::string profiler_report();  // JSON {tag: {launches, ms, flops, bytes}}; waits for the work, clears
+class ProfScope {
+ public:
+  ProfScope(const char* name, double flops, double bytes, hipStream_t s);
+  ~ProfScope();
+  ProfScope(const ProfScope&) = delete;
+  ProfScope& operator=(const ProfScope&) = delete;
+
+ private:
+  hipStream_t s_;
+  bool on_;
+};
+
+// ---------------------------------------------------------------------------------------------
 // Implicit-GEMM convolution / batched GEMM on MFMA.
 //   out[b][p][f] = epilogue( sum_k  X[b][p][k] * Wt[b][f][k] )
 // p = output pixel (n, oy, ox) of an NHWC activation tensor, k = (r, s, c) with c fastest,
@@ -58,6 +77,7 @@ struct IgemmArgs {
   int ldo;     // out/residual row pitch in elements
   int batch;   // grid.z
   long long in_bs, wt_bs, out_bs;  // batch strides in elements
+  double alg_flops;  // algorithmic flops of the launch for reporting; 0 = 2*P*F*R*S*C*batch
 };
 // in_dt: element type of in/wt (kF32 | kF16); out_dt: element type of out/residual.
 void launch_igemm(const IgemmArgs& a, int in_dt, int out_dt, hipStream_t s);

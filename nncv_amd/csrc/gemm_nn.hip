@@ -125,6 +125,7 @@ __global__ __launch_bounds__(256) void gemm_nn_f32_kernel(const float* __restric
 void launch_gemm_nn_f32(const float* A, const float* B, float* C, int M, int N, int K, hipStream_t s) {
   NNCV_REQUIRE(M > 0 && N > 0 && K > 0, "matmul: empty operand");
   NNCV_REQUIRE(K % 4 == 0 && N % 4 == 0, "matmul: K and N must be multiples of 4 (16-byte rows)");
+  ProfScope prof("gemm_nn_f32", 2.0 * M * N * K, 4.0 * ((double)M * K + (double)K * N + 2.0 * M * N), s);
   const long long big = (long long)((N + 127) / 128) * ((M + 127) / 128);
   if (big >= 256) {
     dim3 grid((N + 127) / 128, (M + 127) / 128);

@@ -213,9 +213,20 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(const IgemmArgs a) {
   }
 }
 
+template <typename T> constexpr const char* tname();
+template <> constexpr const char* tname<half_t>() { return "f16"; }
+template <> constexpr const char* tname<float>() { return "f32"; }
+
 template <typename T, typename OutT, int BP, int BF, int WP, int WF>
 static void launch_cfg(const IgemmArgs& a, hipStream_t s) {
   const int P = a.N * a.OH * a.OW;
+  static const std::string tag = std::string("igemm<") + tname<T>() + "," + tname<OutT>() + "," + std::to_string(BP) +
+                                 "," + std::to_string(BF) + "," + std::to_string(WP) + "," + std::to_string(WF) + ">";
+  const double K = (double)a.R * a.S * a.C;
+  const double flops = a.alg_flops > 0 ? a.alg_flops : 2.0 * P * a.F * K * a.batch;
+  const double bytes = sizeof(T) * ((double)a.N * a.H * a.W * a.C + (double)a.F * K) * a.batch +
+                       sizeof(OutT) * (double)P * a.F * a.batch * (a.residual ? 2 : 1);
+  ProfScope prof(tag.c_str(), flops, bytes, s);
   dim3 grid((P + BP - 1) / BP, (a.F + BF - 1) / BF, a.batch);
   hipLaunchKernelGGL((igemm_kernel<T, OutT, BP, BF, WP, WF>), grid, dim3(kThreads), 0, s, a);
 }

@@ -68,6 +68,7 @@ void launch_maxpool3x3s2_nhwc(const void* in, void* out, int dt, int N, int H, i
   const long long work = (long long)N * OH * OW * (C / vn);
   const long long grid = (work + 255) / 256;
   NNCV_REQUIRE(grid < (1ll << 31), "maxpool: grid too large");
+  ProfScope prof("maxpool3x3s2", 0.0, (double)dtype_size(dt) * N * C * ((double)H * W + (double)OH * OW), s);
   if (dt == kF16)
     hipLaunchKernelGGL((maxpool3x3s2_kernel<half_t>), dim3((unsigned)grid), dim3(256), 0, s, (const half_t*)in, (half_t*)out, N, H, W, C, OH, OW);
   else
@@ -100,6 +101,7 @@ __global__ __launch_bounds__(256) void global_avgpool_kernel(const T* __restrict
 
 void launch_global_avgpool_nhwc(const void* in, void* out, int dt, int N, int HW, int C, hipStream_t s) {
   dim3 grid((C + 63) / 64, N);
+  ProfScope prof("global_avgpool", 0.0, (double)dtype_size(dt) * N * C * (HW + 1.0), s);
   if (dt == kF16)
     hipLaunchKernelGGL((global_avgpool_kernel<half_t>), grid, dim3(256), 0, s, (const half_t*)in, (half_t*)out, HW, C);
   else
@@ -180,6 +182,7 @@ void launch_stem_pack(const void* src, int src_dt, void* dst, int dst_dt, int N,
   const long long work = (long long)N * HP * WP;
   const long long grid = (work + 255) / 256;
   NNCV_REQUIRE(grid < (1ll << 31), "stem_pack: grid too large");
+  ProfScope prof("stem_pack", 0.0, (double)dtype_size(src_dt) * N * 3 * H * W + (double)dtype_size(dst_dt) * work * 8, s);
 #define LAUNCH(TS, TD) \
   hipLaunchKernelGGL((stem_pack_kernel<TS, TD>), dim3((unsigned)grid), dim3(256), 0, s, (const TS*)src, (TD*)dst, N, H, W, HP, WP)
   if (src_dt == kF32 && dst_dt == kF32) LAUNCH(float, float);

@@ -259,6 +259,9 @@ void launch_wino43_input(const void* in, int in_dt, Strides4 st, void* V, int v_
   const long long grid = (work + blk - 1) / blk;
   NNCV_REQUIRE(grid < (1ll << 31), "wino43_input: grid too large");
   const bool contig = st.c == 1;
+  const double es = dtype_size(in_dt), vs = dtype_size(v_dt);
+  ProfScope prof(contig ? "wino43_input<nhwc>" : "wino43_input<strided>", 0.0,
+                 es * N * C * H * W + vs * 36.0 * N * TH * TW * C, s);
 #define LAUNCH(TI, TV, CC)                                                                               \
   hipLaunchKernelGGL((wino43_input_kernel<TI, TV, CC>), dim3((unsigned)grid), dim3(blk), 0, s, (const TI*)in, st, \
                      (TV*)V, N, C, H, W, pad, TH, TW)
@@ -277,6 +280,9 @@ void launch_wino43_output(const WinoOutArgs& a, int m_dt, int out_dt, hipStream_
   const long long grid = (work + blk - 1) / blk;
   NNCV_REQUIRE(grid < (1ll << 31), "wino43_output: grid too large");
   const bool contig = a.st.c == 1;
+  const double ms = dtype_size(m_dt), os = dtype_size(out_dt);
+  ProfScope prof(contig ? "wino43_output<nhwc>" : "wino43_output<strided>", 0.0,
+                 ms * 36.0 * a.N * TH * TW * a.F + os * (double)a.N * a.F * a.OH * a.OW * (a.residual ? 2 : 1), s);
 #define LAUNCH(TM, TO, CC) \
   hipLaunchKernelGGL((wino43_output_kernel<TM, TO, CC>), dim3((unsigned)grid), dim3(blk), 0, s, a, TH, TW)
   if (m_dt == kF32 && out_dt == kF32) { if (contig) LAUNCH(float, float, true); else LAUNCH(float, float, false); }

@@ -20,7 +20,8 @@ def test_maxpool(dt, N, C, H, W):
     want = oracle.maxpool3x3s2(x)
     OH, OW = want.shape[2:]
     out = empty((N, OH, OW, C), dt)
-    abi.check(abi.lib().nncv_hip_maxpool3x3s2(dt, dev(nhwc(x), dt).data_ptr(), out.data_ptr(), N, H, W, C, None))
+    xd = dev(nhwc(x), dt)  # keep every device operand alive in a variable until the call returns
+    abi.check(abi.lib().nncv_hip_maxpool3x3s2(dt, xd.data_ptr(), out.data_ptr(), N, H, W, C, None))
     got = nchw(host(out))
     assert np.array_equal(np.isnan(got), np.isnan(want))
     assert np.array_equal(np.nan_to_num(got, nan=7.0), np.nan_to_num(want, nan=7.0))  # max is exact
@@ -34,7 +35,8 @@ def test_global_avgpool(dt, N, C, H, W):
         x = synth.round_fp16(x)
     want = oracle.global_avgpool(x)
     out = empty((N, C), dt)
-    abi.check(abi.lib().nncv_hip_global_avgpool(dt, dev(nhwc(x), dt).data_ptr(), out.data_ptr(), N, H, W, C, None))
+    xd = dev(nhwc(x), dt)
+    abi.check(abi.lib().nncv_hip_global_avgpool(dt, xd.data_ptr(), out.data_ptr(), N, H, W, C, None))
     tol = 1e-6 if dt == abi.F32 else 1e-3  # fp16 result is rounded to half once
     assert np.abs(host(out) - want).max() <= tol * max(1.0, np.abs(want).max())
 
@@ -45,8 +47,8 @@ def test_matmul_device(M, N, K):
     b = synth.uniform(321, (K, N), -1, 1)
     c0 = synth.uniform(322, (M, N), -1, 1)
     want = oracle.matmul(a, b, c0)
-    c = dev(c0)
-    abi.check(abi.lib().nncv_hip_matmul_f32(dev(a).data_ptr(), dev(b).data_ptr(), c.data_ptr(), M, N, K, None))
+    ad, bd, c = dev(a), dev(b), dev(c0)
+    abi.check(abi.lib().nncv_hip_matmul_f32(ad.data_ptr(), bd.data_ptr(), c.data_ptr(), M, N, K, None))
     err = max_rel(host(c), want)
     print("matmul", M, N, K, "max_rel", err, flush=True)
     assert err < FP32_MAX_REL

@@ -23,7 +23,8 @@ def test_stages_fp32(N, C, F, H, W, layout):
     tiles = N * TH * TW
     # filter
     U = empty((36, F, C), abi.F32)
-    abi.check(L.nncv_hip_wino43_filter(abi.F32, dev(w).data_ptr(), U.data_ptr(), F, C, None))
+    wd = dev(w)  # every device operand stays alive in a variable until the call returns
+    abi.check(L.nncv_hip_wino43_filter(abi.F32, wd.data_ptr(), U.data_ptr(), F, C, None))
     U_ref = oracle.wino43_filter_transform(w)
     assert max_rel(host(U), U_ref) < 1e-6
     # input
@@ -43,8 +44,9 @@ def test_stages_fp32(N, C, F, H, W, layout):
     res = synth.normal(204, (N, F, H, W))
     out = empty((N, H, W, F) if layout == abi.NHWC else (N, F, H, W), abi.F32)
     rdev = dev(nhwc(res) if layout == abi.NHWC else res)
+    scd, shd = dev(scale), dev(shift)
     abi.check(L.nncv_hip_wino43_output(abi.F32, M.data_ptr(), out.data_ptr(), layout, N, F, H, W,
-                                       dev(scale).data_ptr(), dev(shift).data_ptr(), rdev.data_ptr(), 1, None))
+                                       scd.data_ptr(), shd.data_ptr(), rdev.data_ptr(), 1, None))
     y_ref = oracle.wino43_output_transform(M_ref, N, H, W).astype(np.float64)
     y_ref = np.maximum(y_ref * scale[None, :, None, None] + shift[None, :, None, None] + res, 0)
     got = host(out)
@@ -71,8 +73,9 @@ def test_stages_fp16_storage():
     V = empty((36, tiles, C), abi.F16)
     M = empty((36, tiles, F), abi.F16)
     out = empty((N, H, W, F), abi.F16)
-    abi.check(L.nncv_hip_wino43_filter(abi.F16, dev(w, abi.F16).data_ptr(), U.data_ptr(), F, C, None))
-    abi.check(L.nncv_hip_wino43_input(abi.F16, dev(nhwc(x), abi.F16).data_ptr(), abi.NHWC, V.data_ptr(), N, C, H, W, 1, None))
+    wd, xd = dev(w, abi.F16), dev(nhwc(x), abi.F16)
+    abi.check(L.nncv_hip_wino43_filter(abi.F16, wd.data_ptr(), U.data_ptr(), F, C, None))
+    abi.check(L.nncv_hip_wino43_input(abi.F16, xd.data_ptr(), abi.NHWC, V.data_ptr(), N, C, H, W, 1, None))
     abi.check(L.nncv_hip_wino43_gemm(abi.F16, V.data_ptr(), U.data_ptr(), M.data_ptr(), tiles, C, F, None))
     abi.check(L.nncv_hip_wino43_output(abi.F16, M.data_ptr(), out.data_ptr(), abi.NHWC, N, F, H, W, None, None, None, 0, None))
     # stage-wise: each stored tensor is the oracle's value rounded to half (up to 1 half ulp)

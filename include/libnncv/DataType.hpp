@@ -10,9 +10,16 @@
 #ifndef NNCV_LIB_NNCV_RT_DATA_TYPE_HPP_
 #define NNCV_LIB_NNCV_RT_DATA_TYPE_HPP_
 
+// the reference header pulls these in and callers (examples/Res18/main.cpp) rely on it
+#include <array>
+#include <cassert>
+#include <cmath>
+#include <complex>
 #include <cstddef>
 #include <cstdint>
+#include <iomanip>
 #include <initializer_list>
+#include <iostream>
 #include <memory>
 #include <string>
 #include <vector>

@@ -78,9 +78,20 @@ struct IgemmArgs {
   int batch;   // grid.z
   long long in_bs, wt_bs, out_bs;  // batch strides in elements
   double alg_flops;  // algorithmic flops of the launch for reporting; 0 = 2*P*F*R*S*C*batch
+  int pix_stride;    // elements between horizontally adjacent pixels; 0 = C (the stem reads 32
+                     // contiguous elements = 4 packed pixel pairs at a pixel pitch of 8)
+  unsigned in_bytes, wt_bytes;  // size of one batch slice of in / wt; 0 = derived from the geometry
 };
 // in_dt: element type of in/wt (kF32 | kF16); out_dt: element type of out/residual.
+// Dispatches to the fast kernel (igemm_fast.hip) when C is a multiple of one K step and the
+// tensors are below 2 GiB, else to the generic one (igemm.hip).
 void launch_igemm(const IgemmArgs& a, int in_dt, int out_dt, hipStream_t s);
+// 3x3 stride-1 pad-1 layers: direct convolution with the haloed input patch resident in LDS
+// (conv3x3_patch.hip); same arguments and epilogue as the igemm kernels.
+bool conv3x3_patch_applicable(const IgemmArgs& a, int in_dt);
+void launch_conv3x3_patch(const IgemmArgs& a, int in_dt, int out_dt, hipStream_t s);
+bool igemm_fast_applicable(const IgemmArgs& a, int in_dt, int out_dt);
+void launch_igemm_fast(const IgemmArgs& a, int in_dt, int out_dt, hipStream_t s);
 
 // fp32 row-major C += A.B  (linalg.matmul)
 void launch_gemm_nn_f32(const float* A, const float* B, float* C, int M, int N, int K, hipStream_t s);

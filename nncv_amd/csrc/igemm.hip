@@ -82,6 +82,7 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(const IgemmArgs a) {
   const int wp = wave % WP, wf = wave / WP;
   const int P = a.N * a.OH * a.OW;
   const int Ktot = a.R * a.S * a.C;
+  const int pix = a.pix_stride ? a.pix_stride : a.C;  // element pitch between adjacent pixels
   const int bz = blockIdx.z;
   const T* in = static_cast<const T*>(a.in) + (long long)bz * a.in_bs;
   const T* wt = static_cast<const T*>(a.wt) + (long long)bz * a.wt_bs;
@@ -98,7 +99,7 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(const IgemmArgs a) {
       const int oy = rem / a.OW, ox = rem - oy * a.OW;
       iy0[i] = oy * a.stride_h - a.pad_h;
       ix0[i] = ox * a.stride_w - a.pad_w;
-      pbase[i] = in + ((long long)n * a.H * a.W + (long long)iy0[i] * a.W + ix0[i]) * a.C;
+      pbase[i] = in + ((long long)n * a.H * a.W + (long long)iy0[i] * a.W + ix0[i]) * pix;
     } else {
       iy0[i] = ix0[i] = -(1 << 28);  // never inside the image
       pbase[i] = in;
@@ -118,7 +119,7 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(const IgemmArgs a) {
   uint4 regP[PCH], regW[FCH];
   auto load_step = [&]() {
     const bool kval = kidx < Ktot;
-    const long long koff = ((long long)kr * a.W + ks) * a.C + kc;
+    const long long koff = ((long long)kr * a.W + ks) * pix + kc;
 #pragma unroll
     for (int i = 0; i < PCH; ++i) {
       const bool ok = kval && (unsigned)(iy0[i] + kr) < (unsigned)a.H && (unsigned)(ix0[i] + ks) < (unsigned)a.W;
@@ -255,8 +256,14 @@ static void launch_typed(const IgemmArgs& a, hipStream_t s) {
   }
 }
 
-void launch_igemm(const IgemmArgs& a, int in_dt, int out_dt, hipStream_t s) {
+void launch_igemm(const IgemmArgs& a_in, int in_dt, int out_dt, hipStream_t s) {
+  IgemmArgs a = a_in;
   const int ce = in_dt == kF16 ? 8 : 4;
+  const int pix = a.pix_stride ? a.pix_stride : a.C;
+  const unsigned long long in_b = (unsigned long long)a.N * a.H * a.W * pix * dtype_size(in_dt);
+  const unsigned long long wt_b = (unsigned long long)a.F * a.R * a.S * a.C * dtype_size(in_dt);
+  if (!a.in_bytes) a.in_bytes = in_b < 0xffffffffull ? (unsigned)in_b : 0xffffffffu;
+  if (!a.wt_bytes) a.wt_bytes = wt_b < 0xffffffffull ? (unsigned)wt_b : 0xffffffffu;
   NNCV_REQUIRE(a.C % ce == 0, "igemm: C must be a multiple of the 16-byte chunk");
   NNCV_REQUIRE(a.F % 4 == 0 && a.ldo % 4 == 0, "igemm: F and ldo must be multiples of 4");
   NNCV_REQUIRE(a.batch >= 1 && a.batch <= 65535, "igemm: batch out of range");
@@ -266,6 +273,15 @@ void launch_igemm(const IgemmArgs& a, int in_dt, int out_dt, hipStream_t s) {
   NNCV_REQUIRE(a.OH >= 1 && a.OW >= 1 && a.OH <= (a.H + 2 * a.pad_h - a.R) / a.stride_h + 1 &&
                    a.OW <= (a.W + 2 * a.pad_w - a.S) / a.stride_w + 1,
                "igemm: output size does not match input/filter/stride/pad");
+  if (in_dt == out_dt && conv3x3_patch_applicable(a, in_dt)) {
+    launch_conv3x3_patch(a, in_dt, out_dt, s);
+    return;
+  }
+  if (igemm_fast_applicable(a, in_dt, out_dt)) {
+    launch_igemm_fast(a, in_dt, out_dt, s);
+    NNCV_HIP_CHECK(hipGetLastError());
+    return;
+  }
   if (in_dt == kF16 && out_dt == kF16) launch_typed<half_t, half_t>(a, s);
   else if (in_dt == kF16 && out_dt == kF32) launch_typed<half_t, float>(a, s);
   else if (in_dt == kF32 && out_dt == kF32) launch_typed<float, float>(a, s);

@@ -1,0 +1,149 @@
+// Pieces shared by the MFMA convolution kernels (igemm_fast.hip, conv3x3_patch.hip):
+// operand types, the MFMA wrappers, exact small-integer division without the ~40-instruction
+// integer divide, and the coalescing epilogue of a 64x64 wave tile.
+#pragma once
+#include "common.hpp"
+
+namespace nncv_hip {
+namespace mt {
+
+typedef half_t half8 __attribute__((ext_vector_type(8)));
+typedef half_t half4 __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T>
+struct Mma;
+template <>
+struct Mma<half_t> {  // lane = row l%32, k = 8*(l/32) .. +7
+  static __device__ __forceinline__ void run(const u32x4& a, const u32x4& b, floatx16& c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mma<float> {  // lane = row l%32, k = l/32; the 4 floats of a chunk feed 4 MFMAs
+  static __device__ __forceinline__ void run(const u32x4& a, const u32x4& b, floatx16& c) {
+    const floatx4 fa = __builtin_bit_cast(floatx4, a), fb = __builtin_bit_cast(floatx4, b);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) c = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[j], fb[j], c, 0, 0, 0);
+  }
+};
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+}
+
+// ReLU with the reference's predicate (`arith.cmpf ugt`, tests/Nets/Res18.mlir:139-141): NaN stays.
+__device__ __forceinline__ float relu_ugt(float x) { return (x <= 0.0f) ? 0.0f : x; }
+
+// x / d for 0 <= x < 2^24 and 1 <= d, given inv = 1.0f / d computed on the host: one float
+// multiply and a +-1 correction instead of the integer-divide expansion (which costs more VALU
+// time in a kernel prologue than a whole K step of MFMAs).
+__device__ __forceinline__ int fast_div(int x, int d, float inv, int* rem) {
+  int q = (int)((float)x * inv);
+  int r = x - q * d;
+  if (r >= d) { ++q; r -= d; }
+  if (r < 0) { --q; r += d; }
+  *rem = r;
+  return q;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Epilogue of one wave's 64 (pixel slots) x 64 (channels) accumulator tile, acc[i][j] = channels
+// 32i.. x slots 32j.. in the MFMA layout (lane: slot l%32, channels 8g + 4*(l/32) + e).
+// Per half tile (32 slots) the raw fp32 accumulators go through a wave-private LDS tile and come
+// back with 8 (fp16) / 16 (fp32) consecutive lanes covering the 64 channels of one pixel, so the
+// residual read and the store are whole 128/256-byte rows.  BN scale/shift, residual add and ReLU
+// are applied in fp32 on the way out: one rounding.  The scale/shift values a lane needs there
+// (its FPL channels) are loaded by EpiScale at kernel start, long before they are used.
+// Every wave of the workgroup must call epilogue_64x64 (it contains barriers); `active` disables
+// a wave.
+// ---------------------------------------------------------------------------------------------
+constexpr int kEpiPitch = 68 * 4;                    // bytes per slot row: 64 floats + 4 pad
+constexpr int kEpiWaveBytes = 32 * kEpiPitch + 128;  // + 32 row offsets
+
+template <typename OutT>
+struct EpiScale {
+  static constexpr int FPL = 16 / (int)sizeof(OutT);  // channels per lane on the way out
+  static constexpr int LPR = 64 / FPL;                // lanes per pixel row
+  float sc[FPL], sh[FPL];
+  __device__ __forceinline__ void load(int lane, int f0, int F, const float* scale, const float* shift) {
+    const int f = f0 + (lane % LPR) * FPL;
+    const bool ok = f < F;
+#pragma unroll
+    for (int q = 0; q < FPL / 4; ++q) {
+      const floatx4 a = (ok && scale) ? *reinterpret_cast<const floatx4*>(scale + f + 4 * q) : floatx4{1.f, 1.f, 1.f, 1.f};
+      const floatx4 b = (ok && shift) ? *reinterpret_cast<const floatx4*>(shift + f + 4 * q) : floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        sc[4 * q + e] = a[e];
+        sh[4 * q + e] = b[e];
+      }
+    }
+  }
+};
+
+template <typename OutT>
+__device__ __forceinline__ void epilogue_64x64(const floatx16 (&acc)[2][2], unsigned char* lds_wave, bool active,
+                                               int lane, const int (&rowoff)[2], int f0, int F, const EpiScale<OutT>& ss,
+                                               const OutT* res, OutT* out, int relu) {
+  const int lrow = lane & 31, lchunk = lane >> 5;
+  int* ro = reinterpret_cast<int*>(lds_wave + 32 * kEpiPitch);
+  constexpr int FPL = EpiScale<OutT>::FPL, LPR = EpiScale<OutT>::LPR;
+  constexpr int RPI = 64 / LPR;  // pixel rows per store instruction
+  typedef OutT VO __attribute__((ext_vector_type(FPL)));
+  const int fc = (lane % LPR) * FPL;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    __syncthreads();  // the LDS tile is free (main loop or previous half done)
+    if (active) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const floatx4 y = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+          *reinterpret_cast<floatx4*>(lds_wave + lrow * kEpiPitch + (i * 32 + 8 * g + 4 * lchunk) * 4) = y;
+        }
+      if (lchunk == 0) ro[lrow] = rowoff[j];
+    }
+    __syncthreads();
+    if (active && f0 + fc < F) {
+      // residual rows first: their latency overlaps the LDS reads
+      VO rv[32 / RPI];
+      int o[32 / RPI];
+#pragma unroll
+      for (int it = 0; it < 32 / RPI; ++it) {
+        o[it] = ro[it * RPI + lane / LPR];
+        if (res && o[it] >= 0) rv[it] = *reinterpret_cast<const VO*>(res + (long long)o[it] + f0 + fc);
+      }
+#pragma unroll
+      for (int it = 0; it < 32 / RPI; ++it) {
+        if (o[it] < 0) continue;
+        const unsigned char* src = lds_wave + (it * RPI + lane / LPR) * kEpiPitch + fc * 4;
+        float y[FPL];
+#pragma unroll
+        for (int q = 0; q < FPL / 4; ++q) {
+          const floatx4 v = *reinterpret_cast<const floatx4*>(src + q * 16);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) y[4 * q + e] = v[e] * ss.sc[4 * q + e] + ss.sh[4 * q + e];
+        }
+        if (res) {
+#pragma unroll
+          for (int e = 0; e < FPL; ++e) y[e] += (float)rv[it][e];
+        }
+        if (relu) {
+#pragma unroll
+          for (int e = 0; e < FPL; ++e) y[e] = relu_ugt(y[e]);
+        }
+        VO ov;
+#pragma unroll
+        for (int e = 0; e < FPL; ++e) ov[e] = (OutT)y[e];
+        *reinterpret_cast<VO*>(out + (long long)o[it] + f0 + fc) = ov;
+      }
+    }
+  }
+}
+
+}  // namespace mt
+}  // namespace nncv_hip

@@ -82,7 +82,8 @@ void ConvLayer::forward(const void* in, int N, int H, int W, const void* residua
     IgemmArgs a{};
     a.in = wsp; a.wt = wt_.get(); a.out = out;
     a.scale = scale_.as<float>(); a.shift = shift_.as<float>(); a.residual = residual;
-    a.N = N; a.H = HP; a.W = WP; a.C = 8; a.F = d_.F; a.R = 7; a.S = 4; a.OH = OH; a.OW = OW;
+    // a filter row is 4 consecutive pixel pairs = 32 contiguous elements: one K step
+    a.N = N; a.H = HP; a.W = WP; a.C = 32; a.pix_stride = 8; a.F = d_.F; a.R = 7; a.S = 1; a.OH = OH; a.OW = OW;
     a.stride_h = 2; a.stride_w = 1; a.pad_h = 0; a.pad_w = 0;
     a.relu = d_.relu; a.ldo = d_.F; a.batch = 1;
     a.alg_flops = 2.0 * N * OH * OW * d_.F * 147.0;  // the 7x7x3 filter, not its padded 7x8x4 packing

@@ -89,7 +89,7 @@ class Conv:
         return out
 
     def close(self):
-        if self.h:
+        if self.h and abi is not None:
             abi.lib().nncv_hip_conv_destroy(self.h)
             self.h = None
 
@@ -123,7 +123,7 @@ class Model:
         return logits, tap
 
     def close(self):
-        if self.h:
+        if self.h and abi is not None:
             abi.lib().nncv_hip_resnet18_destroy(self.h)
             self.h = None
 

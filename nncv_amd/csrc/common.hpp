@@ -81,6 +81,7 @@ struct IgemmArgs {
   int pix_stride;    // elements between horizontally adjacent pixels; 0 = C (the stem reads 32
                      // contiguous elements = 4 packed pixel pairs at a pixel pitch of 8)
   unsigned in_bytes, wt_bytes;  // size of one batch slice of in / wt; 0 = derived from the geometry
+  const void* wt_frag;  // the same 3x3 filters in fragment-major order (launch_weight_frag3x3), or null
 };
 // in_dt: element type of in/wt (kF32 | kF16); out_dt: element type of out/residual.
 // Dispatches to the fast kernel (igemm_fast.hip) when C is a multiple of one K step and the
@@ -130,6 +131,8 @@ void launch_stem_pack(const void* src, int src_dt, void* dst, int dst_dt, int N,
 // weights FCRS -> [F][R][S][Cp] (Cp >= C, zero filled), cast to dst_dt
 void launch_weight_frsc(const void* w, int w_dt, void* dst, int dst_dt, int F, int C, int R, int S, int Cp,
                         hipStream_t s);
+// 3x3 weights FCHW -> fragment-major order of conv3x3_patch.hip, F padded to a multiple of 64
+void launch_weight_frag3x3(const void* w, int w_dt, void* dst, int dst_dt, int F, int C, hipStream_t s);
 // stem weights [64,3,7,7] -> [64][7][4][8] over (pixel-pair, channel4)
 void launch_stem_weight(const void* w, int w_dt, void* dst, int dst_dt, int F, hipStream_t s);
 // BN fold: scale = gamma / sqrt(var + eps), shift = beta - mean*scale (fp32 out)

@@ -16,8 +16,8 @@
 //    output blocks still give every SIMD of the chip a 64x64 accumulator tile to work on.
 //  * A stage is KS K-steps; global loads run two stages ahead of the MFMAs (two register sets,
 //    two LDS buffers, one barrier per stage).
-//  * The epilogue goes through LDS so that residual reads and result stores are whole 128-byte
-//    rows (mfma_tile.hpp).
+//  * K groups meet in an fp32 LDS tile and the epilogue reads it back so that residual reads and
+//    result stores are whole 128-byte rows (mfma_tile.hpp).
 //  * Workgroups are renumbered so that each XCD (8 of them, round-robin over the linear workgroup
 //    id) gets a contiguous range of pixel tiles: neighbouring tiles share input rows, and each
 //    XCD has its own L2.
@@ -47,7 +47,7 @@ __global__ __launch_bounds__(64 * WP * WF * WK) void igemm_fast_kernel(const Ige
   constexpr int STAGE = KS * ROWS * kRow;
   static_assert(KS % WK == 0, "every K group needs the same number of steps per stage");
 
-  extern __shared__ __align__(16) unsigned char smem[];  // max(2 * STAGE, reduction, epilogue) bytes
+  extern __shared__ __align__(16) unsigned char smem[];  // max(2 * STAGE, output tiles) bytes
 
   // ---- which output block (XCD-aware renumbering along x) ----
   const int per_xcd = (tiles_x + kXcds - 1) / kXcds;
@@ -198,34 +198,8 @@ __global__ __launch_bounds__(64 * WP * WF * WK) void igemm_fast_kernel(const Ige
   }
   __syncthreads();
 
-  // ---- K groups meet in LDS (all stage buffers are free after the last barrier) ----
-  if (WK > 1) {
-    float* red = reinterpret_cast<float*>(smem);
-    if (wk > 0) {
-      float* dst = red + ((size_t)((wk - 1) * (WP * WF) + wpos) * 64) * 64 + lane;
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) dst[((i * 2 + j) * 16 + v) * 64] = acc[i][j][v];
-    }
-    __syncthreads();
-    if (wk == 0) {
-#pragma unroll 1
-      for (int g = 1; g < WK; ++g) {
-        const float* src = red + ((size_t)((g - 1) * (WP * WF) + wpos) * 64) * 64 + lane;
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] += src[((i * 2 + j) * 16 + v) * 64];
-      }
-    }
-  }
-
-  // ---- epilogue through LDS (only the wk == 0 waves own a finished tile) ----
+  // ---- K groups meet in an LDS tile, then whole-row stores (all stage buffers are free after the
+  // last barrier) ----
   int rowoff[2];
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
@@ -234,8 +208,7 @@ __global__ __launch_bounds__(64 * WP * WF * WK) void igemm_fast_kernel(const Ige
   }
   OutT* out = static_cast<OutT*>(a.out) + (long long)bz * a.out_bs;
   const OutT* res = a.residual ? static_cast<const OutT*>(a.residual) + (long long)bz * a.out_bs : nullptr;
-  epilogue_64x64<OutT>(acc, smem + wpos * kEpiWaveBytes, wk == 0, lane, rowoff, by * BF + wf * 64, a.F, ess, res, out,
-                       a.relu);
+  tile_reduce_store<OutT, WK>(acc, smem + wpos * kTileBytes, wk, lane, rowoff, by * BF + wf * 64, a.F, ess, res, out, a.relu);
 }
 
 namespace {
@@ -248,9 +221,8 @@ template <typename T, typename OutT, int WP, int WF, int WK, int KS>
 void launch_fast_cfg(const IgemmArgs& a, hipStream_t s) {
   constexpr int BP = 64 * WP, BF = 64 * WF;
   constexpr int stage2 = 2 * KS * (BP + BF) * kRow;
-  constexpr int red = (WK - 1) * WP * WF * 64 * 64 * 4;
-  constexpr int epi = WP * WF * kEpiWaveBytes;
-  constexpr int smem = stage2 > red ? (stage2 > epi ? stage2 : epi) : (red > epi ? red : epi);
+  constexpr int epi = WP * WF * kTileBytes;
+  constexpr int smem = stage2 > epi ? stage2 : epi;
   static const std::string tag = std::string("igemm_fast<") + tn<T>() + "," + tn<OutT>() + "," + std::to_string(WP) + "," +
                                  std::to_string(WF) + "," + std::to_string(WK) + "," + std::to_string(KS) + ">";
   auto kern = igemm_fast_kernel<T, OutT, WP, WF, WK, KS>;

@@ -50,18 +50,21 @@ __device__ __forceinline__ int fast_div(int x, int d, float inv, int* rem) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Epilogue of one wave's 64 (pixel slots) x 64 (channels) accumulator tile, acc[i][j] = channels
-// 32i.. x slots 32j.. in the MFMA layout (lane: slot l%32, channels 8g + 4*(l/32) + e).
-// Per half tile (32 slots) the raw fp32 accumulators go through a wave-private LDS tile and come
-// back with 8 (fp16) / 16 (fp32) consecutive lanes covering the 64 channels of one pixel, so the
-// residual read and the store are whole 128/256-byte rows.  BN scale/shift, residual add and ReLU
-// are applied in fp32 on the way out: one rounding.  The scale/shift values a lane needs there
-// (its FPL channels) are loaded by EpiScale at kernel start, long before they are used.
-// Every wave of the workgroup must call epilogue_64x64 (it contains barriers); `active` disables
-// a wave.
+// Reduction + epilogue of one 64 (pixel slots) x 64 (channels) output tile that NG waves ("K
+// groups") hold partial sums of, acc[i][j] = channels 32i.. x slots 32j.. in the MFMA layout
+// (lane: slot l%32, channels 8q + 4*(l/32) + e).
+//   1. In NG rounds the groups add their accumulators into one fp32 LDS tile [slot][channel]
+//      (group 0 writes, the others read-add-write; a barrier between rounds).
+//   2. Each group then takes 64/NG of the tile's rows and writes them out with 8 (fp16) / 16
+//      (fp32) consecutive lanes covering the 64 channels of one pixel, so residual reads and
+//      stores are whole 128/256-byte rows.  BN scale/shift, residual add and ReLU are applied in
+//      fp32 on the way out: one rounding.  The scale/shift values a lane needs there are loaded
+//      by EpiScale at kernel start, long before they are used.
+// Every wave of the workgroup must call tile_reduce_store (it contains NG barriers), after a
+// barrier that freed the LDS region.
 // ---------------------------------------------------------------------------------------------
-constexpr int kEpiPitch = 68 * 4;                    // bytes per slot row: 64 floats + 4 pad
-constexpr int kEpiWaveBytes = 32 * kEpiPitch + 128;  // + 32 row offsets
+constexpr int kTilePitch = 68 * 4;                     // bytes per slot row: 64 floats + 16 pad
+constexpr int kTileBytes = 64 * kTilePitch + 64 * 4;   // + 64 row offsets
 
 template <typename OutT>
 struct EpiScale {
@@ -84,64 +87,77 @@ struct EpiScale {
   }
 };
 
-template <typename OutT>
-__device__ __forceinline__ void epilogue_64x64(const floatx16 (&acc)[2][2], unsigned char* lds_wave, bool active,
-                                               int lane, const int (&rowoff)[2], int f0, int F, const EpiScale<OutT>& ss,
-                                               const OutT* res, OutT* out, int relu) {
+template <typename OutT, int NG>
+__device__ __forceinline__ void tile_reduce_store(const floatx16 (&acc)[2][2], unsigned char* tile, int g, int lane,
+                                                  const int (&rowoff)[2], int f0, int F, const EpiScale<OutT>& ss,
+                                                  const OutT* res, OutT* out, int relu) {
   const int lrow = lane & 31, lchunk = lane >> 5;
-  int* ro = reinterpret_cast<int*>(lds_wave + 32 * kEpiPitch);
-  constexpr int FPL = EpiScale<OutT>::FPL, LPR = EpiScale<OutT>::LPR;
-  constexpr int RPI = 64 / LPR;  // pixel rows per store instruction
-  typedef OutT VO __attribute__((ext_vector_type(FPL)));
-  const int fc = (lane % LPR) * FPL;
+  int* ro = reinterpret_cast<int*>(tile + 64 * kTilePitch);
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    __syncthreads();  // the LDS tile is free (main loop or previous half done)
-    if (active) {
+  for (int round = 0; round < NG; ++round) {
+    if (g == round) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const floatx4 y = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-          *reinterpret_cast<floatx4*>(lds_wave + lrow * kEpiPitch + (i * 32 + 8 * g + 4 * lchunk) * 4) = y;
-        }
-      if (lchunk == 0) ro[lrow] = rowoff[j];
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            floatx4* p = reinterpret_cast<floatx4*>(tile + (j * 32 + lrow) * kTilePitch + (i * 32 + 8 * q + 4 * lchunk) * 4);
+            floatx4 y = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+            if (round > 0) y += *p;
+            *p = y;
+          }
+      if (round == 0 && lchunk == 0) {
+        ro[lrow] = rowoff[0];
+        ro[32 + lrow] = rowoff[1];
+      }
     }
     __syncthreads();
-    if (active && f0 + fc < F) {
-      // residual rows first: their latency overlaps the LDS reads
-      VO rv[32 / RPI];
-      int o[32 / RPI];
+  }
+  constexpr int FPL = EpiScale<OutT>::FPL, LPR = EpiScale<OutT>::LPR;
+  constexpr int RPI = 64 / LPR;          // pixel rows per store instruction
+  constexpr int NIT = 64 / NG / RPI;     // store instructions per wave
+  static_assert(NIT >= 1, "too many K groups for this output type");
+  typedef OutT VO __attribute__((ext_vector_type(FPL)));
+  const int fc = (lane % LPR) * FPL;
+  const bool fok = f0 + fc < F;
+  int o[NIT];
+  floatx4 v[NIT][FPL / 4];
 #pragma unroll
-      for (int it = 0; it < 32 / RPI; ++it) {
-        o[it] = ro[it * RPI + lane / LPR];
-        if (res && o[it] >= 0) rv[it] = *reinterpret_cast<const VO*>(res + (long long)o[it] + f0 + fc);
-      }
+  for (int it = 0; it < NIT; ++it) {
+    const int row = g * (64 / NG) + it * RPI + lane / LPR;
+    o[it] = ro[row];
 #pragma unroll
-      for (int it = 0; it < 32 / RPI; ++it) {
-        if (o[it] < 0) continue;
-        const unsigned char* src = lds_wave + (it * RPI + lane / LPR) * kEpiPitch + fc * 4;
-        float y[FPL];
+    for (int q = 0; q < FPL / 4; ++q) v[it][q] = *reinterpret_cast<const floatx4*>(tile + row * kTilePitch + fc * 4 + q * 16);
+  }
+  VO rv[NIT];
+  if (res) {
 #pragma unroll
-        for (int q = 0; q < FPL / 4; ++q) {
-          const floatx4 v = *reinterpret_cast<const floatx4*>(src + q * 16);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) y[4 * q + e] = v[e] * ss.sc[4 * q + e] + ss.sh[4 * q + e];
-        }
-        if (res) {
-#pragma unroll
-          for (int e = 0; e < FPL; ++e) y[e] += (float)rv[it][e];
-        }
-        if (relu) {
-#pragma unroll
-          for (int e = 0; e < FPL; ++e) y[e] = relu_ugt(y[e]);
-        }
-        VO ov;
-#pragma unroll
-        for (int e = 0; e < FPL; ++e) ov[e] = (OutT)y[e];
-        *reinterpret_cast<VO*>(out + (long long)o[it] + f0 + fc) = ov;
-      }
+    for (int it = 0; it < NIT; ++it) {
+      // rows that are not stored read element 0 of the tensor: a valid address, no branch
+      const long long off = (fok && o[it] >= 0) ? (long long)o[it] + f0 + fc : 0;
+      rv[it] = *reinterpret_cast<const VO*>(res + off);
     }
+  }
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    float y[FPL];
+#pragma unroll
+    for (int q = 0; q < FPL / 4; ++q)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) y[4 * q + e] = v[it][q][e] * ss.sc[4 * q + e] + ss.sh[4 * q + e];
+    if (res) {
+#pragma unroll
+      for (int e = 0; e < FPL; ++e) y[e] += (float)rv[it][e];
+    }
+    if (relu) {
+#pragma unroll
+      for (int e = 0; e < FPL; ++e) y[e] = relu_ugt(y[e]);
+    }
+    VO ov;
+#pragma unroll
+    for (int e = 0; e < FPL; ++e) ov[e] = (OutT)y[e];
+    if (fok && o[it] >= 0) *reinterpret_cast<VO*>(out + (long long)o[it] + f0 + fc) = ov;
   }
 }
 

@@ -43,6 +43,10 @@ ConvLayer::ConvLayer(const Desc& d, const void* w, const void* gamma, const void
     wt_.reset((size_t)Fp * d.R * d.S * Cp * es);
     NNCV_HIP_CHECK(hipMemsetAsync(wt_.get(), 0, wt_.bytes(), s));
     launch_weight_frsc(w, d.dt, wt_.get(), d.dt, d.F, d.C, d.R, d.S, Cp, s);
+    if (d.R == 3 && d.S == 3 && d.stride == 1 && d.pad == 1 && d.C % (128 / (int)es) == 0) {
+      wfrag_.reset((size_t)((d.F + 63) / 64) * 64 * 9 * d.C * es);
+      launch_weight_frag3x3(w, d.dt, wfrag_.get(), d.dt, d.F, d.C, s);
+    }
   }
   if (gamma) {
     NNCV_REQUIRE(beta && mean && var, "conv: BN needs gamma, beta, mean and var");
@@ -96,7 +100,7 @@ void ConvLayer::forward(const void* in, int N, int H, int W, const void* residua
   }
   NNCV_REQUIRE(d_.C % (16 / (int)es) == 0 && d_.F % 4 == 0, "conv: NHWC igemm needs C %% chunk == 0 and F %% 4 == 0");
   IgemmArgs a{};
-  a.in = in; a.wt = wt_.get(); a.out = out;
+  a.in = in; a.wt = wt_.get(); a.wt_frag = wfrag_.get(); a.out = out;
   a.scale = scale_.as<float>(); a.shift = shift_.as<float>(); a.residual = residual;
   a.N = N; a.H = H; a.W = W; a.C = d_.C; a.F = d_.F; a.R = d_.R; a.S = d_.S; a.OH = OH; a.OW = OW;
   a.stride_h = a.stride_w = d_.stride; a.pad_h = a.pad_w = d_.pad;

@@ -12,7 +12,8 @@ enum ConvAlgo : int { kAlgoAuto = 0, kAlgoWinograd = 1, kAlgoIgemm = 2 };
 
 // linalg.conv_2d_nchw_fchw + BatchNorm + (residual add) + ReLU as one device operation.
 // Weights arrive in the reference's FCHW order; they are re-laid once at creation:
-//   igemm    : [F][R][S][C]   (K = (r,s,c) contiguous per filter)
+//   igemm    : [F][R][S][C]   (K = (r,s,c) contiguous per filter); 3x3 stride-1 layers also keep
+//              a fragment-major copy for the LDS-patch kernel (conv3x3_patch.hip)
 //   winograd : U[36][F][C]    (filter transform done here, like the reference folds it at
 //                              compile time, OptimizeConv2dUsingWinograd.cpp:106-150)
 class ConvLayer {
@@ -44,7 +45,7 @@ class ConvLayer {
  private:
   Desc d_;
   int algo_;
-  DeviceBuffer wt_, U_, scale_, shift_;
+  DeviceBuffer wt_, wfrag_, U_, scale_, shift_;
 };
 
 class ResNet18 {

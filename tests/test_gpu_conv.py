@@ -32,6 +32,14 @@ CASES = [  # N, C, F, H, W, R, stride, pad
     (2, 128, 64, 9, 13, 3, 1, 1),     # ragged: odd, non-square
     (1, 32, 200, 7, 7, 3, 1, 1),      # F not a multiple of the tile
     (5, 16, 8, 6, 5, 3, 2, 1),        # tiny
+    # shapes that exercise the LDS-patch 3x3 kernel's wave arrangements and tile planner
+    (4, 64, 64, 56, 56, 3, 1, 1),     # 4x2 waves, TH=4 row tiles, one channel slab
+    (3, 128, 128, 28, 28, 3, 1, 1),   # 4x2 waves, TH=7, two slabs, two filter blocks
+    (5, 256, 64, 14, 14, 3, 1, 1),    # few workgroups -> 2x4 waves, four slabs
+    (9, 64, 128, 7, 7, 3, 1, 1),      # several images per tile, last tile short of images
+    (2, 64, 72, 30, 62, 3, 1, 1),     # widest row the patch loader takes, F not a multiple of 64
+    (1, 64, 64, 20, 64, 3, 1, 1),     # too wide for the patch kernel: falls back to implicit GEMM
+    (2, 64, 64, 23, 17, 3, 1, 1),     # ragged: H not a multiple of the row tile
 ]
 
 

@@ -20,8 +20,11 @@
 // fp32 LDS tile from which the epilogue (scale/shift, residual, ReLU) stores whole rows
 // (mfma_tile.hpp).  Splitting K inside the workgroup rather than shrinking the pixel tile keeps
 // one 16-byte LDS read per MFMA, gives every SIMD two resident waves, and lets small feature maps
-// still fill 256 CUs:   56x56, 28x28 -> WS=4, WK=2 ; 14x14 -> WS=2, WK=4 ; 7x7 -> WS=1, WK=4.
+// still fill 256 CUs.  All instances are 4 waves (one per SIMD; two workgroups share a CU):
+//   56x56, 28x28 -> WS=4, WK=1 ; 14x14 -> WS=2, WK=2 ; 7x7 -> WS=1, WK=4.
 // LDS pixel pitch is 128 + 16 bytes: consecutive pixels land 36 banks apart.
+#include <type_traits>
+
 #include "mfma_tile.hpp"
 
 namespace nncv_hip {
@@ -32,7 +35,6 @@ namespace {
 constexpr int kPitch = 144;            // LDS bytes per patch pixel: 128 payload + 16 pad
 constexpr unsigned kOOBp = 0x7fff0000u;
 constexpr int kXcdsP = 8;
-constexpr int kPasses = 6;             // patch loader passes per thread (upper bound)
 
 template <int WS> struct PatchCap;     // patch capacity in pixels for 64*WS slots
 template <> struct PatchCap<4> { static constexpr int pix = 384; };
@@ -59,20 +61,24 @@ struct PatchArgs {
 template <int WS, int WK>
 struct PatchCfg {
   static constexpr int NW = WS * WK, NT = 64 * NW;
+  static constexpr int cover = WS == 4 ? 384 : WS == 2 ? 256 : 192;  // padded patch pixels the loader can walk
+  static constexpr int passes = cover / (NT / 8);  // loader passes per thread: NT/8 pixels each
+  static constexpr int nset = WK == 1 ? 2 : 3;     // weight register sets (taps in flight)
   static constexpr int cap = PatchCap<WS>::pix;
   static constexpr int patch_bytes = cap * kPitch;
+  static constexpr int load_bytes = patch_bytes + NT * 16;  // + one dump slot per thread
   static constexpr int tile_bytes = WS * kTileBytes;
-  static constexpr int smem = patch_bytes > tile_bytes ? patch_bytes : tile_bytes;
+  static constexpr int smem = load_bytes > tile_bytes ? load_bytes : tile_bytes;
 };
 
 template <typename T, typename OutT, int WS, int WK>
 __global__ __launch_bounds__(64 * WS * WK) void conv3x3_patch_kernel(const PatchArgs a) {
   typedef PatchCfg<WS, WK> Cfg;
-  constexpr int NT = Cfg::NT;
+  constexpr int NT = Cfg::NT, kPasses = Cfg::passes, NSET = Cfg::nset;
   constexpr int ES = sizeof(T);
   constexpr int KPG = 4 / WK;     // 32-byte K sub-steps per K group and tap
   constexpr int NF = 2 * KPG;     // weight fragments (kilobytes) per wave and tap
-  static_assert(WK == 2 || WK == 4, "K groups split the four sub-steps of a tap");
+  static_assert(WK == 1 || WK == 2 || WK == 4, "K groups split the four sub-steps of a tap");
   extern __shared__ __align__(16) unsigned char smem[];
   unsigned char* patch = smem;
 
@@ -89,11 +95,12 @@ __global__ __launch_bounds__(64 * WS * WK) void conv3x3_patch_kernel(const Patch
   const int lrow = lane & 31, lchunk = lane >> 5;
   const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(a.in, a.in_bytes);
   const __amdgpu_buffer_rsrc_t rs_wf = make_rsrc(a.wf, a.wf_bytes);
-  const int nslab = a.C * ES / 128;
+  // The widest tile keeps no patch prefetch registers alive in the tap loop: single-slab layers only.
+  const int nslab = WS == 4 ? 1 : a.C * ES / 128;
   const int niter = nslab * 9;  // one iteration = one tap of one slab
 
   // ---- weights: iteration `it`, sub-step k of this K group, filter half i is the kilobyte at
-  //      wbase + it*8192 + (k*2+i)*1024; three register sets hold iterations it, it+1, it+2 ----
+  //      wbase + it*8192 + (k*2+i)*1024; NSET register sets hold iterations it .. it+NSET-1 ----
   const int wbase = (blockIdx.y * niter * 8 + wk * KPG * 2) * 1024;
   const unsigned wlane = lane * 16;
   auto wload = [&](u32x4(&r)[NF], int it) {
@@ -101,47 +108,59 @@ __global__ __launch_bounds__(64 * WS * WK) void conv3x3_patch_kernel(const Patch
 #pragma unroll
     for (int q = 0; q < NF; ++q) r[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_wf, wlane, so + q * 1024, 0);
   };
-  u32x4 wregs[3][NF];
-  wload(wregs[0], 0);
-  wload(wregs[1], 1);
-  wload(wregs[2], 2);
+  u32x4 wregs[NSET][NF];
+#pragma unroll
+  for (int q = 0; q < NSET; ++q) wload(wregs[q], q);
 
   // epilogue scale/shift of this lane's output channels: requested now, used at the very end
   EpiScale<OutT> ess;
   ess.load(lane, f0blk, a.F, a.scale, a.shift);
 
-  // ---- patch loader: 8 threads per pixel; loader rows of 2^rw_log pixels, no integer division ----
+  // ---- patch loader: 8 threads per pixel, NT/8 pixels per pass; the patch is walked as rows of
+  //      2^rw_log pixels (>= W+2), so row and column of a pass are shifts and masks ----
   const int p8 = tid >> 3, pc = (tid & 7) * 16;
-  const int px = p8 & ((1 << a.rw_log) - 1), rsub = p8 >> a.rw_log;
-  const int rpp = (NT / 8) >> a.rw_log;  // patch rows per pass
   const int prows = a.TN * PH;
+  const int rwm = (1 << a.rw_log) - 1;
+  const unsigned ces = (unsigned)(a.C * ES);
   unsigned pvoff[kPasses];
-  unsigned pmask = 0;
+  if (a.TN == 1) {  // one image per tile: patch row r is image row y0 - 1 + r
+    const int rowbase = (n0 * a.H + y0 - 1) * a.W - 1;
 #pragma unroll
-  for (int i = 0; i < kPasses; ++i) {
-    const int r = i * rpp + rsub;
-    unsigned off = kOOBp;
-    if (px < PW && r < prows) {
-      pmask |= 1u << i;
-      int py;
-      const int nl = fast_div(r, PH, a.inv_ph, &py);
-      const int n = n0 + nl, iy = y0 + py - 1, ix = px - 1;
-      if (n < a.N && (unsigned)iy < (unsigned)a.H && (unsigned)ix < (unsigned)a.W)
-        off = (unsigned)((((n * a.H + iy) * a.W + ix) * a.C) * ES + pc);
+    for (int i = 0; i < kPasses; ++i) {
+      const int q = i * (NT / 8) + p8;
+      const int r = q >> a.rw_log, px = q & rwm;
+      const bool ok = (r < prows) & ((unsigned)(y0 - 1 + r) < (unsigned)a.H) & ((unsigned)(px - 1) < (unsigned)a.W);
+      const unsigned off = __umul24((unsigned)(rowbase + (int)__umul24(r, a.W) + px), ces) + pc;
+      pvoff[i] = ok ? off : kOOBp;
     }
-    pvoff[i] = off;
+  } else {
+#pragma unroll
+    for (int i = 0; i < kPasses; ++i) {
+      const int q = i * (NT / 8) + p8;
+      const int r = q >> a.rw_log, px = q & rwm;
+      int py;
+      const int n = n0 + fast_div(r, PH, a.inv_ph, &py);
+      const int iy = y0 + py - 1;
+      const bool ok = (r < prows) & (n < a.N) & ((unsigned)iy < (unsigned)a.H) & ((unsigned)(px - 1) < (unsigned)a.W);
+      const unsigned off = __umul24((unsigned)((n * a.H + iy) * a.W + px - 1), ces) + pc;
+      pvoff[i] = ok ? off : kOOBp;
+    }
   }
-  unsigned char* const pdst = patch + (rsub * PW + px) * kPitch + pc;
-  const int ppass = rpp * PW * kPitch;  // LDS bytes between passes
   u32x4 pregs[kPasses];
   auto pload = [&](int slab) {
 #pragma unroll
     for (int i = 0; i < kPasses; ++i) pregs[i] = __builtin_amdgcn_raw_buffer_load_b128(rs_in, pvoff[i] + slab * 128, 0, 0);
   };
+  // Lanes whose pass lies outside the patch store to a private dump slot behind it: no divergence.
+  const int dump = Cfg::patch_bytes + tid * 16;
   auto pstore = [&]() {
 #pragma unroll
-    for (int i = 0; i < kPasses; ++i)
-      if (pmask & (1u << i)) *reinterpret_cast<u32x4*>(pdst + i * ppass) = pregs[i];
+    for (int i = 0; i < kPasses; ++i) {
+      const int q = i * (NT / 8) + p8;
+      const int r = q >> a.rw_log, px = q & rwm;
+      const int dst = (int)__umul24(__umul24(r, PW) + px, kPitch) + pc;
+      *reinterpret_cast<u32x4*>(patch + (((px < PW) & (r < prows)) ? dst : dump)) = pregs[i];
+    }
   };
   pload(0);
 
@@ -152,15 +171,12 @@ __global__ __launch_bounds__(64 * WS * WK) void conv3x3_patch_kernel(const Patch
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int sl = ws * 64 + j * 32 + lrow;
-    int nl = 0, ty = 0, tx = 0;
-    bool ok = sl < nslots;
-    if (ok) {
-      int rem;
-      nl = fast_div(sl, a.TH * a.W, a.inv_thw, &rem);
-      ty = fast_div(rem, a.W, a.inv_w, &tx);
-      ok = (n0 + nl) < a.N && (y0 + ty) < a.H;
-    }
-    sbase[j] = ((nl * PH + ty) * PW + tx) * kPitch + (lchunk + 2 * wk * KPG) * 16;
+    int nl = 0, rem = sl, tx;
+    if (a.TN > 1) nl = fast_div(sl, a.TH * a.W, a.inv_thw, &rem);
+    const int ty = fast_div(rem, a.W, a.inv_w, &tx);
+    const bool ok = (sl < nslots) & ((n0 + nl) < a.N) & ((y0 + ty) < a.H);
+    // slots beyond the tile read pixel 0 of the patch; their results are never stored
+    sbase[j] = (ok ? (int)__umul24(__umul24(__umul24(nl, PH) + ty, PW) + tx, kPitch) : 0) + (lchunk + 2 * wk * KPG) * 16;
     obase[j] = ok ? (((n0 + nl) * a.H + y0 + ty) * a.W + tx) * a.F : -1;
   }
 
@@ -182,14 +198,18 @@ __global__ __launch_bounds__(64 * WS * WK) void conv3x3_patch_kernel(const Patch
 
   u32x4 fp[2];
   ldp(fp, 0, 0);
-  // One trip = one filter row = three taps, so the weight register sets rotate statically.
   int tr = 0, slab = 0;
-  for (int it0 = 0; it0 < niter; it0 += 3) {
+  // One filter row = three taps; `s0` is the register set of its first tap (sets rotate per tap).
+  auto filter_row = [&](int it0, auto s0) {
+    constexpr int S0 = decltype(s0)::value;
     // next slab's patch is requested at the first tap of this slab and lands after its last tap
     if (tr == 0 && slab + 1 < nslab) pload(slab + 1);
     const int ntr = tr == 2 ? 0 : tr + 1;
 #pragma unroll
     for (int ts = 0; ts < 3; ++ts) {
+      constexpr int dummy = 0;
+      (void)dummy;
+      const int set = (S0 + ts) % NSET;
       const bool new_patch = ts == 2 && tr == 2 && slab + 1 < nslab;  // the patch changes after this tap
       const int tapoff = (tr * PW + ts) * kPitch;
       const int ntapoff = ts == 2 ? (ntr * PW) * kPitch : tapoff + kPitch;
@@ -201,11 +221,11 @@ __global__ __launch_bounds__(64 * WS * WK) void conv3x3_patch_kernel(const Patch
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
-          for (int j = 0; j < 2; ++j) Mma<T>::run(wregs[ts][k * 2 + i], fp[j], acc[i][j]);
+          for (int j = 0; j < 2; ++j) Mma<T>::run(wregs[set][k * 2 + i], fp[j], acc[i][j]);
 #pragma unroll
         for (int j = 0; j < 2; ++j) fp[j] = np[j];
       }
-      wload(wregs[ts], it0 + ts + 3);  // this set is consumed: refill it three taps ahead
+      wload(wregs[set], it0 + ts + NSET);  // this set is consumed: refill it NSET taps ahead
       if (new_patch) {
         __syncthreads();  // every wave is done with the old patch
         pstore();
@@ -215,6 +235,14 @@ __global__ __launch_bounds__(64 * WS * WK) void conv3x3_patch_kernel(const Patch
     }
     tr = ntr;
     if (tr == 0) ++slab;
+  };
+  if (NSET == 3) {
+    for (int it0 = 0; it0 < niter; it0 += 3) filter_row(it0, std::integral_constant<int, 0>());
+  } else {  // two sets: the rotation repeats every two rows
+    for (int it0 = 0; it0 < niter; it0 += 6) {
+      filter_row(it0, std::integral_constant<int, 0>());
+      if (it0 + 3 < niter) filter_row(it0 + 3, std::integral_constant<int, 1>());
+    }
   }
   __syncthreads();  // every wave is done with the patch: LDS becomes the output tiles
 
@@ -223,14 +251,13 @@ __global__ __launch_bounds__(64 * WS * WK) void conv3x3_patch_kernel(const Patch
 }
 
 // Tile choice for 64*ws slots: TN images x TH rows x W columns, patch of at most `cap` pixels,
-// loaded in at most kPasses passes of `pix_per_pass` pixels (rows of 2^rw_log).
-static bool plan_tile(int N, int H, int W, int slots, int cap, int pix_per_pass, int* TN, int* TH, int* rw_log) {
+// which the loader walks as rows of 2^rw_log pixels, `cover` padded pixels at most.
+static bool plan_tile(int N, int H, int W, int slots, int cap, int cover, int* TN, int* TH, int* rw_log) {
   const int PW = W + 2;
   int lg = 0;
   while ((1 << lg) < PW) ++lg;
-  if ((1 << lg) > pix_per_pass || W > slots) return false;
-  const int rpp = pix_per_pass >> lg;
-  const int max_rows = kPasses * rpp;  // patch rows the loader can cover
+  if ((1 << lg) > 64 || W > slots) return false;
+  const int max_rows = cover >> lg;  // patch rows the loader can cover
   auto fits = [&](int tn, int th) { return tn * th * W <= slots && tn * (th + 2) * PW <= cap && tn * (th + 2) <= max_rows; };
   int thmax = 0;
   for (int th = 1; th <= H; ++th)
@@ -251,28 +278,31 @@ static bool plan_tile(int N, int H, int W, int slots, int cap, int pix_per_pass,
 }
 
 // Picks the wave arrangement: the largest pixel tile that still gives (about) every CU a workgroup.
-static bool plan_patch(int N, int H, int W, int F, int* WS, int* TN, int* TH, int* rw_log) {
+static bool plan_patch(int N, int H, int W, int F, int slabs, int* WS, int* TN, int* TH, int* rw_log) {
   static const int force = [] {
     const char* e = getenv("NNCV_HIP_PATCH_WS");
     return e ? atoi(e) : 0;
   }();
   const int fb = (F + 63) / 64;
-  long long best_blocks = 0;
+  // Score = fraction of the MFMA slots that carry real pixels x fraction of the 256 CUs that get
+  // a workgroup; ties go to the wider tile (fewer weight re-reads, no cross-wave reduction).
+  double best = 0.0;
   for (int ws : {4, 2, 1}) {
     if (force && ws != force) continue;
+    if (ws == 4 && slabs != 1) continue;  // the WS=4 instance handles one slab
     const int cap = ws == 4 ? PatchCap<4>::pix : ws == 2 ? PatchCap<2>::pix : PatchCap<1>::pix;
-    const int nt = ws == 1 ? 256 : 512;  // threads of the (WS, WK) instance used for this ws
     int tn, th, lg;
-    if (!plan_tile(N, H, W, 64 * ws, cap, nt / 8, &tn, &th, &lg)) continue;
-    const long long blocks = (long long)((N + tn - 1) / tn) * ((H + th - 1) / th) * fb;
-    // the first (largest) arrangement that fills the chip wins; failing that, the one with the
-    // most workgroups
-    if (blocks > best_blocks) {
-      best_blocks = blocks; *WS = ws; *TN = tn; *TH = th; *rw_log = lg;
+    const int cover = ws == 4 ? PatchCfg<4, 1>::cover : ws == 2 ? PatchCfg<2, 2>::cover : PatchCfg<1, 4>::cover;
+    if (!plan_tile(N, H, W, 64 * ws, cap, cover, &tn, &th, &lg)) continue;
+    const long long tiles = (long long)((N + tn - 1) / tn) * ((H + th - 1) / th);
+    const double used = (double)N * H * W / ((double)tiles * 64 * ws);
+    const double fill = tiles * fb >= 256 ? 1.0 : (double)(tiles * fb) / 256.0;
+    const double score = used * fill;
+    if (score > best * 1.05) {
+      best = score; *WS = ws; *TN = tn; *TH = th; *rw_log = lg;
     }
-    if (blocks >= 224) break;
   }
-  return best_blocks != 0;
+  return best > 0.0;
 }
 
 bool conv3x3_patch_applicable(const IgemmArgs& a, int in_dt) {
@@ -281,9 +311,9 @@ bool conv3x3_patch_applicable(const IgemmArgs& a, int in_dt) {
   int ws, tn, th, lg;
   return !off && a.wt_frag && a.R == 3 && a.S == 3 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 1 && a.pad_w == 1 &&
          a.batch == 1 && a.pix_stride == 0 && a.C % slab == 0 && a.F % 8 == 0 && a.ldo == a.F &&
-         (long long)a.N * a.H * a.W * a.F < (1ll << 31) && a.in_bytes < kOOBp &&
+         (long long)a.N * a.H * a.W * a.F < (1ll << 31) && (long long)a.N * a.H * a.W < (1 << 24) && a.in_bytes < kOOBp &&
          (long long)((a.F + 63) / 64) * 64 * 9 * a.C * (long long)dtype_size(in_dt) < (1ll << 31) &&
-         plan_patch(a.N, a.H, a.W, a.F, &ws, &tn, &th, &lg);
+         plan_patch(a.N, a.H, a.W, a.F, a.C / slab, &ws, &tn, &th, &lg);
 }
 
 template <typename T, typename OutT, int WS, int WK>
@@ -305,7 +335,8 @@ void launch_conv3x3_patch(const IgemmArgs& g, int in_dt, int out_dt, hipStream_t
   a.in = g.in; a.wf = g.wt_frag; a.out = g.out; a.scale = g.scale; a.shift = g.shift; a.residual = g.residual;
   a.N = g.N; a.H = g.H; a.W = g.W; a.C = g.C; a.F = g.F; a.relu = g.relu;
   int ws = 0;
-  NNCV_REQUIRE(plan_patch(a.N, a.H, a.W, a.F, &ws, &a.TN, &a.TH, &a.rw_log), "conv3x3_patch: no tile fits");
+  NNCV_REQUIRE(plan_patch(a.N, a.H, a.W, a.F, a.C * (int)dtype_size(in_dt) / 128, &ws, &a.TN, &a.TH, &a.rw_log),
+               "conv3x3_patch: no tile fits");
   a.tiles_y = (a.H + a.TH - 1) / a.TH;
   a.tiles = ((a.N + a.TN - 1) / a.TN) * a.tiles_y;
   a.in_bytes = g.in_bytes;
@@ -320,12 +351,12 @@ void launch_conv3x3_patch(const IgemmArgs& g, int in_dt, int out_dt, hipStream_t
   const bool h = in_dt == kF16 && out_dt == kF16, f = in_dt == kF32 && out_dt == kF32;
   NNCV_REQUIRE(h || f, "conv3x3_patch: unsupported dtype combination");
   if (h) {
-    if (ws == 4) launch_patch_cfg<half_t, half_t, 4, 2>(a, flops, bytes, "conv3x3_patch<f16,4,2>", s);
-    else if (ws == 2) launch_patch_cfg<half_t, half_t, 2, 4>(a, flops, bytes, "conv3x3_patch<f16,2,4>", s);
+    if (ws == 4) launch_patch_cfg<half_t, half_t, 4, 1>(a, flops, bytes, "conv3x3_patch<f16,4,1>", s);
+    else if (ws == 2) launch_patch_cfg<half_t, half_t, 2, 2>(a, flops, bytes, "conv3x3_patch<f16,2,2>", s);
     else launch_patch_cfg<half_t, half_t, 1, 4>(a, flops, bytes, "conv3x3_patch<f16,1,4>", s);
   } else {
-    if (ws == 4) launch_patch_cfg<float, float, 4, 2>(a, flops, bytes, "conv3x3_patch<f32,4,2>", s);
-    else if (ws == 2) launch_patch_cfg<float, float, 2, 4>(a, flops, bytes, "conv3x3_patch<f32,2,4>", s);
+    if (ws == 4) launch_patch_cfg<float, float, 4, 1>(a, flops, bytes, "conv3x3_patch<f32,4,1>", s);
+    else if (ws == 2) launch_patch_cfg<float, float, 2, 2>(a, flops, bytes, "conv3x3_patch<f32,2,2>", s);
     else launch_patch_cfg<float, float, 1, 4>(a, flops, bytes, "conv3x3_patch<f32,1,4>", s);
   }
   NNCV_HIP_CHECK(hipGetLastError());

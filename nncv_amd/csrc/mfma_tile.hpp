@@ -64,24 +64,36 @@ __device__ __forceinline__ int fast_div(int x, int d, float inv, int* rem) {
 // barrier that freed the LDS region.
 // ---------------------------------------------------------------------------------------------
 constexpr int kTilePitch = 68 * 4;                     // bytes per slot row: 64 floats + 16 pad
-constexpr int kTileBytes = 64 * kTilePitch + 64 * 4;   // + 64 row offsets
+constexpr int kTileBytes = 64 * kTilePitch;
 
 template <typename OutT>
 struct EpiScale {
   static constexpr int FPL = 16 / (int)sizeof(OutT);  // channels per lane on the way out
   static constexpr int LPR = 64 / FPL;                // lanes per pixel row
   float sc[FPL], sh[FPL];
+  // F must be a multiple of FPL; lanes past F read the last valid group (their rows are not stored).
   __device__ __forceinline__ void load(int lane, int f0, int F, const float* scale, const float* shift) {
-    const int f = f0 + (lane % LPR) * FPL;
-    const bool ok = f < F;
+    int f = f0 + (lane % LPR) * FPL;
+    f = f < F ? f : F - FPL;
 #pragma unroll
-    for (int q = 0; q < FPL / 4; ++q) {
-      const floatx4 a = (ok && scale) ? *reinterpret_cast<const floatx4*>(scale + f + 4 * q) : floatx4{1.f, 1.f, 1.f, 1.f};
-      const floatx4 b = (ok && shift) ? *reinterpret_cast<const floatx4*>(shift + f + 4 * q) : floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int e = 0; e < FPL; ++e) {
+      sc[e] = 1.f;
+      sh[e] = 0.f;
+    }
+    if (scale) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        sc[4 * q + e] = a[e];
-        sh[4 * q + e] = b[e];
+      for (int q = 0; q < FPL / 4; ++q) {
+        const floatx4 a = *reinterpret_cast<const floatx4*>(scale + f + 4 * q);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sc[4 * q + e] = a[e];
+      }
+    }
+    if (shift) {
+#pragma unroll
+      for (int q = 0; q < FPL / 4; ++q) {
+        const floatx4 b = *reinterpret_cast<const floatx4*>(shift + f + 4 * q);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sh[4 * q + e] = b[e];
       }
     }
   }
@@ -92,7 +104,32 @@ __device__ __forceinline__ void tile_reduce_store(const floatx16 (&acc)[2][2], u
                                                   const int (&rowoff)[2], int f0, int F, const EpiScale<OutT>& ss,
                                                   const OutT* res, OutT* out, int relu) {
   const int lrow = lane & 31, lchunk = lane >> 5;
-  int* ro = reinterpret_cast<int*>(tile + 64 * kTilePitch);
+  constexpr int FPL = EpiScale<OutT>::FPL, LPR = EpiScale<OutT>::LPR;
+  constexpr int RPI = 64 / LPR;          // pixel rows per store instruction
+  constexpr int NIT = 64 / NG / RPI;     // store instructions per wave
+  static_assert(NIT >= 1, "too many K groups for this output type");
+  typedef OutT VO __attribute__((ext_vector_type(FPL)));
+  const int fc = (lane % LPR) * FPL;
+  const bool fok = f0 + fc < F;
+  // Output offsets of the rows this lane stores, fetched from the lanes that own those slots, and
+  // the residual rows requested before the reduction so that their latency hides behind it.
+  int o[NIT];
+  VO rv[NIT];
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int row = g * (64 / NG) + it * RPI + lane / LPR;
+    const int o0 = __shfl(rowoff[0], row & 31), o1 = __shfl(rowoff[1], row & 31);
+    o[it] = (row & 32) ? o1 : o0;
+    if (!fok) o[it] = -1;
+  }
+  if (res) {
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      // rows that are not stored read element 0 of the tensor: a valid address, no branch
+      const long long off = o[it] >= 0 ? (long long)o[it] + f0 + fc : 0;
+      rv[it] = *reinterpret_cast<const VO*>(res + off);
+    }
+  }
 #pragma unroll
   for (int round = 0; round < NG; ++round) {
     if (g == round) {
@@ -107,37 +144,15 @@ __device__ __forceinline__ void tile_reduce_store(const floatx16 (&acc)[2][2], u
             if (round > 0) y += *p;
             *p = y;
           }
-      if (round == 0 && lchunk == 0) {
-        ro[lrow] = rowoff[0];
-        ro[32 + lrow] = rowoff[1];
-      }
     }
     __syncthreads();
   }
-  constexpr int FPL = EpiScale<OutT>::FPL, LPR = EpiScale<OutT>::LPR;
-  constexpr int RPI = 64 / LPR;          // pixel rows per store instruction
-  constexpr int NIT = 64 / NG / RPI;     // store instructions per wave
-  static_assert(NIT >= 1, "too many K groups for this output type");
-  typedef OutT VO __attribute__((ext_vector_type(FPL)));
-  const int fc = (lane % LPR) * FPL;
-  const bool fok = f0 + fc < F;
-  int o[NIT];
   floatx4 v[NIT][FPL / 4];
 #pragma unroll
   for (int it = 0; it < NIT; ++it) {
     const int row = g * (64 / NG) + it * RPI + lane / LPR;
-    o[it] = ro[row];
 #pragma unroll
     for (int q = 0; q < FPL / 4; ++q) v[it][q] = *reinterpret_cast<const floatx4*>(tile + row * kTilePitch + fc * 4 + q * 16);
-  }
-  VO rv[NIT];
-  if (res) {
-#pragma unroll
-    for (int it = 0; it < NIT; ++it) {
-      // rows that are not stored read element 0 of the tensor: a valid address, no branch
-      const long long off = (fok && o[it] >= 0) ? (long long)o[it] + f0 + fc : 0;
-      rv[it] = *reinterpret_cast<const VO*>(res + off);
-    }
   }
 #pragma unroll
   for (int it = 0; it < NIT; ++it) {
@@ -157,7 +172,7 @@ __device__ __forceinline__ void tile_reduce_store(const floatx16 (&acc)[2][2], u
     VO ov;
 #pragma unroll
     for (int e = 0; e < FPL; ++e) ov[e] = (OutT)y[e];
-    if (fok && o[it] >= 0) *reinterpret_cast<VO*>(out + (long long)o[it] + f0 + fc) = ov;
+    if (o[it] >= 0) *reinterpret_cast<VO*>(out + (long long)o[it] + f0 + fc) = ov;
   }
 }
 

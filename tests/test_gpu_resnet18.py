@@ -75,3 +75,32 @@ def test_fp16_small_batch(blob):
         assert err < FP16_REL_L2
         if algo == abi.ALGO_IGEMM:
             assert (got.argmax(1) == want.argmax(1)).all()
+
+
+def test_graph_replay_matches_eager_every_time(blob):
+    """The device entry point captures the forward into a HIP graph on the second call with the
+    same buffers and replays it afterwards: every replay must equal the eager result, also when the
+    input buffer's contents change between replays and other work runs in between."""
+    hb = synth.round_fp16(blob)
+    m = Model(hb, abi.F16)
+    xs = [synth.round_fp16(synth.uniform(4100 + i, (2, 3, 64, 64), 0.0, 1.0)) for i in range(3)]
+    xd = dev(xs[0], abi.F16)
+    logits = torch.empty((2, 1000), dtype=torch.float32, device="cuda")
+    L = abi.lib()
+
+    def run():
+        abi.check(L.nncv_hip_resnet18_forward(m.h, xd.data_ptr(), 2, 64, 64, logits.data_ptr(), None))
+        return logits.cpu().numpy().copy()
+
+    eager = run()  # first sighting: eager
+    want = oracle.resnet18_forward(xs[0], hb)
+    assert rel_l2(eager, want) < FP16_REL_L2
+    for rep in range(6):  # capture on the first of these, replay on the rest
+        x = xs[rep % 3]
+        xd.copy_(torch.from_numpy(x.astype(np.float16)))
+        other = torch.randn(256, 256, device="cuda") @ torch.randn(256, 256, device="cuda")  # unrelated eager work
+        torch.cuda.synchronize()
+        got = run()
+        ref = host(Model(hb, abi.F16)(dev(x, abi.F16)))  # a fresh handle never replays: eager result
+        assert np.array_equal(got, ref), rep
+        assert other.shape == (256, 256)

@@ -54,6 +54,7 @@ struct PatchArgs {
   int tiles_y;           // ceil(H / TH)
   int tiles;             // ceil(N / TN) * tiles_y
   int rw_log;            // patch loader: 2^rw_log >= W + 2 pixels per loader row
+  int xcd_by_filter;     // XCD <- filter block instead of XCD <- tile range
   unsigned in_bytes, wf_bytes;
   float inv_ph, inv_thw, inv_w;  // 1/(TH+2), 1/(TH*W), 1/W
 };
@@ -72,7 +73,7 @@ struct PatchCfg {
 };
 
 template <typename T, typename OutT, int WS, int WK>
-__global__ __launch_bounds__(64 * WS * WK) void conv3x3_patch_kernel(const PatchArgs a) {
+__global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv3x3_patch_kernel(const PatchArgs a) {
   typedef PatchCfg<WS, WK> Cfg;
   constexpr int NT = Cfg::NT, kPasses = Cfg::passes, NSET = Cfg::nset;
   constexpr int ES = sizeof(T);
@@ -82,10 +83,22 @@ __global__ __launch_bounds__(64 * WS * WK) void conv3x3_patch_kernel(const Patch
   extern __shared__ __align__(16) unsigned char smem[];
   unsigned char* patch = smem;
 
-  const int per_xcd = (a.tiles + kXcdsP - 1) / kXcdsP;
-  const int tile = (blockIdx.x % kXcdsP) * per_xcd + blockIdx.x / kXcdsP;
+  // Workgroups are dealt to the 8 XCDs (each with its own L2) round-robin by linear id.  Normally an
+  // XCD takes a contiguous range of pixel tiles (neighbouring tiles share halo rows); when the
+  // filters outgrow one L2 it takes one 64-filter block instead, so that its weights stay resident.
+  int tile, fblk;
+  if (a.xcd_by_filter) {
+    const int lin = blockIdx.y * gridDim.x + blockIdx.x, per = gridDim.y / kXcdsP;
+    const int k = lin / kXcdsP;
+    fblk = lin % kXcdsP + kXcdsP * (k % per);
+    tile = k / per;
+  } else {
+    const int per_xcd = (a.tiles + kXcdsP - 1) / kXcdsP;
+    tile = (blockIdx.x % kXcdsP) * per_xcd + blockIdx.x / kXcdsP;
+    fblk = blockIdx.y;
+  }
   if (tile >= a.tiles) return;
-  const int f0blk = blockIdx.y * 64;
+  const int f0blk = fblk * 64;
   const int n0 = (tile / a.tiles_y) * a.TN, y0 = (tile % a.tiles_y) * a.TH;
   const int PH = a.TH + 2, PW = a.W + 2;
 
@@ -95,26 +108,11 @@ __global__ __launch_bounds__(64 * WS * WK) void conv3x3_patch_kernel(const Patch
   const int lrow = lane & 31, lchunk = lane >> 5;
   const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(a.in, a.in_bytes);
   const __amdgpu_buffer_rsrc_t rs_wf = make_rsrc(a.wf, a.wf_bytes);
-  // The widest tile keeps no patch prefetch registers alive in the tap loop: single-slab layers only.
-  const int nslab = WS == 4 ? 1 : a.C * ES / 128;
+  // The widest tile keeps no patch prefetch registers alive in the tap loop: the host only picks it
+  // for single-slab layers, and its loop never reloads the patch.
+  constexpr bool kReload = WS != 4;
+  const int nslab = a.C * ES / 128;
   const int niter = nslab * 9;  // one iteration = one tap of one slab
-
-  // ---- weights: iteration `it`, sub-step k of this K group, filter half i is the kilobyte at
-  //      wbase + it*8192 + (k*2+i)*1024; NSET register sets hold iterations it .. it+NSET-1 ----
-  const int wbase = (blockIdx.y * niter * 8 + wk * KPG * 2) * 1024;
-  const unsigned wlane = lane * 16;
-  auto wload = [&](u32x4(&r)[NF], int it) {
-    const int so = it < niter ? wbase + it * 8192 : 0;  // past the end: re-read block 0 (never used)
-#pragma unroll
-    for (int q = 0; q < NF; ++q) r[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_wf, wlane, so + q * 1024, 0);
-  };
-  u32x4 wregs[NSET][NF];
-#pragma unroll
-  for (int q = 0; q < NSET; ++q) wload(wregs[q], q);
-
-  // epilogue scale/shift of this lane's output channels: requested now, used at the very end
-  EpiScale<OutT> ess;
-  ess.load(lane, f0blk, a.F, a.scale, a.shift);
 
   // ---- patch loader: 8 threads per pixel, NT/8 pixels per pass; the patch is walked as rows of
   //      2^rw_log pixels (>= W+2), so row and column of a pass are shifts and masks ----
@@ -162,7 +160,25 @@ __global__ __launch_bounds__(64 * WS * WK) void conv3x3_patch_kernel(const Patch
       *reinterpret_cast<u32x4*>(patch + (((px < PW) & (r < prows)) ? dst : dump)) = pregs[i];
     }
   };
-  pload(0);
+  pload(0);  // first in the queue: the patch gates the tap loop, the weights below only its first taps
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- weights: iteration `it`, sub-step k of this K group, filter half i is the kilobyte at
+  //      wbase + it*8192 + (k*2+i)*1024; NSET register sets hold iterations it .. it+NSET-1 ----
+  const int wbase = (fblk * niter * 8 + wk * KPG * 2) * 1024;
+  const unsigned wlane = lane * 16;
+  auto wload = [&](u32x4(&r)[NF], int it) {
+    const int so = it < niter ? wbase + it * 8192 : 0;  // past the end: re-read block 0 (never used)
+#pragma unroll
+    for (int q = 0; q < NF; ++q) r[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_wf, wlane, so + q * 1024, 0);
+  };
+  u32x4 wregs[NSET][NF];
+#pragma unroll
+  for (int q = 0; q < NSET; ++q) wload(wregs[q], q);
+
+  // epilogue scale/shift of this lane's output channels: requested now, used at the very end
+  EpiScale<OutT> ess;
+  ess.load(lane, f0blk, a.F, a.scale, a.shift);
 
   // ---- this lane's two pixel slots ----
   const int nslots = a.TN * a.TH * a.W;
@@ -203,29 +219,39 @@ __global__ __launch_bounds__(64 * WS * WK) void conv3x3_patch_kernel(const Patch
   auto filter_row = [&](int it0, auto s0) {
     constexpr int S0 = decltype(s0)::value;
     // next slab's patch is requested at the first tap of this slab and lands after its last tap
-    if (tr == 0 && slab + 1 < nslab) pload(slab + 1);
+    if (kReload && tr == 0 && slab + 1 < nslab) pload(slab + 1);
     const int ntr = tr == 2 ? 0 : tr + 1;
 #pragma unroll
     for (int ts = 0; ts < 3; ++ts) {
       constexpr int dummy = 0;
       (void)dummy;
       const int set = (S0 + ts) % NSET;
-      const bool new_patch = ts == 2 && tr == 2 && slab + 1 < nslab;  // the patch changes after this tap
+      const bool new_patch = kReload && ts == 2 && tr == 2 && slab + 1 < nslab;  // the patch changes after this tap
       const int tapoff = (tr * PW + ts) * kPitch;
       const int ntapoff = ts == 2 ? (ntr * PW) * kPitch : tapoff + kPitch;
+      const int it_next = it0 + ts + NSET;
+      const int wso = it_next < niter ? wbase + it_next * 8192 : 0;  // past the end: re-read block 0 (never used)
+      // Scheduling fences pin the software pipeline: the pixel operands of step k+1 are requested
+      // before the MFMAs of step k, and a weight register is refilled (NSET taps ahead) right
+      // after its last use.  Left alone, the scheduler sinks both kinds of load to just before
+      // their consumers and the loop runs at memory latency.
 #pragma unroll
       for (int k = 0; k < KPG; ++k) {
         u32x4 np[2];
         if (k + 1 < KPG) ldp(np, tapoff, k + 1);
         else if (!new_patch) ldp(np, ntapoff, 0);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
           for (int j = 0; j < 2; ++j) Mma<T>::run(wregs[set][k * 2 + i], fp[j], acc[i][j]);
 #pragma unroll
+        for (int i = 0; i < 2; ++i)
+          wregs[set][k * 2 + i] = __builtin_amdgcn_raw_buffer_load_b128(rs_wf, wlane, wso + (k * 2 + i) * 1024, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
         for (int j = 0; j < 2; ++j) fp[j] = np[j];
       }
-      wload(wregs[set], it0 + ts + NSET);  // this set is consumed: refill it NSET taps ahead
       if (new_patch) {
         __syncthreads();  // every wave is done with the old patch
         pstore();
@@ -341,6 +367,7 @@ void launch_conv3x3_patch(const IgemmArgs& g, int in_dt, int out_dt, hipStream_t
   a.tiles = ((a.N + a.TN - 1) / a.TN) * a.tiles_y;
   a.in_bytes = g.in_bytes;
   a.wf_bytes = (unsigned)((size_t)((a.F + 63) / 64) * 64 * 9 * a.C * dtype_size(in_dt));
+  a.xcd_by_filter = ((a.F + 63) / 64) % kXcdsP == 0 && a.wf_bytes > (2u << 20);
   a.inv_ph = 1.0f / (a.TH + 2);
   a.inv_thw = 1.0f / (a.TH * a.W);
   a.inv_w = 1.0f / a.W;

@@ -82,6 +82,14 @@ struct IgemmArgs {
                      // contiguous elements = 4 packed pixel pairs at a pixel pitch of 8)
   unsigned in_bytes, wt_bytes;  // size of one batch slice of in / wt; 0 = derived from the geometry
   const void* wt_frag;  // the same 3x3 filters in fragment-major order (launch_weight_frag3x3), or null
+  // Auxiliary filters fused into the same launch (the 1x1 stride-2 shortcut convolution of a
+  // down-sampling block rides on the 3x3 stride-2 one: same input pixels, centre tap only).
+  // Filters [aux_f0, F) are auxiliary: their rows of `wt` are zero outside tap `aux_tap`
+  // (= r*S + s), only that tap's K range is walked for them, and their results go to `aux_out`
+  // (row pitch aux_ldo, channel f - aux_f0) with aux_relu and no residual.  scale/shift cover
+  // all F filters.  aux_f0 = 0: none; otherwise a multiple of 128.  Fast kernel only.
+  int aux_f0, aux_tap, aux_relu, aux_ldo;
+  void* aux_out;
 };
 // in_dt: element type of in/wt (kF32 | kF16); out_dt: element type of out/residual.
 // Dispatches to the fast kernel (igemm_fast.hip) when C is a multiple of one K step and the

@@ -64,7 +64,7 @@ struct PatchCfg {
   static constexpr int NW = WS * WK, NT = 64 * NW;
   static constexpr int cover = WS == 4 ? 384 : WS == 2 ? 256 : 192;  // padded patch pixels the loader can walk
   static constexpr int passes = cover / (NT / 8);  // loader passes per thread: NT/8 pixels each
-  static constexpr int nset = WK == 1 ? 2 : 3;     // weight register sets (taps in flight)
+  static constexpr int nset = WK == 4 ? 9 : 3;  // weight register sets = taps in flight; divides 9
   static constexpr int cap = PatchCap<WS>::pix;
   static constexpr int patch_bytes = cap * kPitch;
   static constexpr int load_bytes = patch_bytes + NT * 16;  // + one dump slot per thread
@@ -76,6 +76,7 @@ template <typename T, typename OutT, int WS, int WK>
 __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv3x3_patch_kernel(const PatchArgs a) {
   typedef PatchCfg<WS, WK> Cfg;
   constexpr int NT = Cfg::NT, kPasses = Cfg::passes, NSET = Cfg::nset;
+  constexpr int kDepth = WK == 1 ? 3 : 4;  // pixel-operand ring: LDS reads run kDepth-1 steps ahead of their MFMAs
   constexpr int ES = sizeof(T);
   constexpr int KPG = 4 / WK;     // 32-byte K sub-steps per K group and tap
   constexpr int NF = 2 * KPG;     // weight fragments (kilobytes) per wave and tap
@@ -204,70 +205,66 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  auto ldp = [&](u32x4(&f)[2], int tapoff, int k) {
+  // ---- tap loop.  One trip = one slab = 9 taps x KPG K sub-steps ("steps"), fully unrolled, so
+  // that tap offsets, weight register sets (NSET divides 9) and the ring slot of the pixel
+  // operands are all static.  Per step: four MFMAs; the pixel operands come from LDS kDepth-1
+  // steps ahead, a weight register is refilled (NSET taps ahead) right after its last use.
+  // Scheduling fences pin that software pipeline: left alone, the scheduler sinks both kinds of
+  // load to just before their consumers and the loop runs at memory latency.
+  constexpr int kSteps = 9 * KPG;
+  int rowbase[3][2];  // slot base + filter row r
 #pragma unroll
-    for (int j = 0; j < 2; ++j) f[j] = *reinterpret_cast<const u32x4*>(patch + sbase[j] + tapoff + k * 32);
+  for (int r = 0; r < 3; ++r)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) rowbase[r][j] = sbase[j] + r * PW * kPitch;
+  u32x4 ring[kDepth][2];
+  auto ldp = [&](auto step_c) {
+    constexpr int st = decltype(step_c)::value;
+    constexpr int t = st / KPG, k = st % KPG;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      ring[st % kDepth][j] = *reinterpret_cast<const u32x4*>(patch + rowbase[t / 3][j] + (t % 3) * kPitch + k * 32);
+  };
+  auto prime = [&](auto self, auto d_c) -> void {  // the first kDepth-1 steps of a fresh patch
+    constexpr int d = decltype(d_c)::value;
+    if constexpr (d < kDepth - 1) {
+      ldp(d_c);
+      self(self, std::integral_constant<int, d + 1>());
+    }
   };
 
   pstore();
   __syncthreads();
+  prime(prime, std::integral_constant<int, 0>());
 
-  u32x4 fp[2];
-  ldp(fp, 0, 0);
-  int tr = 0, slab = 0;
-  // One filter row = three taps; `s0` is the register set of its first tap (sets rotate per tap).
-  auto filter_row = [&](int it0, auto s0) {
-    constexpr int S0 = decltype(s0)::value;
-    // next slab's patch is requested at the first tap of this slab and lands after its last tap
-    if (kReload && tr == 0 && slab + 1 < nslab) pload(slab + 1);
-    const int ntr = tr == 2 ? 0 : tr + 1;
-#pragma unroll
-    for (int ts = 0; ts < 3; ++ts) {
-      constexpr int dummy = 0;
-      (void)dummy;
-      const int set = (S0 + ts) % NSET;
-      const bool new_patch = kReload && ts == 2 && tr == 2 && slab + 1 < nslab;  // the patch changes after this tap
-      const int tapoff = (tr * PW + ts) * kPitch;
-      const int ntapoff = ts == 2 ? (ntr * PW) * kPitch : tapoff + kPitch;
-      const int it_next = it0 + ts + NSET;
-      const int wso = it_next < niter ? wbase + it_next * 8192 : 0;  // past the end: re-read block 0 (never used)
-      // Scheduling fences pin the software pipeline: the pixel operands of step k+1 are requested
-      // before the MFMAs of step k, and a weight register is refilled (NSET taps ahead) right
-      // after its last use.  Left alone, the scheduler sinks both kinds of load to just before
-      // their consumers and the loop runs at memory latency.
-#pragma unroll
-      for (int k = 0; k < KPG; ++k) {
-        u32x4 np[2];
-        if (k + 1 < KPG) ldp(np, tapoff, k + 1);
-        else if (!new_patch) ldp(np, ntapoff, 0);
+  for (int slab = 0; slab < nslab; ++slab) {
+    const bool more = kReload && slab + 1 < nslab;
+    if (kReload && more) pload(slab + 1);  // lands after the last tap of this slab
+    auto steps = [&](auto self, auto step_c) -> void {
+      constexpr int st = decltype(step_c)::value;
+      if constexpr (st < kSteps) {
+        constexpr int t = st / KPG, k = st % KPG, set = t % NSET;
+        if constexpr (st + kDepth - 1 < kSteps) ldp(std::integral_constant<int, st + kDepth - 1>());
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
-          for (int j = 0; j < 2; ++j) Mma<T>::run(wregs[set][k * 2 + i], fp[j], acc[i][j]);
+          for (int j = 0; j < 2; ++j) Mma<T>::run(wregs[set][k * 2 + i], ring[st % kDepth][j], acc[i][j]);
+        const int it_next = slab * 9 + t + NSET;
+        const int wso = it_next < niter ? wbase + it_next * 8192 : 0;  // past the end: re-read block 0 (never used)
 #pragma unroll
         for (int i = 0; i < 2; ++i)
           wregs[set][k * 2 + i] = __builtin_amdgcn_raw_buffer_load_b128(rs_wf, wlane, wso + (k * 2 + i) * 1024, 0);
         __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int j = 0; j < 2; ++j) fp[j] = np[j];
+        self(self, std::integral_constant<int, st + 1>());
       }
-      if (new_patch) {
-        __syncthreads();  // every wave is done with the old patch
-        pstore();
-        __syncthreads();
-        ldp(fp, 0, 0);
-      }
-    }
-    tr = ntr;
-    if (tr == 0) ++slab;
-  };
-  if (NSET == 3) {
-    for (int it0 = 0; it0 < niter; it0 += 3) filter_row(it0, std::integral_constant<int, 0>());
-  } else {  // two sets: the rotation repeats every two rows
-    for (int it0 = 0; it0 < niter; it0 += 6) {
-      filter_row(it0, std::integral_constant<int, 0>());
-      if (it0 + 3 < niter) filter_row(it0 + 3, std::integral_constant<int, 1>());
+    };
+    steps(steps, std::integral_constant<int, 0>());
+    if (kReload && more) {
+      __syncthreads();  // every wave is done with the old patch
+      pstore();
+      __syncthreads();
+      prime(prime, std::integral_constant<int, 0>());
     }
   }
   __syncthreads();  // every wave is done with the patch: LDS becomes the output tiles
@@ -335,7 +332,7 @@ bool conv3x3_patch_applicable(const IgemmArgs& a, int in_dt) {
   static const bool off = getenv("NNCV_HIP_NO_PATCH") != nullptr;
   const int slab = in_dt == kF16 ? 64 : 32;
   int ws, tn, th, lg;
-  return !off && a.wt_frag && a.R == 3 && a.S == 3 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 1 && a.pad_w == 1 &&
+  return !off && a.aux_f0 == 0 && a.wt_frag && a.R == 3 && a.S == 3 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 1 && a.pad_w == 1 &&
          a.batch == 1 && a.pix_stride == 0 && a.C % slab == 0 && a.F % 8 == 0 && a.ldo == a.F &&
          (long long)a.N * a.H * a.W * a.F < (1ll << 31) && (long long)a.N * a.H * a.W < (1 << 24) && a.in_bytes < kOOBp &&
          (long long)((a.F + 63) / 64) * 64 * 9 * a.C * (long long)dtype_size(in_dt) < (1ll << 31) &&

@@ -282,6 +282,7 @@ void launch_igemm(const IgemmArgs& a_in, int in_dt, int out_dt, hipStream_t s) {
     NNCV_HIP_CHECK(hipGetLastError());
     return;
   }
+  NNCV_REQUIRE(a.aux_f0 == 0, "igemm: auxiliary filters need the fast kernel");
   if (in_dt == kF16 && out_dt == kF16) launch_typed<half_t, half_t>(a, s);
   else if (in_dt == kF16 && out_dt == kF32) launch_typed<half_t, float>(a, s);
   else if (in_dt == kF32 && out_dt == kF32) launch_typed<float, float>(a, s);

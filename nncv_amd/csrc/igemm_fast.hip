@@ -59,7 +59,12 @@ __global__ __launch_bounds__(64 * WP * WF * WK) void igemm_fast_kernel(const Ige
   const int wpos = wave % (WP * WF), wk = wave / (WP * WF);
   const int wp = wpos % WP, wf = wpos / WP;
   const int P = a.N * a.OH * a.OW;
-  const int nk = (a.R * a.S * a.C) / BKE;  // K steps in total (exact: C % BKE == 0)
+  const int nk_row = (a.R * a.S * a.C) / BKE;  // K steps of a whole filter row (exact: C % BKE == 0)
+  // auxiliary filter blocks walk one tap only
+  const bool aux = a.aux_f0 > 0 && by * BF >= a.aux_f0;
+  const int spt = a.C / BKE;  // K steps per tap
+  const int k_begin = aux ? a.aux_tap * spt : 0;
+  const int nk = aux ? k_begin + spt : nk_row;  // end of the K walk
   const int pix = a.pix_stride ? a.pix_stride : a.C;
 
   const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(static_cast<const T*>(a.in) + (long long)bz * a.in_bs, a.in_bytes);
@@ -87,7 +92,7 @@ __global__ __launch_bounds__(64 * WP * WF * WK) void igemm_fast_kernel(const Ige
 #pragma unroll
   for (int g = 0; g < WF; ++g) {
     const int f = by * BF + r0 + 64 * g;
-    wbase[g] = f < a.F ? (f * (nk * BKE) + ck * CE) * ES : -1;
+    wbase[g] = f < a.F ? (f * (nk_row * BKE) + ck * CE) * ES : -1;
   }
 
   // epilogue scale/shift of this lane's output channels: requested now, used at the very end
@@ -95,7 +100,7 @@ __global__ __launch_bounds__(64 * WP * WF * WK) void igemm_fast_kernel(const Ige
   ess.load(lane, by * BF + wf * 64, a.F, a.scale, a.shift);
 
   // scalar K walk
-  int kstep = 0, kr = 0, ks = 0, kc = 0;
+  int kstep = k_begin, kr = aux ? a.aux_tap / a.S : 0, ks = aux ? a.aux_tap % a.S : 0, kc = 0;
 
   u32x4 regs[2][LPT];
   auto issue = [&](u32x4(&r)[LPT]) {
@@ -163,7 +168,7 @@ __global__ __launch_bounds__(64 * WP * WF * WK) void igemm_fast_kernel(const Ige
     }
   };
 
-  const int nst = (nk + KS - 1) / KS;
+  const int nst = (nk - k_begin + KS - 1) / KS;
   issue(regs[0]);
   if (nst > 1) issue(regs[1]);
   store(regs[0], 0);
@@ -204,11 +209,14 @@ __global__ __launch_bounds__(64 * WP * WF * WK) void igemm_fast_kernel(const Ige
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int gp = bx * BP + wp * 64 + j * 32 + lrow;
-    rowoff[j] = gp < P ? gp * a.ldo : -1;
+    rowoff[j] = gp < P ? gp * (aux ? a.aux_ldo : a.ldo) : -1;
   }
-  OutT* out = static_cast<OutT*>(a.out) + (long long)bz * a.out_bs;
-  const OutT* res = a.residual ? static_cast<const OutT*>(a.residual) + (long long)bz * a.out_bs : nullptr;
-  tile_reduce_store<OutT, WK>(acc, smem + wpos * kTileBytes, wk, lane, rowoff, by * BF + wf * 64, a.F, ess, res, out, a.relu);
+  OutT* out = aux ? static_cast<OutT*>(a.aux_out) : static_cast<OutT*>(a.out) + (long long)bz * a.out_bs;
+  const OutT* res = (a.residual && !aux) ? static_cast<const OutT*>(a.residual) + (long long)bz * a.out_bs : nullptr;
+  const int fo = aux ? a.aux_f0 : 0;                     // first filter of this output tensor
+  const int fend = (aux || a.aux_f0 == 0) ? a.F : a.aux_f0;  // one past its last filter
+  tile_reduce_store<OutT, WK>(acc, smem + wpos * kTileBytes, wk, lane, rowoff, by * BF + wf * 64 - fo, fend - fo, ess, res, out,
+                              aux ? a.aux_relu : a.relu);
 }
 
 namespace {
@@ -275,7 +283,9 @@ bool igemm_fast_applicable(const IgemmArgs& a, int in_dt, int out_dt) {
   static const bool off = getenv("NNCV_HIP_IGEMM_GENERIC") != nullptr;
   const long long P = (long long)a.N * a.OH * a.OW;
   return !off && a.C % bke == 0 && a.F % fvec == 0 && a.ldo % fvec == 0 && a.in_bytes > 0 && a.in_bytes < kOOB &&
-         a.wt_bytes > 0 && a.wt_bytes < kOOB && P < (1 << 24) && P * a.ldo < (1ll << 31);
+         a.wt_bytes > 0 && a.wt_bytes < kOOB && P < (1 << 24) && P * a.ldo < (1ll << 31) &&
+         (a.aux_f0 == 0 || (a.aux_f0 % 128 == 0 && a.batch == 1 && a.aux_out && a.aux_ldo % fvec == 0 &&
+                            P * a.aux_ldo < (1ll << 31) && a.aux_tap >= 0 && a.aux_tap < a.R * a.S));
 }
 
 void launch_igemm_fast(const IgemmArgs& a, int in_dt, int out_dt, hipStream_t s) {

@@ -108,6 +108,48 @@ void ConvLayer::forward(const void* in, int N, int H, int W, const void* residua
   launch_igemm(a, d_.dt, d_.dt, s);
 }
 
+bool ConvLayer::fuse_shortcut(const ConvLayer& ds, hipStream_t s) {
+  const Desc& q = ds.d_;
+  const size_t es = dtype_size(d_.dt);
+  const int ce = d_.dt == kF16 ? 8 : 4;
+  if (d_.stem || algo_ != kAlgoIgemm || ds.algo_ != kAlgoIgemm || q.dt != d_.dt || q.C != d_.C || q.stride != d_.stride ||
+      d_.R != 3 || d_.S != 3 || d_.pad != 1 || q.R != 1 || q.S != 1 || q.pad != 0 || d_.F % 128 != 0 || q.F % 8 != 0 ||
+      d_.C % ce != 0 || !scale_.get() || !ds.scale_.get())
+    return false;
+  const size_t row = (size_t)9 * d_.C * es;
+  wt_cat_.reset((size_t)(d_.F + q.F) * row);
+  NNCV_HIP_CHECK(hipMemsetAsync(wt_cat_.get(), 0, wt_cat_.bytes(), s));
+  NNCV_HIP_CHECK(hipMemcpyAsync(wt_cat_.get(), wt_.get(), (size_t)d_.F * row, hipMemcpyDeviceToDevice, s));
+  // the shortcut's [F][C] rows become the centre tap (r = s = 1) of otherwise zero 3x3 filters
+  NNCV_HIP_CHECK(hipMemcpy2DAsync(wt_cat_.as<char>() + (size_t)d_.F * row + (size_t)4 * d_.C * es, row, ds.wt_.get(),
+                                  (size_t)d_.C * es, (size_t)d_.C * es, q.F, hipMemcpyDeviceToDevice, s));
+  scale_cat_.reset((size_t)(d_.F + q.F) * 4);
+  shift_cat_.reset((size_t)(d_.F + q.F) * 4);
+  NNCV_HIP_CHECK(hipMemcpyAsync(scale_cat_.get(), scale_.get(), (size_t)d_.F * 4, hipMemcpyDeviceToDevice, s));
+  NNCV_HIP_CHECK(hipMemcpyAsync(shift_cat_.get(), shift_.get(), (size_t)d_.F * 4, hipMemcpyDeviceToDevice, s));
+  NNCV_HIP_CHECK(hipMemcpyAsync(scale_cat_.as<float>() + d_.F, ds.scale_.get(), (size_t)q.F * 4, hipMemcpyDeviceToDevice, s));
+  NNCV_HIP_CHECK(hipMemcpyAsync(shift_cat_.as<float>() + d_.F, ds.shift_.get(), (size_t)q.F * 4, hipMemcpyDeviceToDevice, s));
+  aux_F_ = q.F;
+  aux_relu_ = q.relu;
+  aux_flops_per_pixel_ = 2.0 * q.F * q.C;
+  return true;
+}
+
+void ConvLayer::forward_with_shortcut(const void* in, int N, int H, int W, void* out, void* shortcut_out, hipStream_t s) const {
+  NNCV_REQUIRE(aux_F_ > 0, "conv: no fused shortcut");
+  const int OH = out_h(H), OW = out_w(W);
+  NNCV_REQUIRE(N > 0 && OH > 0 && OW > 0, "conv: empty tensor");
+  IgemmArgs a{};
+  a.in = in; a.wt = wt_cat_.get(); a.out = out;
+  a.scale = scale_cat_.as<float>(); a.shift = shift_cat_.as<float>();
+  a.N = N; a.H = H; a.W = W; a.C = d_.C; a.F = d_.F + aux_F_; a.R = 3; a.S = 3; a.OH = OH; a.OW = OW;
+  a.stride_h = a.stride_w = d_.stride; a.pad_h = a.pad_w = 1;
+  a.relu = d_.relu; a.ldo = d_.F; a.batch = 1;
+  a.aux_f0 = d_.F; a.aux_tap = 4; a.aux_relu = aux_relu_; a.aux_ldo = aux_F_; a.aux_out = shortcut_out;
+  a.alg_flops = (2.0 * d_.F * 9.0 * d_.C + aux_flops_per_pixel_) * N * OH * OW;
+  launch_igemm(a, d_.dt, d_.dt, s);
+}
+
 void ConvLayer::forward_strided(const void* in, Strides4 in_st, int N, int H, int W, const void* residual, void* out,
                                 Strides4 out_st, bool accumulate, void* ws, hipStream_t s) const {
   NNCV_REQUIRE(!d_.stem, "conv: the stem has no strided form");
@@ -182,7 +224,11 @@ ResNet18::ResNet18(const void* params, long long n_elems, int dt, int algo3x3, h
       Block b;
       b.c1 = make(cin, F, 3, stride, 1, true, false);
       b.c2 = make(F, F, 3, 1, 1, true, false);  // ReLU after the residual add
-      if (stride != 1 || cin != F) b.ds = make(cin, F, 1, stride, 0, false, false);
+      if (stride != 1 || cin != F) {
+        b.ds = make(cin, F, 1, stride, 0, false, false);
+        static const bool no_fuse = getenv("NNCV_HIP_NO_SHORTCUT_FUSION") != nullptr;
+        if (!no_fuse) b.c1->fuse_shortcut(*b.ds, s);
+      }
       blocks_.push_back(std::move(b));
       cin = F;
     }
@@ -254,11 +300,16 @@ void ResNet18::forward(const void* src, int N, int H, int W, void* logits, void*
     char* idn = act[(cur + 2) & 3];
     char* y2 = act[(cur + 3) & 3];
     const int oh = b.c1->out_h(h), ow = b.c1->out_w(w);
-    b.c1->forward(x, N, h, w, nullptr, y1, cws, s);
     const void* shortcut = x;
-    if (b.ds) {
-      b.ds->forward(x, N, h, w, nullptr, idn, cws, s);
+    if (b.ds && b.c1->has_shortcut()) {
+      b.c1->forward_with_shortcut(x, N, h, w, y1, idn, s);
       shortcut = idn;
+    } else {
+      b.c1->forward(x, N, h, w, nullptr, y1, cws, s);
+      if (b.ds) {
+        b.ds->forward(x, N, h, w, nullptr, idn, cws, s);
+        shortcut = idn;
+      }
     }
     b.c2->forward(y1, N, oh, ow, shortcut, y2, cws, s);
     cur = (cur + 3) & 3;

@@ -41,11 +41,22 @@ class ConvLayer {
   // generic-layout form used by the operator-level ABI: strides for in / out (residual shares out's)
   void forward_strided(const void* in, Strides4 in_st, int N, int H, int W, const void* residual, void* out, Strides4 out_st,
                        bool accumulate, void* ws, hipStream_t s) const;
+  // Fuses the 1x1 shortcut convolution `ds` of a down-sampling block (same input, same stride, no
+  // padding) into this 3x3 pad-1 convolution: one launch then produces both tensors.  Returns
+  // false (and changes nothing) when the pair does not qualify.
+  bool fuse_shortcut(const ConvLayer& ds, hipStream_t s);
+  bool has_shortcut() const { return aux_F_ > 0; }
+  // forward() of this layer into `out` and of the fused shortcut into `shortcut_out`
+  void forward_with_shortcut(const void* in, int N, int H, int W, void* out, void* shortcut_out, hipStream_t s) const;
 
  private:
   Desc d_;
   int algo_;
   DeviceBuffer wt_, wfrag_, U_, scale_, shift_;
+  DeviceBuffer wt_cat_, scale_cat_, shift_cat_;  // this layer's filters followed by the fused shortcut's
+  int aux_F_ = 0;
+  bool aux_relu_ = false;
+  double aux_flops_per_pixel_ = 0.0;
 };
 
 class ResNet18 {

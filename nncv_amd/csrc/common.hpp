@@ -141,8 +141,14 @@ void launch_weight_frsc(const void* w, int w_dt, void* dst, int dst_dt, int F, i
                         hipStream_t s);
 // 3x3 weights FCHW -> fragment-major order of conv3x3_patch.hip, F padded to a multiple of 64
 void launch_weight_frag3x3(const void* w, int w_dt, void* dst, int dst_dt, int F, int C, hipStream_t s);
-// stem weights [64,3,7,7] -> [64][7][4][8] over (pixel-pair, channel4)
-void launch_stem_weight(const void* w, int w_dt, void* dst, int dst_dt, int F, hipStream_t s);
+// stem weights [64,3,7,7] -> [64][7][4][8] over (pixel-pair, channel4); pair sp / pixel p holds
+// filter column 2*sp + p - col_shift (zero outside 0..6)
+void launch_stem_weight(const void* w, int w_dt, void* dst, int dst_dt, int F, int col_shift, hipStream_t s);
+// fused stem: conv7x7 s2 p3 + scale/shift + ReLU + maxpool 3x3 s2 p1, NCHW fp16 in, NHWC out
+// (stem_pool.hip); wt in the col_shift = 1 layout above
+bool stem_pool_applicable(int dt, int N, int H, int W, int F);
+void launch_stem_pool(const void* in, const void* wt, const float* scale, const float* shift, void* out, int N, int H, int W,
+                      hipStream_t s);
 // BN fold: scale = gamma / sqrt(var + eps), shift = beta - mean*scale (fp32 out)
 void launch_bn_fold(const void* gamma, const void* beta, const void* mean, const void* var, int dt, float* scale,
                     float* shift, int C, hipStream_t s);

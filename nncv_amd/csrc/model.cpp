@@ -34,7 +34,9 @@ ConvLayer::ConvLayer(const Desc& d, const void* w, const void* gamma, const void
     NNCV_REQUIRE(d.C == 3 && d.R == 7 && d.S == 7 && d.stride == 2 && d.pad == 3, "stem: must be 7x7 s2 p3 over 3 channels");
     NNCV_REQUIRE(d.F % 4 == 0, "stem: F must be a multiple of 4");
     wt_.reset((size_t)d.F * 224 * es);
-    launch_stem_weight(w, d.dt, wt_.get(), d.dt, d.F, s);
+    launch_stem_weight(w, d.dt, wt_.get(), d.dt, d.F, 0, s);
+    wt_shift_.reset((size_t)d.F * 224 * es);  // pairs start one column further left (fused stem)
+    launch_stem_weight(w, d.dt, wt_shift_.get(), d.dt, d.F, 1, s);
   } else if (algo_ == kAlgoWinograd) {
     U_.reset((size_t)36 * d.F * d.C * es);
     launch_wino43_filter(w, d.dt, U_.get(), d.dt, d.F, d.C, s);
@@ -106,6 +108,12 @@ void ConvLayer::forward(const void* in, int N, int H, int W, const void* residua
   a.stride_h = a.stride_w = d_.stride; a.pad_h = a.pad_w = d_.pad;
   a.relu = d_.relu; a.ldo = d_.F; a.batch = 1;
   launch_igemm(a, d_.dt, d_.dt, s);
+}
+
+bool ConvLayer::forward_stem_pool(const void* in, int N, int H, int W, void* pooled_out, hipStream_t s) const {
+  if (!d_.stem || !d_.relu || !stem_pool_applicable(d_.dt, N, H, W, d_.F)) return false;
+  launch_stem_pool(in, wt_shift_.get(), scale_.as<float>(), shift_.as<float>(), pooled_out, N, H, W, s);
+  return true;
 }
 
 bool ConvLayer::fuse_shortcut(const ConvLayer& ds, hipStream_t s) {
@@ -288,8 +296,10 @@ void ResNet18::forward(const void* src, int N, int H, int W, void* logits, void*
   char* cws = base;
 
   // stem: conv7x7 s2 + BN + ReLU (Res18.mlir:118-142), then maxpool 3x3 s2 (:144-151)
-  stem_->forward(src, N, H, W, nullptr, stem_out, cws, s);
-  launch_maxpool3x3s2_nhwc(stem_out, act[0], dt_, N, p.h1, p.w1, 64, s);
+  if (!stem_->forward_stem_pool(src, N, H, W, act[0], s)) {
+    stem_->forward(src, N, H, W, nullptr, stem_out, cws, s);
+    launch_maxpool3x3s2_nhwc(stem_out, act[0], dt_, N, p.h1, p.w1, 64, s);
+  }
   int cur = 0, h = p.h2, w = p.w2, nblk = 0, ch = 64;
   const size_t es = dtype_size(dt_);
   if (tap_stage == 0) NNCV_HIP_CHECK(hipMemcpyAsync(tap, act[0], (size_t)N * h * w * 64 * es, hipMemcpyDeviceToDevice, s));

@@ -44,6 +44,9 @@ class ConvLayer {
   // Fuses the 1x1 shortcut convolution `ds` of a down-sampling block (same input, same stride, no
   // padding) into this 3x3 pad-1 convolution: one launch then produces both tensors.  Returns
   // false (and changes nothing) when the pair does not qualify.
+  // stem only: conv + BN + ReLU + the 3x3 stride-2 max-pool in one launch, NCHW in, pooled NHWC
+  // out.  Returns false (nothing launched) when the fused kernel does not cover the case.
+  bool forward_stem_pool(const void* in, int N, int H, int W, void* pooled_out, hipStream_t s) const;
   bool fuse_shortcut(const ConvLayer& ds, hipStream_t s);
   bool has_shortcut() const { return aux_F_ > 0; }
   // forward() of this layer into `out` and of the fused shortcut into `shortcut_out`
@@ -52,7 +55,7 @@ class ConvLayer {
  private:
   Desc d_;
   int algo_;
-  DeviceBuffer wt_, wfrag_, U_, scale_, shift_;
+  DeviceBuffer wt_, wfrag_, U_, scale_, shift_, wt_shift_;
   DeviceBuffer wt_cat_, scale_cat_, shift_cat_;  // this layer's filters followed by the fused shortcut's
   int aux_F_ = 0;
   bool aux_relu_ = false;

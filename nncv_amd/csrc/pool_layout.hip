@@ -262,17 +262,18 @@ void launch_weight_frag3x3(const void* w, int w_dt, void* dst, int dst_dt, int F
 }
 
 template <typename Ts, typename Td>
-__global__ void stem_weight_kernel(const Ts* __restrict__ w, Td* __restrict__ dst, int F) {
+__global__ void stem_weight_kernel(const Ts* __restrict__ w, Td* __restrict__ dst, int F, int col_shift) {
   const int idx = blockIdx.x * blockDim.x + threadIdx.x;  // over [F][7][4][8]
   if (idx >= F * 7 * 4 * 8) return;
   const int e = idx & 7, sp = (idx >> 3) & 3, r = (idx >> 5) % 7, f = idx / 224;
-  const int p = e >> 2, c = e & 3, s = 2 * sp + p;
-  dst[idx] = (c < 3 && s < 7) ? (Td)(float)w[((f * 3 + c) * 7 + r) * 7 + s] : (Td)0.0f;
+  const int p = e >> 2, c = e & 3, s = 2 * sp + p - col_shift;
+  dst[idx] = (c < 3 && s >= 0 && s < 7) ? (Td)(float)w[((f * 3 + c) * 7 + r) * 7 + s] : (Td)0.0f;
 }
 
-void launch_stem_weight(const void* w, int w_dt, void* dst, int dst_dt, int F, hipStream_t s) {
+void launch_stem_weight(const void* w, int w_dt, void* dst, int dst_dt, int F, int col_shift, hipStream_t s) {
   const unsigned grid = (unsigned)((F * 224 + 255) / 256);
-#define LAUNCH(TS, TD) hipLaunchKernelGGL((stem_weight_kernel<TS, TD>), dim3(grid), dim3(256), 0, s, (const TS*)w, (TD*)dst, F)
+#define LAUNCH(TS, TD) \
+  hipLaunchKernelGGL((stem_weight_kernel<TS, TD>), dim3(grid), dim3(256), 0, s, (const TS*)w, (TD*)dst, F, col_shift)
   if (w_dt == kF32 && dst_dt == kF32) LAUNCH(float, float);
   else if (w_dt == kF16 && dst_dt == kF16) LAUNCH(half_t, half_t);
   else if (w_dt == kF32 && dst_dt == kF16) LAUNCH(float, half_t);

@@ -184,8 +184,11 @@ def resnet18_forward(x, params, tap_layer=-1):
     tp = None
     if tap_layer >= 0:
         ch = [64, 64, 128, 256, 512][tap_layer]
-        h = H // 4 if tap_layer == 0 else H // (4 * 2 ** (tap_layer - 1))
-        tap = np.empty((N, ch, h, h * W // H), np.float32)
+        down = lambda v: (v - 1) // 2 + 1  # every stride-2 stage (7x7 p3, 3x3 p1): ceil(v / 2)
+        h, w = down(down(H)), down(down(W))
+        for _ in range(max(0, tap_layer - 1)):
+            h, w = down(h), down(w)
+        tap = np.empty((N, ch, h, w), np.float32)
         tp = tap.ctypes.data_as(ctypes.c_void_p)
     rc = lib().orc_resnet18_forward(x, N, H, W, params, y, tap_layer, tp)
     assert rc == 0

@@ -115,8 +115,10 @@ class Model:
             abi.check(abi.lib().nncv_hip_resnet18_forward(self.h, x_dev.data_ptr(), N, H, W, logits.data_ptr(), None))
             return logits
         ch = [64, 64, 128, 256, 512][tap_stage]
-        h = H // 4 if tap_stage == 0 else H // (4 * 2 ** (tap_stage - 1))
-        w = W // 4 if tap_stage == 0 else W // (4 * 2 ** (tap_stage - 1))
+        down = lambda v: (v - 1) // 2 + 1  # every stride-2 stage halves, rounding up
+        h, w = down(down(H)), down(down(W))
+        for _ in range(max(0, tap_stage - 1)):
+            h, w = down(h), down(w)
         tap = empty((N, h, w, ch), self.dt)
         abi.check(abi.lib().nncv_hip_resnet18_forward_tap(self.h, x_dev.data_ptr(), N, H, W, logits.data_ptr(),
                                                           tap_stage, tap.data_ptr(), None))

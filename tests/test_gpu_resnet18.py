@@ -104,3 +104,45 @@ def test_graph_replay_matches_eager_every_time(blob):
         ref = host(Model(hb, abi.F16)(dev(x, abi.F16)))  # a fresh handle never replays: eager result
         assert np.array_equal(got, ref), rep
         assert other.shape == (256, 256)
+
+
+def _stage0(m, x16, N, H, W):
+    """Pooled stem activation (NHWC) and logits through the tap entry point, any image size."""
+    oh, ow = (H - 1) // 2 + 1, (W - 1) // 2 + 1
+    ph, pw = (oh - 1) // 2 + 1, (ow - 1) // 2 + 1
+    xd = dev(x16, abi.F16)
+    logits = torch.empty((N, 1000), dtype=torch.float32, device="cuda")
+    tap = torch.empty((N, ph, pw, 64), dtype=torch.float16, device="cuda")
+    abi.check(abi.lib().nncv_hip_resnet18_forward_tap(m.h, xd.data_ptr(), N, H, W, logits.data_ptr(), 0, tap.data_ptr(), None))
+    return host(logits), nchw(host(tap))
+
+
+@pytest.mark.parametrize("shape", [(2, 64, 64), (1, 96, 160), (1, 70, 90), (3, 224, 224), (1, 34, 32)])
+def test_fp16_fused_stem_and_pool(blob, shape):
+    """conv7x7 + BN + ReLU + max-pool in one launch: pooled activation and logits vs the oracle for
+    square, wide, odd-sized and minimum images (partial tiles on every edge)."""
+    N, H, W = shape
+    hb = synth.round_fp16(blob)
+    x = synth.round_fp16(synth.uniform(4200 + H, (N, 3, H, W), -1.0, 1.0))
+    want_logits, want_tap = oracle.resnet18_forward(x, hb, tap_layer=0)
+    m = Model(hb, abi.F16)
+    logits, tap = _stage0(m, x, N, H, W)
+    assert tap.shape == want_tap.shape
+    e_tap, e_log = rel_l2(tap, want_tap), rel_l2(logits, want_logits)
+    print("shape", shape, "stage0 rel_l2", e_tap, "logits rel_l2", e_log, flush=True)
+    assert e_tap < 2e-3  # one fp16 rounding of an O(1) activation
+    assert e_log < FP16_REL_L2
+
+
+def test_fp16_fused_stem_propagates_nan(blob):
+    """arith.maximumf keeps NaN: a NaN pixel poisons exactly the pooled outputs whose windows see it."""
+    hb = synth.round_fp16(blob)
+    x = synth.round_fp16(synth.uniform(4300, (1, 3, 64, 64), -1.0, 1.0))
+    x[0, 1, 20, 41] = np.nan
+    want_logits, want_tap = oracle.resnet18_forward(x, hb, tap_layer=0)
+    m = Model(hb, abi.F16)
+    _, tap = _stage0(m, x, 1, 64, 64)
+    assert np.isnan(want_tap).any() and not np.isnan(want_tap).all()
+    assert np.array_equal(np.isnan(tap), np.isnan(want_tap))
+    ok = ~np.isnan(want_tap)
+    assert rel_l2(tap[ok], want_tap[ok]) < 2e-3

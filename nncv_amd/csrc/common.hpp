@@ -131,6 +131,9 @@ void launch_wino43_output(const WinoOutArgs& a, int m_dt, int out_dt, hipStream_
 // ---------------------------------------------------------------------------------------------
 void launch_maxpool3x3s2_nhwc(const void* in, void* out, int dt, int N, int H, int W, int C, hipStream_t s);
 void launch_global_avgpool_nhwc(const void* in, void* out, int dt, int N, int HW, int C, hipStream_t s);
+// head: global average pool + fully connected layer with bias, fp32 logits (C must be 512)
+void launch_avgpool_fc(const void* in, const void* w, const float* bias, float* out, int dt, int N, int HW, int C, int F,
+                       hipStream_t s);
 // generic strided copy/cast between layouts: dst[n,c,h,w] (+)= (c < Csrc ? src[n,c,h,w] : 0) for c < Cdst
 void launch_relayout(const void* src, int src_dt, Strides4 ss, void* dst, int dst_dt, Strides4 ds, int N,
                      int Csrc, int Cdst, int H, int W, bool accumulate, hipStream_t s);

@@ -330,6 +330,11 @@ void ResNet18::forward(const void* src, int N, int H, int W, void* logits, void*
       NNCV_HIP_CHECK(hipMemcpyAsync(tap, act[cur], (size_t)N * h * w * ch * es, hipMemcpyDeviceToDevice, s));
   }
   // head: global average pool (sum, one divide), FC with bias (Res18.mlir:609-628)
+  static const bool split_head = getenv("NNCV_HIP_NO_HEAD_FUSION") != nullptr;
+  if (!split_head) {
+    launch_avgpool_fc(act[cur], fc_w_.get(), fc_b_.as<float>(), static_cast<float*>(logits), dt_, N, h * w, 512, 1000, s);
+    return;
+  }
   launch_global_avgpool_nhwc(act[cur], pooled, dt_, N, h * w, 512, s);
   IgemmArgs a{};
   a.in = pooled; a.wt = fc_w_.get(); a.out = logits; a.shift = fc_b_.as<float>();

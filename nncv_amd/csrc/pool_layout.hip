@@ -110,6 +110,89 @@ void launch_global_avgpool_nhwc(const void* in, void* out, int dt, int N, int HW
 }
 
 // ---------------------------------------------------------------------------------------------
+// Network head in one launch: global average pool (sum over the image, one divide,
+// tests/Nets/Res18.mlir:609-614) and the 512 -> F fully connected layer with bias (:615-628).
+// A workgroup = one image x a slice of the F outputs.  Phase 1: the 256 threads sum the image's
+// pixels, two channels each (one coalesced kilobyte per pixel), fp32, and leave the 512 means in
+// LDS; the pooled vector is never rounded to the storage type.  Phase 2: a wave takes one output
+// at a time, its 64 lanes each hold 8 of the 512 means and read 8 consecutive weights (the whole
+// filter row is one contiguous kilobyte), and a shuffle tree adds the 64 partial dot products.
+// Slices recompute the (cheap, L2-resident) pooling instead of synchronising across workgroups.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void avgpool_fc_kernel(const T* __restrict__ in, const T* __restrict__ w,
+                                                         const float* __restrict__ bias, float* __restrict__ out, int HW,
+                                                         int F, int f_per_block) {
+  __shared__ float mean[512];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n = blockIdx.y;
+  {
+    typedef T V2 __attribute__((ext_vector_type(2)));
+    const V2* src = reinterpret_cast<const V2*>(in + (long long)n * HW * 512) + tid;
+    float s0 = 0.0f, s1 = 0.0f;
+    int p = 0;
+    for (; p + 16 <= HW; p += 16) {  // sixteen loads in flight; the additions stay in pixel order
+      V2 v[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) v[u] = src[(long long)(p + u) * 256];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        s0 += (float)v[u][0];
+        s1 += (float)v[u][1];
+      }
+    }
+    for (; p < HW; ++p) {
+      const V2 v = src[(long long)p * 256];
+      s0 += (float)v[0];
+      s1 += (float)v[1];
+    }
+    mean[2 * tid] = s0 / (float)HW;
+    mean[2 * tid + 1] = s1 / (float)HW;
+  }
+  __syncthreads();
+  float m[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) m[e] = mean[lane * 8 + e];
+  const int f_begin = blockIdx.x * f_per_block;
+  const int f_end = f_begin + f_per_block < F ? f_begin + f_per_block : F;
+  typedef T V8 __attribute__((ext_vector_type(8)));
+  for (int f0 = f_begin + wave; f0 < f_end; f0 += 32) {  // eight filters of this wave per trip: eight loads in flight
+    V8 wv[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int f = f0 + 4 * u < f_end ? f0 + 4 * u : f0;
+      wv[u] = *reinterpret_cast<const V8*>(w + (long long)f * 512 + lane * 8);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      float acc = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc += m[e] * (float)wv[u][e];
+#pragma unroll
+      for (int d = 32; d >= 1; d >>= 1) acc += __shfl_xor(acc, d);
+      const int f = f0 + 4 * u;
+      if (lane == 0 && f < f_end) out[(long long)n * F + f] = acc + (bias ? bias[f] : 0.0f);
+    }
+  }
+}
+
+// in: NHWC [N][HW][512] of dt; w: [F][512] of dt; bias: [F] fp32 or null; out: [N][F] fp32.
+void launch_avgpool_fc(const void* in, const void* w, const float* bias, float* out, int dt, int N, int HW, int C, int F,
+                       hipStream_t s) {
+  NNCV_REQUIRE(C == 512, "avgpool_fc: the head is built for 512 channels");
+  NNCV_REQUIRE(N > 0 && N <= 65535 && HW > 0 && F > 0, "avgpool_fc: bad shape");
+  const int fpb = 32;  // one trip of eight filters per wave: the kernel is a chain of memory latencies, so keep it short
+  dim3 grid((F + fpb - 1) / fpb, N);
+  const double es = (double)dtype_size(dt);
+  ProfScope prof("avgpool_fc", 2.0 * N * F * 512.0, es * ((double)N * HW * 512 + (double)F * 512) + 4.0 * N * F, s);
+  if (dt == kF16)
+    hipLaunchKernelGGL((avgpool_fc_kernel<half_t>), grid, dim3(256), 0, s, (const half_t*)in, (const half_t*)w, bias, out, HW, F, fpb);
+  else
+    hipLaunchKernelGGL((avgpool_fc_kernel<float>), grid, dim3(256), 0, s, (const float*)in, (const float*)w, bias, out, HW, F, fpb);
+  NNCV_HIP_CHECK(hipGetLastError());
+}
+
+// ---------------------------------------------------------------------------------------------
 // generic strided relayout / cast, dst (+)= src (operator-level ABI only; not on the ResNet-18 path)
 // ---------------------------------------------------------------------------------------------
 template <typename Ts, typename Td>

@@ -108,6 +108,11 @@ int nncv_hip_conv_algo(const nncv_hip_conv* c);
  * in is [N,C,H,W] UNPADDED, out [N,F,OH,OW]; residual may be NULL. NHWC is the native layout. */
 int nncv_hip_conv_forward(nncv_hip_conv* c, const void* in, int N, int H, int W, int layout, const void* residual,
                           void* out, void* stream);
+/* Measurement helper: `reps` NHWC launches of the layer back to back on `stream` between one pair
+ * of HIP events (after 5 untimed ones); *avg_us = elapsed / reps. Includes the gap between
+ * consecutive dispatches, so it reads slightly above a profiler's per-kernel time. */
+int nncv_hip_conv_time(nncv_hip_conv* c, const void* in, int N, int H, int W, const void* residual, void* out, int reps,
+                       void* stream, float* avg_us);
 
 /* C += A.B, fp32 row-major, DEVICE pointers (K and N multiples of 4). */
 int nncv_hip_matmul_f32(const float* A, const float* B, float* C, int M, int N, int K, void* stream);

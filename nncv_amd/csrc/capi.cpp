@@ -547,6 +547,33 @@ int nncv_hip_conv_forward(nncv_hip_conv* c, const void* in, int N, int H, int W,
   });
 }
 
+int nncv_hip_conv_time(nncv_hip_conv* c, const void* in, int N, int H, int W, const void* residual, void* out, int reps,
+                       void* stream, float* avg_us) {
+  return guarded([&] {
+    NNCV_REQUIRE(c && c->c && in && out && avg_us && reps > 0, "null argument");
+    Context& ctx = Context::get();
+    Sync sy(stream);
+    const ConvLayer& L = *c->c;
+    const size_t wsb = L.workspace_bytes(N, H, W, false);
+    ctx.arena.reserve(wsb + 1024, sy.s);
+    void* ws = ctx.arena.take(wsb);
+    hipEvent_t e0, e1;
+    NNCV_HIP_CHECK(hipEventCreate(&e0));
+    NNCV_HIP_CHECK(hipEventCreate(&e1));
+    for (int i = 0; i < 5; ++i) L.forward(in, N, H, W, residual, out, ws, sy.s);
+    NNCV_HIP_CHECK(hipEventRecord(e0, sy.s));
+    for (int i = 0; i < reps; ++i) L.forward(in, N, H, W, residual, out, ws, sy.s);
+    NNCV_HIP_CHECK(hipEventRecord(e1, sy.s));
+    NNCV_HIP_CHECK(hipEventSynchronize(e1));
+    float ms = 0.0f;
+    NNCV_HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    *avg_us = ms * 1000.0f / (float)reps;
+    sy.finish();
+  });
+}
+
 int nncv_hip_matmul_f32(const float* A, const float* B, float* C, int M, int N, int K, void* stream) {
   return guarded([&] {
     NNCV_REQUIRE(A && B && C, "null argument");

@@ -12,10 +12,12 @@
 //   2. K = 7 filter rows x 32 halves; the 64x224 filter matrix sits in registers for the whole
 //      life of the (persistent) workgroup, so the tap loop is 14 x (2 LDS reads + 4 MFMAs);
 //   3. scale/shift + ReLU in fp32, one rounding to fp16, tile to LDS ([slot][64 ch]); pixels
-//      outside the convolution output become -inf, which is the pooling halo;
-//   4. each thread takes one pooled pixel x 16 channels: nine 32-byte LDS reads, packed fp16
-//      max, NaN propagated separately (v_pk_max_f16 drops NaNs; arith.maximumf keeps them),
-//      one 32-byte store: four threads write a pixel's 128 contiguous bytes.
+//      outside the convolution output become +0, a neutral pooling halo after ReLU (every window
+//      holds at least one real, non-negative pixel);
+//   4. each thread takes one pooled pixel x 16 channels: nine 32-byte LDS reads, a packed
+//      UNSIGNED 16-bit max per tap (on non-negative halves the bit patterns sort like the values
+//      and NaNs sort above +inf, so this is arith.maximumf with its NaN propagation), one 32-byte
+//      store: four threads write a pixel's 128 contiguous bytes.
 // Workgroups are persistent (tiles strided by the grid) and request the next tile's image
 // pixels before the MFMAs of the current one.
 #include "mfma_tile.hpp"
@@ -131,7 +133,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int s = wave * 64 + j * 32 + lrow;
     cy[j] = s / kCTW;
     cx[j] = s - cy[j] * kCTW;
-    if (s >= 255) cy[j] = cx[j] = 0;  // the spare slot recomputes pixel 0; it is stored as -inf
+    if (s >= 255) cy[j] = cx[j] = 0;  // the spare slot recomputes pixel 0; it is stored as the halo value
     abase[j] = 2 * cy[j] * kInPitch + cx[j] * 16 + lchunk * 16;
   }
   // pooling role: pooled pixel tid/4 of the tile, channels 16*(tid%4)..
@@ -193,7 +195,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           for (int e = 0; e < 4; ++e) o[e] = (half_t)relu_ugt(acc[i][j][4 * q + e] * sc[e] + sh[e]);
           typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
           u32x2 bits = __builtin_bit_cast(u32x2, o);
-          if (!live) bits = u32x2{0xfc00fc00u, 0xfc00fc00u};
+          if (!live) bits = u32x2{0u, 0u};
           *reinterpret_cast<u32x2*>(conv_t + s * kConvPitch + c * 2) = bits;
         }
     }
@@ -201,13 +203,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     // ---- 3x3 stride-2 max over the convolution tile ----
     if (pp < kPTH * kPTW && py0 + ppy < a.PH && px0 + ppx < a.PW) {
-      half2v m[8];
-      ushort2v nanmax[8];
+      // After ReLU every value is +0, positive, +inf or NaN: as unsigned 16-bit patterns they sort
+      // like the numbers, with every NaN (either sign) above +inf.  One packed unsigned max per
+      // tap is therefore the NaN-propagating maximum of arith.maximumf, and +0 is a neutral halo.
+      ushort2v m[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        m[e] = __builtin_bit_cast(half2v, 0xfc00fc00u);
-        nanmax[e] = ushort2v{0, 0};
-      }
+      for (int e = 0; e < 8; ++e) m[e] = ushort2v{0, 0};
 #pragma unroll
       for (int dy = 0; dy < 3; ++dy)
 #pragma unroll
@@ -215,18 +216,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           const unsigned char* src = conv_t + ((2 * ppy + dy) * kCTW + 2 * ppx + dx) * kConvPitch + pg * 32;
           const u32x4 v0 = *reinterpret_cast<const u32x4*>(src), v1 = *reinterpret_cast<const u32x4*>(src + 16);
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const unsigned w = e < 4 ? v0[e] : v1[e - 4];
-            m[e] = __builtin_elementwise_max(m[e], __builtin_bit_cast(half2v, w));
-            nanmax[e] = __builtin_elementwise_max(nanmax[e], __builtin_bit_cast(ushort2v, w & 0x7fff7fffu));
-          }
+          for (int e = 0; e < 8; ++e) m[e] = __builtin_elementwise_max(m[e], __builtin_bit_cast(ushort2v, e < 4 ? v0[e] : v1[e - 4]));
         }
       u32x4 o0, o1;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        unsigned w = __builtin_bit_cast(unsigned, m[e]);
-        if (nanmax[e][0] > 0x7c00) w = (w & 0xffff0000u) | 0x7e00u;  // a NaN in the window wins
-        if (nanmax[e][1] > 0x7c00) w = (w & 0x0000ffffu) | 0x7e000000u;
+        const unsigned w = __builtin_bit_cast(unsigned, m[e]);
         if (e < 4) o0[e] = w; else o1[e - 4] = w;
       }
       half_t* dst = a.out + (((long long)n * a.PH + py0 + ppy) * a.PW + px0 + ppx) * 64 + pg * 16;

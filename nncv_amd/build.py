@@ -21,7 +21,10 @@ HOST_SOURCES = ["model.cpp", "capi.cpp", "datatype.cpp", "profiler.cpp"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-Wall", "-Wno-unused-function"]
 # packed-fp32 instruction selection is switched off for all device code
-DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# the first kernel arguments (up to 14 dwords of scalars/pointers) arrive preloaded in SGPRs
+# instead of through a scalar load at the top of every wave
+DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+          "-mllvm", "-amdgpu-kernarg-preload-count=14"]
 
 
 def _stale(src, obj):

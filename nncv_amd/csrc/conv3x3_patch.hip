@@ -73,7 +73,14 @@ struct PatchCfg {
 };
 
 template <typename T, typename OutT, int WS, int WK>
-__global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv3x3_patch_kernel(const PatchArgs a) {
+__global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv3x3_patch_kernel(
+    // the values the patch addressing needs first, as plain leading arguments: those are preloaded
+    // into SGPRs at wave launch, the struct behind them is fetched by a scalar load as usual
+    const void* in_p, int tiles_p, int tiles_y_p, int tn_p, int th_p, int n_p, int h_p, int w_p, int c_p, int rw_log_p,
+    int xcd_by_filter_p, unsigned in_bytes_p, const PatchArgs a_rest) {
+  PatchArgs a = a_rest;
+  a.in = in_p; a.tiles = tiles_p; a.tiles_y = tiles_y_p; a.TN = tn_p; a.TH = th_p; a.N = n_p; a.H = h_p; a.W = w_p; a.C = c_p;
+  a.rw_log = rw_log_p; a.xcd_by_filter = xcd_by_filter_p; a.in_bytes = in_bytes_p;
   typedef PatchCfg<WS, WK> Cfg;
   constexpr int NT = Cfg::NT, kPasses = Cfg::passes, NSET = Cfg::nset;
   constexpr int kDepth = WK == 1 ? 3 : 4;  // pixel-operand ring: LDS reads run kDepth-1 steps ahead of their MFMAs
@@ -350,7 +357,8 @@ static void launch_patch_cfg(const PatchArgs& a, double flops, double bytes, con
   (void)attr;
   ProfScope prof(tag, flops, bytes, s);
   dim3 grid((a.tiles + kXcdsP - 1) / kXcdsP * kXcdsP, (a.F + 63) / 64);
-  hipLaunchKernelGGL(kern, grid, dim3(Cfg::NT), Cfg::smem, s, a);
+  hipLaunchKernelGGL(kern, grid, dim3(Cfg::NT), Cfg::smem, s, a.in, a.tiles, a.tiles_y, a.TN, a.TH, a.N, a.H, a.W, a.C, a.rw_log,
+                     a.xcd_by_filter, a.in_bytes, a);
 }
 
 void launch_conv3x3_patch(const IgemmArgs& g, int in_dt, int out_dt, hipStream_t s) {

@@ -1,0 +1,68 @@
+"""BASELINE configurations at their full sizes on the GPU.
+
+The oracle is too slow for whole batches, so every full-size case is checked two ways: the first
+images of the batch against the oracle (a convolution / the network treats images independently),
+and size-independent properties of the full batch (batch independence, permutation equivariance).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from nncv_amd import abi, synth
+from gpu_util import Conv, Model, dev, host, nhwc, nchw, rel_l2, FP16_REL_L2
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle_layer(x, w, stride, bn, res):
+    y = oracle.batchnorm(oracle.conv2d_nchw_fchw(oracle.pad_nchw(x, 1), w, stride=stride), *bn)
+    if res is not None:
+        y = y + res
+    return oracle.relu(y)
+
+
+@pytest.mark.parametrize("i", range(len(synth.CFG5_LAYERS)))
+def test_conv3x3_layer_sweep_fp16_batch64(i):
+    """3x3 conv + BN + ReLU (+ residual) of every ResNet-18 stage, fp16, batch 64."""
+    c, k, h, s = synth.CFG5_LAYERS[i]
+    x, w, bn, res = synth.cfg5_layer(i, 64)
+    bn = tuple(synth.round_fp16(b) for b in bn)
+    layer = Conv(abi.F16, w, s, 1, bn=bn, relu=True)
+    xd = dev(nhwc(x), abi.F16)
+    rd = dev(nhwc(res), abi.F16) if res is not None else None
+    got = nchw(host(layer(xd, abi.NHWC, residual=rd)))
+    # first two images against the oracle
+    want = _oracle_layer(x[:2], w, s, bn, res[:2] if res is not None else None)
+    err = rel_l2(got[:2], want)
+    print("layer", (c, k, h, s), "rel_l2", err, flush=True)
+    assert err < FP16_REL_L2
+    assert np.isfinite(got).all() and (got >= 0).all()
+    # permutation equivariance over the batch, bit for bit (same launch geometry)
+    perm = np.random.default_rng(i).permutation(64)
+    xp = dev(nhwc(x[perm]), abi.F16)
+    rp = dev(nhwc(res[perm]), abi.F16) if res is not None else None
+    got_p = nchw(host(layer(xp, abi.NHWC, residual=rp)))
+    assert np.array_equal(got_p, got[perm])
+
+
+def test_resnet18_fp16_batch32_full_size():
+    """BASELINE config 4 at its real size: [32,3,224,224] fp16."""
+    hb = synth.round_fp16(synth.resnet18_params())
+    x = synth.round_fp16(synth.cfg4_input(32))
+    m = Model(hb, abi.F16)
+    got = host(m(dev(x, abi.F16)))
+    assert got.shape == (32, 1000) and np.isfinite(got).all()
+    want = oracle.resnet18_forward(x[:2], hb)
+    err = rel_l2(got[:2], want)
+    print("bs32 first two images rel_l2", err, "top1", got[:2].argmax(1), want.argmax(1), flush=True)
+    assert err < FP16_REL_L2
+    assert (got[:2].argmax(1) == want.argmax(1)).all()
+    # batch 1 (other tile shapes and K-group counts, hence another summation order) agrees closely
+    one = host(m(dev(x[5:6], abi.F16)))
+    assert rel_l2(one, got[5:6]) < 2e-3
+    assert one.argmax(1) == got[5:6].argmax(1)
+    # permuting the batch permutes the logits, bit for bit
+    perm = np.random.default_rng(7).permutation(32)
+    got_p = host(m(dev(x[perm], abi.F16)))
+    assert np.array_equal(got_p, got[perm])

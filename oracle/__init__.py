@@ -195,6 +195,68 @@ def resnet18_forward(x, params, tap_layer=-1):
     return (y, tap) if tap_layer >= 0 else y
 
 
+# ---- AVX2/OpenMP restatement of the HostWParallel schedule (hostwparallel.cpp): the timed CPU baseline ----
+_HWP = None
+
+
+def hwp_lib():
+    global _HWP
+    if _HWP is None:
+        p = os.path.join(_HERE, "libhostwparallel.so")
+        if not os.path.exists(p):
+            raise RuntimeError("%s is missing: run `make -C oracle`" % p)
+        L = ctypes.CDLL(p)
+        L.hwp_conv2d_nchw_fchw.argtypes = [_f32p, _f32p, _f32p] + [ctypes.c_int] * 9
+        _HWP = L
+    return _HWP
+
+
+def hwp_conv2d(x, w, stride=1, pad=0):
+    """conv_2d_nchw_fchw over a zero halo of `pad`, fp32 accumulation, OpenMP x AVX2."""
+    x, w = _c(x), _c(w)
+    N, C, H, W = x.shape
+    F, C2, R, S = w.shape
+    assert C == C2
+    OH, OW = (H + 2 * pad - R) // stride + 1, (W + 2 * pad - S) // stride + 1
+    y = np.empty((N, F, OH, OW), np.float32)
+    rc = hwp_lib().hwp_conv2d_nchw_fchw(x, w, y, N, C, H, W, F, R, S, stride, pad)
+    assert rc == 0
+    return y
+
+
+def hwp_resnet18_forward(x, params):
+    """ResNet-18 of tests/Nets/Res18.mlir with the convolutions on the AVX2/OpenMP routine above and
+    every other op on the scalar oracle's; same parameter blob order as resnet18_forward."""
+    from nncv_amd import resnet18_spec as spec
+    x, params = _c(x), _c(params)
+    tensors, off = {}, 0
+    for name, shape in spec.tensor_table():
+        n = spec.numel(shape)
+        tensors[name] = params[off:off + n].reshape(shape)
+        off += n
+    assert off == params.size
+
+    def bn(y, prefix):
+        return batchnorm(y, tensors[prefix + ".weight"], tensors[prefix + ".bias"], tensors[prefix + ".running_mean"],
+                         tensors[prefix + ".running_var"])
+
+    y = relu(bn(hwp_conv2d(x, tensors["conv1.weight"], 2, 3), "bn1"))
+    y = maxpool3x3s2(y)
+    cin = 64
+    for li, f in enumerate(spec.WIDTHS, start=1):
+        for blk in range(2):
+            p = "layer%d.%d" % (li, blk)
+            stride = 2 if (li > 1 and blk == 0) else 1
+            t = relu(bn(hwp_conv2d(y, tensors[p + ".conv1.weight"], stride, 1), p + ".bn1"))
+            t = bn(hwp_conv2d(t, tensors[p + ".conv2.weight"], 1, 1), p + ".bn2")
+            idn = y
+            if stride != 1 or cin != f:
+                idn = bn(hwp_conv2d(y, tensors[p + ".downsample.0.weight"], stride, 0), p + ".downsample.1")
+            y = relu(t + idn)
+            cin = f
+    return fc(global_avgpool(y), tensors["fc.weight"], tensors["fc.bias"])
+
+
 # ---- reference-built model.bin reader/writer (oracle/_ref), present only where it was built ----
 def ref_lib():
     global _REF

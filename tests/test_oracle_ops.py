@@ -164,3 +164,24 @@ def test_winograd_equals_direct_ragged(H, W):
     np.testing.assert_allclose(wino, direct, rtol=1e-5, atol=1e-5)
     V = oracle.wino43_input_transform(x, pad=1)
     assert V.shape == (36, 2 * ((H + 3) // 4) * ((W + 3) // 4), 5)
+
+
+@pytest.mark.parametrize("R,stride,pad", [(3, 1, 1), (3, 2, 1), (1, 2, 0), (7, 2, 3), (3, 1, 0)])
+def test_hostwparallel_conv_matches_scalar_oracle(R, stride, pad):
+    """The AVX2/OpenMP convolution timed as the CPU baseline computes the same convolution as the
+    scalar oracle (fp32 vs fp64 accumulation: agreement to fp32 rounding), ragged sizes included."""
+    x = synth.normal(910, (2, 12, 19, 23))
+    w = synth.normal(911, (10, 12, R, R), std=0.2)
+    got = oracle.hwp_conv2d(x, w, stride, pad)
+    want = oracle.conv2d_nchw_fchw(oracle.pad_nchw(x, pad), w, stride=stride)
+    assert got.shape == want.shape
+    assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max()
+
+
+def test_hostwparallel_resnet18_matches_scalar_oracle():
+    blob = synth.resnet18_params()
+    x = synth.uniform(912, (1, 3, 64, 96), 0.0, 1.0)
+    got = oracle.hwp_resnet18_forward(x, blob)
+    want = oracle.resnet18_forward(x, blob)
+    assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+    assert got.argmax(1) == want.argmax(1)

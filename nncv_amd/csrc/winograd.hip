@@ -233,6 +233,165 @@ __global__ __launch_bounds__(256) void wino43_output_kernel(const WinoOutArgs a,
 }
 
 // ---------------------------------------------------------------------------------------------
+// LDS-staged forms for dense NHWC tensors whose channel count is a multiple of 64: the 2-D
+// transform is done as two 1-D passes with the intermediate in LDS (fp32), so that a thread never
+// holds more than one 6-vector per channel, and every global access is 16 bytes per lane with 8
+// (fp16) or 16 (fp32) consecutive lanes covering the 64 channels of one pixel / one V or M row.
+// A workgroup owns kTiles tiles x 64 channels.
+//   input : pass 1  thread = (tile, column x, 16-byte channel group): 6 loads down the column,
+//                   B^T along y, 6 vectors to LDS[tile][i][x][c];
+//           pass 2  thread = (tile, row i, channel group): 6 vectors from LDS, B^T along x,
+//                   6 stores to V[6i+j][tile][c].
+//   output: pass 1  thread = (tile, column j, channel group): 6 loads M[6i+j][tile][f], A^T along
+//                   i, 4 vectors to LDS[tile][r][j][f];
+//           pass 2  thread = (tile, row r, channel group): 6 vectors from LDS, A^T along j, then
+//                   scale/shift, residual, ReLU and one rounding, up to 4 pixel stores.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+struct WinoLds {
+  static constexpr int VW = 16 / (int)sizeof(T);  // channels per thread
+  static constexpr int CG = 64 / VW;              // channel groups per 64 channels
+  static constexpr int kTiles = 240 / (6 * CG);   // fp16: 5, fp32: 2
+  typedef T Vec __attribute__((ext_vector_type(VW)));
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void wino43_input_lds_kernel(const T* __restrict__ in, T* __restrict__ V, int N, int C, int H,
+                                                               int W, int pad, int TH, int TW) {
+  typedef WinoLds<T> L;
+  constexpr int VW = L::VW, CG = L::CG, KT = L::kTiles;
+  typedef typename L::Vec Vec;
+  __shared__ __align__(16) float mid[KT][6][6][64];
+  const int tid = threadIdx.x;
+  const long long tiles = (long long)N * TH * TW;
+  const long long tile0 = (long long)blockIdx.x * KT;
+  const int c0 = blockIdx.y * 64;
+  const int cg = tid % CG, u = (tid / CG) % 6, tl = tid / (6 * CG);
+  const long long tile = tile0 + tl;
+  const bool live = tl < KT && tile < tiles;
+  if (live) {  // pass 1: u = column x
+    const int tx = (int)(tile % TW), ty = (int)((tile / TW) % TH), n = (int)(tile / ((long long)TW * TH));
+    const int ix = tx * 4 - pad + u, y0 = ty * 4 - pad;
+    Vec d[6];
+#pragma unroll
+    for (int y = 0; y < 6; ++y) {
+      const int iy = y0 + y;
+      const bool ok = (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
+      // out-of-image taps read pixel 0 (a valid address) and are zeroed: no divergent branch
+      const long long off = ok ? (((long long)n * H + iy) * W + ix) * C + c0 + cg * VW : 0;
+      Vec v = *reinterpret_cast<const Vec*>(in + off);
+      if (!ok)
+        for (int e = 0; e < VW; ++e) v[e] = (T)0.0f;
+      d[y] = v;
+    }
+#pragma unroll
+    for (int e = 0; e < VW; ++e) {
+      float col[6], o[6];
+#pragma unroll
+      for (int y = 0; y < 6; ++y) col[y] = (float)d[y][e];
+      bt6(col, o);
+#pragma unroll
+      for (int i = 0; i < 6; ++i) mid[tl][i][u][cg * VW + e] = o[i];
+    }
+  }
+  __syncthreads();
+  if (live) {  // pass 2: u = row i
+#pragma unroll
+    for (int e0 = 0; e0 < VW; e0 += 4) {
+      float o[6][4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float row[6], r[6];
+#pragma unroll
+        for (int x = 0; x < 6; ++x) row[x] = mid[tl][u][x][cg * VW + e0 + e];
+        bt6(row, r);
+#pragma unroll
+        for (int j = 0; j < 6; ++j) o[j][e] = r[j];
+      }
+#pragma unroll
+      for (int j = 0; j < 6; ++j) {
+        typedef T V4 __attribute__((ext_vector_type(4)));
+        V4 w;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = (T)o[j][e];
+        *reinterpret_cast<V4*>(V + ((long long)(u * 6 + j) * tiles + tile) * C + c0 + cg * VW + e0) = w;
+      }
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void wino43_output_lds_kernel(const WinoOutArgs a, int TH, int TW) {
+  typedef WinoLds<T> L;
+  constexpr int VW = L::VW, CG = L::CG, KT = L::kTiles;
+  typedef typename L::Vec Vec;
+  __shared__ __align__(16) float mid[KT][4][6][64];
+  const int tid = threadIdx.x;
+  const long long tiles = (long long)a.N * TH * TW;
+  const long long tile0 = (long long)blockIdx.x * KT;
+  const int f0 = blockIdx.y * 64;
+  const int cg = tid % CG, u = (tid / CG) % 6, tl = tid / (6 * CG);
+  const long long tile = tile0 + tl;
+  const bool live = tl < KT && tile < tiles;
+  const T* M = static_cast<const T*>(a.M);
+  if (live) {  // pass 1: u = column j
+    Vec m[6];
+#pragma unroll
+    for (int i = 0; i < 6; ++i) m[i] = *reinterpret_cast<const Vec*>(M + ((long long)(i * 6 + u) * tiles + tile) * a.F + f0 + cg * VW);
+#pragma unroll
+    for (int e = 0; e < VW; ++e) {
+      float col[6], o[4];
+#pragma unroll
+      for (int i = 0; i < 6; ++i) col[i] = (float)m[i][e];
+      at6(col, o);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mid[tl][r][u][cg * VW + e] = o[r];
+    }
+  }
+  __syncthreads();
+  if (live && u < 4) {  // pass 2: u = row r
+    const int tx = (int)(tile % TW), ty = (int)((tile / TW) % TH), n = (int)(tile / ((long long)TW * TH));
+    const int oy = ty * 4 + u;
+    if (oy < a.OH) {
+      T* out = static_cast<T*>(a.out);
+      const T* res = static_cast<const T*>(a.residual);
+      const int f = f0 + cg * VW;
+      float y[4][VW];
+#pragma unroll
+      for (int e = 0; e < VW; ++e) {
+        float row[6], o[4];
+#pragma unroll
+        for (int j = 0; j < 6; ++j) row[j] = mid[tl][u][j][cg * VW + e];
+        at6(row, o);
+        const float sc = a.scale ? a.scale[f + e] : 1.0f, sh = a.shift ? a.shift[f + e] : 0.0f;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) y[q][e] = o[q] * sc + sh;
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int ox = tx * 4 + q;
+        if (ox >= a.OW) continue;
+        const long long o = (((long long)n * a.OH + oy) * a.OW + ox) * a.F + f;
+        if (res) {
+          const Vec rv = *reinterpret_cast<const Vec*>(res + o);
+#pragma unroll
+          for (int e = 0; e < VW; ++e) y[q][e] += (float)rv[e];
+        }
+        if (a.accumulate) {
+          const Vec ov = *reinterpret_cast<const Vec*>(out + o);
+#pragma unroll
+          for (int e = 0; e < VW; ++e) y[q][e] += (float)ov[e];
+        }
+        Vec w;
+#pragma unroll
+        for (int e = 0; e < VW; ++e) w[e] = (T)(a.relu ? relu_ugt(y[q][e]) : y[q][e]);
+        *reinterpret_cast<Vec*>(out + o) = w;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // launchers
 // ---------------------------------------------------------------------------------------------
 void launch_wino43_filter(const void* w, int w_dt, void* U, int u_dt, int F, int C, hipStream_t s) {
@@ -262,6 +421,20 @@ void launch_wino43_input(const void* in, int in_dt, Strides4 st, void* V, int v_
   const double es = dtype_size(in_dt), vs = dtype_size(v_dt);
   ProfScope prof(contig ? "wino43_input<nhwc>" : "wino43_input<strided>", 0.0,
                  es * N * C * H * W + vs * 36.0 * N * TH * TW * C, s);
+  // dense NHWC with whole 64-channel groups: the LDS-staged kernel
+  if (contig && in_dt == v_dt && C % 64 == 0 && st.w == C && st.h == (long long)W * C && st.n == (long long)H * W * C &&
+      getenv("NNCV_HIP_WINO_SIMPLE") == nullptr) {
+    const long long tiles = (long long)N * TH * TW;
+    if (in_dt == kF16) {
+      dim3 g((unsigned)((tiles + WinoLds<half_t>::kTiles - 1) / WinoLds<half_t>::kTiles), C / 64);
+      hipLaunchKernelGGL((wino43_input_lds_kernel<half_t>), g, dim3(256), 0, s, (const half_t*)in, (half_t*)V, N, C, H, W, pad, TH, TW);
+    } else {
+      dim3 g((unsigned)((tiles + WinoLds<float>::kTiles - 1) / WinoLds<float>::kTiles), C / 64);
+      hipLaunchKernelGGL((wino43_input_lds_kernel<float>), g, dim3(256), 0, s, (const float*)in, (float*)V, N, C, H, W, pad, TH, TW);
+    }
+    NNCV_HIP_CHECK(hipGetLastError());
+    return;
+  }
 #define LAUNCH(TI, TV, CC)                                                                               \
   hipLaunchKernelGGL((wino43_input_kernel<TI, TV, CC>), dim3((unsigned)grid), dim3(blk), 0, s, (const TI*)in, st, \
                      (TV*)V, N, C, H, W, pad, TH, TW)
@@ -283,6 +456,19 @@ void launch_wino43_output(const WinoOutArgs& a, int m_dt, int out_dt, hipStream_
   const double ms = dtype_size(m_dt), os = dtype_size(out_dt);
   ProfScope prof(contig ? "wino43_output<nhwc>" : "wino43_output<strided>", 0.0,
                  ms * 36.0 * a.N * TH * TW * a.F + os * (double)a.N * a.F * a.OH * a.OW * (a.residual ? 2 : 1), s);
+  if (contig && m_dt == out_dt && a.F % 64 == 0 && a.st.w == a.F && a.st.h == (long long)a.OW * a.F &&
+      a.st.n == (long long)a.OH * a.OW * a.F && getenv("NNCV_HIP_WINO_SIMPLE") == nullptr) {
+    const long long tiles = (long long)a.N * TH * TW;
+    if (m_dt == kF16) {
+      dim3 g((unsigned)((tiles + WinoLds<half_t>::kTiles - 1) / WinoLds<half_t>::kTiles), a.F / 64);
+      hipLaunchKernelGGL((wino43_output_lds_kernel<half_t>), g, dim3(256), 0, s, a, TH, TW);
+    } else {
+      dim3 g((unsigned)((tiles + WinoLds<float>::kTiles - 1) / WinoLds<float>::kTiles), a.F / 64);
+      hipLaunchKernelGGL((wino43_output_lds_kernel<float>), g, dim3(256), 0, s, a, TH, TW);
+    }
+    NNCV_HIP_CHECK(hipGetLastError());
+    return;
+  }
 #define LAUNCH(TM, TO, CC) \
   hipLaunchKernelGGL((wino43_output_kernel<TM, TO, CC>), dim3((unsigned)grid), dim3(blk), 0, s, a, TH, TW)
   if (m_dt == kF32 && out_dt == kF32) { if (contig) LAUNCH(float, float, true); else LAUNCH(float, float, false); }

@@ -72,7 +72,7 @@ struct PatchCfg {
   static constexpr int smem = load_bytes > tile_bytes ? load_bytes : tile_bytes;
 };
 
-template <typename T, typename OutT, int WS, int WK>
+template <typename T, typename OutT, int WS, int WK, int NI>
 __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv3x3_patch_kernel(
     // the values the patch addressing needs first, as plain leading arguments: those are preloaded
     // into SGPRs at wave launch, the struct behind them is fetched by a scalar load as usual
@@ -86,7 +86,8 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   constexpr int kDepth = WK == 1 ? 3 : 4;  // pixel-operand ring: LDS reads run kDepth-1 steps ahead of their MFMAs
   constexpr int ES = sizeof(T);
   constexpr int KPG = 4 / WK;     // 32-byte K sub-steps per K group and tap
-  constexpr int NF = 2 * KPG;     // weight fragments (kilobytes) per wave and tap
+  constexpr int NF = NI * KPG;    // weight fragments (kilobytes) per wave and tap
+  static_assert(NI == 1 || NI == 2, "a wave owns one or two 32-filter halves");
   static_assert(WK == 1 || WK == 2 || WK == 4, "K groups split the four sub-steps of a tap");
   extern __shared__ __align__(16) unsigned char smem[];
   unsigned char* patch = smem;
@@ -106,7 +107,7 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
     fblk = blockIdx.y;
   }
   if (tile >= a.tiles) return;
-  const int f0blk = fblk * 64;
+  const int f0blk = fblk * (32 * NI);
   const int n0 = (tile / a.tiles_y) * a.TN, y0 = (tile % a.tiles_y) * a.TH;
   const int PH = a.TH + 2, PW = a.W + 2;
 
@@ -171,14 +172,18 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   pload(0);  // first in the queue: the patch gates the tap loop, the weights below only its first taps
   __builtin_amdgcn_sched_barrier(0);
 
-  // ---- weights: iteration `it`, sub-step k of this K group, filter half i is the kilobyte at
-  //      wbase + it*8192 + (k*2+i)*1024; NSET register sets hold iterations it .. it+NSET-1 ----
-  const int wbase = (fblk * niter * 8 + wk * KPG * 2) * 1024;
+  // ---- weights: iteration `it`, sub-step k of this K group, filter half i of 64-filter block fb is
+  //      the kilobyte at (fb*niter*8 + it*8 + k*2 + i)*1024; NSET register sets hold iterations
+  //      it .. it+NSET-1.  An NI = 1 workgroup owns one half of a 64-filter block. ----
+  const int wbase = NI == 2 ? (fblk * niter * 8 + wk * KPG * 2) * 1024 : ((fblk >> 1) * niter * 8 + wk * KPG * 2 + (fblk & 1)) * 1024;
   const unsigned wlane = lane * 16;
+  auto wfrag = [](int k, int i) { return (k * 2 + i) * 1024; };  // byte offset of fragment (k, i) inside an iteration
   auto wload = [&](u32x4(&r)[NF], int it) {
     const int so = it < niter ? wbase + it * 8192 : 0;  // past the end: re-read block 0 (never used)
 #pragma unroll
-    for (int q = 0; q < NF; ++q) r[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_wf, wlane, so + q * 1024, 0);
+    for (int k = 0; k < KPG; ++k)
+#pragma unroll
+      for (int i = 0; i < NI; ++i) r[k * NI + i] = __builtin_amdgcn_raw_buffer_load_b128(rs_wf, wlane, so + wfrag(k, i), 0);
   };
   u32x4 wregs[NSET][NF];
 #pragma unroll
@@ -204,7 +209,7 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
     obase[j] = ok ? (((n0 + nl) * a.H + y0 + ty) * a.W + tx) * a.F : -1;
   }
 
-  floatx16 acc[2][2];
+  floatx16 acc[2][2];  // [filter half][pixel half]; with NI = 1 only acc[0] is used
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -254,14 +259,14 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
         if constexpr (st + kDepth - 1 < kSteps) ldp(std::integral_constant<int, st + kDepth - 1>());
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < NI; ++i)
 #pragma unroll
-          for (int j = 0; j < 2; ++j) Mma<T>::run(wregs[set][k * 2 + i], ring[st % kDepth][j], acc[i][j]);
+          for (int j = 0; j < 2; ++j) Mma<T>::run(wregs[set][k * NI + i], ring[st % kDepth][j], acc[i][j]);
         const int it_next = slab * 9 + t + NSET;
         const int wso = it_next < niter ? wbase + it_next * 8192 : 0;  // past the end: re-read block 0 (never used)
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
-          wregs[set][k * 2 + i] = __builtin_amdgcn_raw_buffer_load_b128(rs_wf, wlane, wso + (k * 2 + i) * 1024, 0);
+        for (int i = 0; i < NI; ++i)
+          wregs[set][k * NI + i] = __builtin_amdgcn_raw_buffer_load_b128(rs_wf, wlane, wso + wfrag(k, i), 0);
         __builtin_amdgcn_sched_barrier(0);
         self(self, std::integral_constant<int, st + 1>());
       }
@@ -276,7 +281,7 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   }
   __syncthreads();  // every wave is done with the patch: LDS becomes the output tiles
 
-  tile_reduce_store<OutT, WK>(acc, smem + ws * kTileBytes, wk, lane, obase, f0blk, a.F, ess,
+  tile_reduce_store<OutT, WK, NI>(acc, smem + ws * kTileBytes, wk, lane, obase, f0blk, a.F, ess,
                               static_cast<const OutT*>(a.residual), static_cast<OutT*>(a.out), a.relu);
 }
 
@@ -346,17 +351,17 @@ bool conv3x3_patch_applicable(const IgemmArgs& a, int in_dt) {
          plan_patch(a.N, a.H, a.W, a.F, a.C / slab, &ws, &tn, &th, &lg);
 }
 
-template <typename T, typename OutT, int WS, int WK>
+template <typename T, typename OutT, int WS, int WK, int NI>
 static void launch_patch_cfg(const PatchArgs& a, double flops, double bytes, const char* tag, hipStream_t s) {
   typedef PatchCfg<WS, WK> Cfg;
-  auto kern = conv3x3_patch_kernel<T, OutT, WS, WK>;
+  auto kern = conv3x3_patch_kernel<T, OutT, WS, WK, NI>;
   static const bool attr = [&] {
     NNCV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::smem));
     return true;
   }();
   (void)attr;
   ProfScope prof(tag, flops, bytes, s);
-  dim3 grid((a.tiles + kXcdsP - 1) / kXcdsP * kXcdsP, (a.F + 63) / 64);
+  dim3 grid((a.tiles + kXcdsP - 1) / kXcdsP * kXcdsP, (a.F + 32 * NI - 1) / (32 * NI));
   hipLaunchKernelGGL(kern, grid, dim3(Cfg::NT), Cfg::smem, s, a.in, a.tiles, a.tiles_y, a.TN, a.TH, a.N, a.H, a.W, a.C, a.rw_log,
                      a.xcd_by_filter, a.in_bytes, a);
 }
@@ -382,14 +387,20 @@ void launch_conv3x3_patch(const IgemmArgs& g, int in_dt, int out_dt, hipStream_t
   const double bytes = es * (P * a.C + 9.0 * a.C * a.F) + os * P * a.F * (a.residual ? 2 : 1);
   const bool h = in_dt == kF16 && out_dt == kF16, f = in_dt == kF32 && out_dt == kF32;
   NNCV_REQUIRE(h || f, "conv3x3_patch: unsupported dtype combination");
+  // Few workgroups (small batch on the deep layers: each streams its filter block's weights through
+  // one CU's 64 B/clk vector-memory path): split the 64-filter blocks in two and use twice the CUs.
+  const bool halves = ws == 1 && (long long)a.tiles * ((a.F + 63) / 64) < 128 && a.F % 64 == 0;
+  if (halves) a.xcd_by_filter = (a.F / 32) % kXcdsP == 0 && a.wf_bytes > (2u << 20);
   if (h) {
-    if (ws == 4) launch_patch_cfg<half_t, half_t, 4, 1>(a, flops, bytes, "conv3x3_patch<f16,4,1>", s);
-    else if (ws == 2) launch_patch_cfg<half_t, half_t, 2, 2>(a, flops, bytes, "conv3x3_patch<f16,2,2>", s);
-    else launch_patch_cfg<half_t, half_t, 1, 4>(a, flops, bytes, "conv3x3_patch<f16,1,4>", s);
+    if (ws == 4) launch_patch_cfg<half_t, half_t, 4, 1, 2>(a, flops, bytes, "conv3x3_patch<f16,4,1>", s);
+    else if (ws == 2) launch_patch_cfg<half_t, half_t, 2, 2, 2>(a, flops, bytes, "conv3x3_patch<f16,2,2>", s);
+    else if (halves) launch_patch_cfg<half_t, half_t, 1, 4, 1>(a, flops, bytes, "conv3x3_patch<f16,1,4,half>", s);
+    else launch_patch_cfg<half_t, half_t, 1, 4, 2>(a, flops, bytes, "conv3x3_patch<f16,1,4>", s);
   } else {
-    if (ws == 4) launch_patch_cfg<float, float, 4, 1>(a, flops, bytes, "conv3x3_patch<f32,4,1>", s);
-    else if (ws == 2) launch_patch_cfg<float, float, 2, 2>(a, flops, bytes, "conv3x3_patch<f32,2,2>", s);
-    else launch_patch_cfg<float, float, 1, 4>(a, flops, bytes, "conv3x3_patch<f32,1,4>", s);
+    if (ws == 4) launch_patch_cfg<float, float, 4, 1, 2>(a, flops, bytes, "conv3x3_patch<f32,4,1>", s);
+    else if (ws == 2) launch_patch_cfg<float, float, 2, 2, 2>(a, flops, bytes, "conv3x3_patch<f32,2,2>", s);
+    else if (halves) launch_patch_cfg<float, float, 1, 4, 1>(a, flops, bytes, "conv3x3_patch<f32,1,4,half>", s);
+    else launch_patch_cfg<float, float, 1, 4, 2>(a, flops, bytes, "conv3x3_patch<f32,1,4>", s);
   }
   NNCV_HIP_CHECK(hipGetLastError());
 }

@@ -99,7 +99,9 @@ struct EpiScale {
   }
 };
 
-template <typename OutT, int NG>
+// NI = 1: the wave tile is 64 slots x 32 channels (acc[0] only); the LDS tile keeps its 64-channel
+// rows and the lanes of the upper 32 channels simply store nothing.
+template <typename OutT, int NG, int NI = 2>
 __device__ __forceinline__ void tile_reduce_store(const floatx16 (&acc)[2][2], unsigned char* tile, int g, int lane,
                                                   const int (&rowoff)[2], int f0, int F, const EpiScale<OutT>& ss,
                                                   const OutT* res, OutT* out, int relu) {
@@ -110,7 +112,7 @@ __device__ __forceinline__ void tile_reduce_store(const floatx16 (&acc)[2][2], u
   static_assert(NIT >= 1, "too many K groups for this output type");
   typedef OutT VO __attribute__((ext_vector_type(FPL)));
   const int fc = (lane % LPR) * FPL;
-  const bool fok = f0 + fc < F;
+  const bool fok = f0 + fc < F && fc < 32 * NI;
   // Output offsets of the rows this lane stores, fetched from the lanes that own those slots, and
   // the residual rows requested before the reduction so that their latency hides behind it.
   int o[NIT];
@@ -136,7 +138,7 @@ __device__ __forceinline__ void tile_reduce_store(const floatx16 (&acc)[2][2], u
 #pragma unroll
       for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < NI; ++i)
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             floatx4* p = reinterpret_cast<floatx4*>(tile + (j * 32 + lrow) * kTilePitch + (i * 32 + 8 * q + 4 * lchunk) * 4);

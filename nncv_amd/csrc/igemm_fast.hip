@@ -33,7 +33,7 @@ constexpr unsigned kOOB = 0x7fffff00u;   // byte offset beyond any buffer this k
 constexpr int kXcds = 8;
 }  // namespace
 
-template <typename T, typename OutT, int WP, int WF, int WK, int KS>
+template <typename T, typename OutT, int WP, int WF, int WK, int KS, int NI>
 __global__ __launch_bounds__(64 * WP * WF * WK) void igemm_fast_kernel(const IgemmArgs a, const int tiles_x,
                                                                        const float inv_ohow, const float inv_ow) {
   constexpr int NT = 64 * WP * WF * WK;
@@ -42,6 +42,10 @@ __global__ __launch_bounds__(64 * WP * WF * WK) void igemm_fast_kernel(const Ige
   constexpr int CE = 16 / ES;       // elements per 16-byte chunk
   constexpr int BKE = 4 * CE;       // elements per K step
   constexpr int BP = 64 * WP, BF = 64 * WF, ROWS = BP + BF;
+  // NI = 1: a workgroup owns 32 filters instead of 64 (twice the workgroups for small problems).
+  // The LDS stage keeps its 64 weight rows; the upper 32 are loaded as zeros and never multiplied.
+  static_assert(NI == 2 || WF == 1, "half filter blocks only with one filter wave");
+  constexpr int BFE = NI == 2 ? BF : 32;  // filters per workgroup
   constexpr int R64 = ROWS / 64;    // 64-row groups per K step
   constexpr int LPT = KS * R64;     // 16-byte loads per thread per stage
   constexpr int STAGE = KS * ROWS * kRow;
@@ -61,7 +65,7 @@ __global__ __launch_bounds__(64 * WP * WF * WK) void igemm_fast_kernel(const Ige
   const int P = a.N * a.OH * a.OW;
   const int nk_row = (a.R * a.S * a.C) / BKE;  // K steps of a whole filter row (exact: C % BKE == 0)
   // auxiliary filter blocks walk one tap only
-  const bool aux = a.aux_f0 > 0 && by * BF >= a.aux_f0;
+  const bool aux = a.aux_f0 > 0 && by * BFE >= a.aux_f0;
   const int spt = a.C / BKE;  // K steps per tap
   const int k_begin = aux ? a.aux_tap * spt : 0;
   const int nk = aux ? k_begin + spt : nk_row;  // end of the K walk
@@ -91,13 +95,13 @@ __global__ __launch_bounds__(64 * WP * WF * WK) void igemm_fast_kernel(const Ige
   int wbase[WF];
 #pragma unroll
   for (int g = 0; g < WF; ++g) {
-    const int f = by * BF + r0 + 64 * g;
-    wbase[g] = f < a.F ? (f * (nk_row * BKE) + ck * CE) * ES : -1;
+    const int f = by * BFE + r0 + 64 * g;
+    wbase[g] = (f < a.F && r0 + 64 * g < BFE) ? (f * (nk_row * BKE) + ck * CE) * ES : -1;
   }
 
   // epilogue scale/shift of this lane's output channels: requested now, used at the very end
   EpiScale<OutT> ess;
-  ess.load(lane, by * BF + wf * 64, a.F, a.scale, a.shift);
+  ess.load(lane, by * BFE + wf * 64, a.F, a.scale, a.shift);
 
   // scalar K walk
   int kstep = k_begin, kr = aux ? a.aux_tap / a.S : 0, ks = aux ? a.aux_tap % a.S : 0, kc = 0;
@@ -157,11 +161,11 @@ __global__ __launch_bounds__(64 * WP * WF * WK) void igemm_fast_kernel(const Ige
       for (int kk = 0; kk < 2; ++kk) {
         u32x4 fw[2], fp[2];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) fw[i] = *reinterpret_cast<const u32x4*>(sW + (st * ROWS + i * 32) * kRow + kk * 32);
+        for (int i = 0; i < NI; ++i) fw[i] = *reinterpret_cast<const u32x4*>(sW + (st * ROWS + i * 32) * kRow + kk * 32);
 #pragma unroll
         for (int j = 0; j < 2; ++j) fp[j] = *reinterpret_cast<const u32x4*>(sP + (st * ROWS + j * 32) * kRow + kk * 32);
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < NI; ++i)
 #pragma unroll
           for (int j = 0; j < 2; ++j) Mma<T>::run(fw[i], fp[j], acc[i][j]);
       }
@@ -215,7 +219,7 @@ __global__ __launch_bounds__(64 * WP * WF * WK) void igemm_fast_kernel(const Ige
   const OutT* res = (a.residual && !aux) ? static_cast<const OutT*>(a.residual) + (long long)bz * a.out_bs : nullptr;
   const int fo = aux ? a.aux_f0 : 0;                     // first filter of this output tensor
   const int fend = (aux || a.aux_f0 == 0) ? a.F : a.aux_f0;  // one past its last filter
-  tile_reduce_store<OutT, WK>(acc, smem + wpos * kTileBytes, wk, lane, rowoff, by * BF + wf * 64 - fo, fend - fo, ess, res, out,
+  tile_reduce_store<OutT, WK, NI>(acc, smem + wpos * kTileBytes, wk, lane, rowoff, by * BFE + wf * 64 - fo, fend - fo, ess, res, out,
                               aux ? a.aux_relu : a.relu);
 }
 
@@ -225,15 +229,15 @@ template <typename T> constexpr const char* tn();
 template <> constexpr const char* tn<half_t>() { return "f16"; }
 template <> constexpr const char* tn<float>() { return "f32"; }
 
-template <typename T, typename OutT, int WP, int WF, int WK, int KS>
+template <typename T, typename OutT, int WP, int WF, int WK, int KS, int NI = 2>
 void launch_fast_cfg(const IgemmArgs& a, hipStream_t s) {
-  constexpr int BP = 64 * WP, BF = 64 * WF;
+  constexpr int BP = 64 * WP, BF = 64 * WF, BFE = NI == 2 ? BF : 32;
   constexpr int stage2 = 2 * KS * (BP + BF) * kRow;
   constexpr int epi = WP * WF * kTileBytes;
   constexpr int smem = stage2 > epi ? stage2 : epi;
   static const std::string tag = std::string("igemm_fast<") + tn<T>() + "," + tn<OutT>() + "," + std::to_string(WP) + "," +
-                                 std::to_string(WF) + "," + std::to_string(WK) + "," + std::to_string(KS) + ">";
-  auto kern = igemm_fast_kernel<T, OutT, WP, WF, WK, KS>;
+                                 std::to_string(WF) + "," + std::to_string(WK) + "," + std::to_string(KS) + (NI == 1 ? ",half>" : ">");
+  auto kern = igemm_fast_kernel<T, OutT, WP, WF, WK, KS, NI>;
   static const bool attr_set = [&] {
     NNCV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
     return true;
@@ -246,7 +250,7 @@ void launch_fast_cfg(const IgemmArgs& a, hipStream_t s) {
                        sizeof(OutT) * (double)P * a.F * a.batch * (a.residual ? 2 : 1);
   ProfScope prof(tag.c_str(), flops, bytes, s);
   const int tiles_x = (P + BP - 1) / BP;
-  dim3 grid((tiles_x + kXcds - 1) / kXcds * kXcds, (a.F + BF - 1) / BF, a.batch);
+  dim3 grid((tiles_x + kXcds - 1) / kXcds * kXcds, (a.F + BFE - 1) / BFE, a.batch);
   hipLaunchKernelGGL(kern, grid, dim3(64 * WP * WF * WK), smem, s, a, tiles_x, 1.0f / (float)(a.OH * a.OW), 1.0f / (float)a.OW);
 }
 
@@ -265,12 +269,14 @@ void launch_fast_typed(const IgemmArgs& a, hipStream_t s) {
     if (a.F % 128 == 0 && blocks(128, 128) >= 256) pick = 1;
     else if (a.F <= 64 && blocks(256, 64) >= 256) pick = 2;
     else if (blocks(128, 64) >= 256) pick = 3;
-    else pick = 4;
+    else if (blocks(64, 64) >= 128 || a.F % 32 != 0) pick = 4;
+    else pick = 5;  // fewer than 128 workgroups of 64x64: halve the filter blocks
   }
   switch (pick) {
     case 1: launch_fast_cfg<T, OutT, 2, 2, 1, 1>(a, s); break;
     case 2: launch_fast_cfg<T, OutT, 4, 1, 1, 1>(a, s); break;
     case 3: launch_fast_cfg<T, OutT, 2, 1, 2, 2>(a, s); break;
+    case 5: launch_fast_cfg<T, OutT, 1, 1, 4, 4, 1>(a, s); break;
     default: launch_fast_cfg<T, OutT, 1, 1, 4, 4>(a, s); break;
   }
 }

@@ -68,7 +68,7 @@ struct PatchCfg {
   static constexpr int cap = PatchCap<WS>::pix;
   static constexpr int patch_bytes = cap * kPitch;
   static constexpr int load_bytes = patch_bytes + NT * 16;  // + one dump slot per thread
-  static constexpr int tile_bytes = WS * kTileBytes;
+  static constexpr int tile_bytes = WS * WK * kTileBytes;  // one copy per K group
   static constexpr int smem = load_bytes > tile_bytes ? load_bytes : tile_bytes;
 };
 
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   }
   __syncthreads();  // every wave is done with the patch: LDS becomes the output tiles
 
-  tile_reduce_store<OutT, WK, NI>(acc, smem + ws * kTileBytes, wk, lane, obase, f0blk, a.F, ess,
+  tile_reduce_store<OutT, WK, NI>(acc, smem + ws * WK * kTileBytes, wk, lane, obase, f0blk, a.F, ess,
                               static_cast<const OutT*>(a.residual), static_cast<OutT*>(a.out), a.relu);
 }
 

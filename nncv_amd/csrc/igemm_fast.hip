@@ -219,7 +219,7 @@ __global__ __launch_bounds__(64 * WP * WF * WK) void igemm_fast_kernel(const Ige
   const OutT* res = (a.residual && !aux) ? static_cast<const OutT*>(a.residual) + (long long)bz * a.out_bs : nullptr;
   const int fo = aux ? a.aux_f0 : 0;                     // first filter of this output tensor
   const int fend = (aux || a.aux_f0 == 0) ? a.F : a.aux_f0;  // one past its last filter
-  tile_reduce_store<OutT, WK, NI>(acc, smem + wpos * kTileBytes, wk, lane, rowoff, by * BFE + wf * 64 - fo, fend - fo, ess, res, out,
+  tile_reduce_store<OutT, WK, NI>(acc, smem + wpos * WK * kTileBytes, wk, lane, rowoff, by * BFE + wf * 64 - fo, fend - fo, ess, res, out,
                               aux ? a.aux_relu : a.relu);
 }
 
@@ -233,7 +233,7 @@ template <typename T, typename OutT, int WP, int WF, int WK, int KS, int NI = 2>
 void launch_fast_cfg(const IgemmArgs& a, hipStream_t s) {
   constexpr int BP = 64 * WP, BF = 64 * WF, BFE = NI == 2 ? BF : 32;
   constexpr int stage2 = 2 * KS * (BP + BF) * kRow;
-  constexpr int epi = WP * WF * kTileBytes;
+  constexpr int epi = WP * WF * WK * kTileBytes;  // one output-tile copy per K group
   constexpr int smem = stage2 > epi ? stage2 : epi;
   static const std::string tag = std::string("igemm_fast<") + tn<T>() + "," + tn<OutT>() + "," + std::to_string(WP) + "," +
                                  std::to_string(WF) + "," + std::to_string(WK) + "," + std::to_string(KS) + (NI == 1 ? ",half>" : ">");

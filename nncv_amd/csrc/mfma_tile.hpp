@@ -53,15 +53,15 @@ __device__ __forceinline__ int fast_div(int x, int d, float inv, int* rem) {
 // Reduction + epilogue of one 64 (pixel slots) x 64 (channels) output tile that NG waves ("K
 // groups") hold partial sums of, acc[i][j] = channels 32i.. x slots 32j.. in the MFMA layout
 // (lane: slot l%32, channels 8q + 4*(l/32) + e).
-//   1. In NG rounds the groups add their accumulators into one fp32 LDS tile [slot][channel]
-//      (group 0 writes, the others read-add-write; a barrier between rounds).
-//   2. Each group then takes 64/NG of the tile's rows and writes them out with 8 (fp16) / 16
+//   1. Every group writes its accumulators into its own fp32 LDS copy of the tile [slot][channel]
+//      (NG copies, kTileBytes apart), all at once, then one barrier.
+//   2. Each group then takes 64/NG of the tile's rows, sums them over the copies and writes them out with 8 (fp16) / 16
 //      (fp32) consecutive lanes covering the 64 channels of one pixel, so residual reads and
 //      stores are whole 128/256-byte rows.  BN scale/shift, residual add and ReLU are applied in
 //      fp32 on the way out: one rounding.  The scale/shift values a lane needs there are loaded
 //      by EpiScale at kernel start, long before they are used.
-// Every wave of the workgroup must call tile_reduce_store (it contains NG barriers), after a
-// barrier that freed the LDS region.
+// Every wave of the workgroup must call tile_reduce_store (it contains one barrier), after a
+// barrier that freed the LDS region; `tile` is the first of the NG copies.
 // ---------------------------------------------------------------------------------------------
 constexpr int kTilePitch = 68 * 4;                     // bytes per slot row: 64 floats + 16 pad
 constexpr int kTileBytes = 64 * kTilePitch;
@@ -132,29 +132,30 @@ __device__ __forceinline__ void tile_reduce_store(const floatx16 (&acc)[2][2], u
       rv[it] = *reinterpret_cast<const VO*>(res + off);
     }
   }
+  // every K group writes its partial sums into its own copy of the tile, at the same time; one
+  // barrier; the rows are summed over the NG copies on the way out
+  unsigned char* mine = tile + g * kTileBytes;
 #pragma unroll
-  for (int round = 0; round < NG; ++round) {
-    if (g == round) {
+  for (int j = 0; j < 2; ++j)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+    for (int i = 0; i < NI; ++i)
 #pragma unroll
-        for (int i = 0; i < NI; ++i)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            floatx4* p = reinterpret_cast<floatx4*>(tile + (j * 32 + lrow) * kTilePitch + (i * 32 + 8 * q + 4 * lchunk) * 4);
-            floatx4 y = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-            if (round > 0) y += *p;
-            *p = y;
-          }
-    }
-    __syncthreads();
-  }
+      for (int q = 0; q < 4; ++q) {
+        floatx4* p = reinterpret_cast<floatx4*>(mine + (j * 32 + lrow) * kTilePitch + (i * 32 + 8 * q + 4 * lchunk) * 4);
+        *p = floatx4{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+      }
+  __syncthreads();
   floatx4 v[NIT][FPL / 4];
 #pragma unroll
   for (int it = 0; it < NIT; ++it) {
     const int row = g * (64 / NG) + it * RPI + lane / LPR;
 #pragma unroll
-    for (int q = 0; q < FPL / 4; ++q) v[it][q] = *reinterpret_cast<const floatx4*>(tile + row * kTilePitch + fc * 4 + q * 16);
+    for (int q = 0; q < FPL / 4; ++q) {
+      floatx4 sum = *reinterpret_cast<const floatx4*>(tile + row * kTilePitch + fc * 4 + q * 16);
+#pragma unroll
+      for (int k = 1; k < NG; ++k) sum += *reinterpret_cast<const floatx4*>(tile + k * kTileBytes + row * kTilePitch + fc * 4 + q * 16);
+      v[it][q] = sum;
+    }
   }
 #pragma unroll
   for (int it = 0; it < NIT; ++it) {

@@ -115,6 +115,15 @@ int nncv_hip_conv_time(nncv_hip_conv* c, const void* in, int N, int H, int W, co
                        void* stream, float* avg_us);
 
 /* C += A.B, fp32 row-major, DEVICE pointers (K and N multiples of 4). */
+/* Activation arena planner: "greedy by size" offset calculation of arXiv 2001.03288 sec. 5.2, the
+ * algorithm of the reference's MemSolver (src/nncv/compiler/Optimizer/MemSolver.cpp:15-47; known
+ * answer tests/MemSolver/test.cpp:17-37 = 124). Tensor i is live during operators
+ * first_op[i]..last_op[i] (inclusive) and needs bytes[i]; offsets[i] receives its place in one
+ * allocation whose size is returned (~0 on error). Host-only, needs no device. The ResNet-18
+ * workspace of this library is laid out with it. */
+unsigned long long nncv_hip_plan_arena(int n, const int* first_op, const int* last_op, const unsigned long long* bytes,
+                                       unsigned long long align, unsigned long long* offsets);
+
 int nncv_hip_matmul_f32(const float* A, const float* B, float* C, int M, int N, int K, void* stream);
 
 /* Winograd F(4x4,3x3) stages on DEVICE buffers (layouts: U[36][F][C], V[36][tiles][C], M[36][tiles][F],

@@ -36,7 +36,7 @@ EXPORTS = [
     "nncv_hip_resnet18_create", "nncv_hip_resnet18_destroy", "nncv_hip_resnet18_forward",
     "nncv_hip_resnet18_forward_tap",
     "nncv_hip_conv_create", "nncv_hip_conv_destroy", "nncv_hip_conv_algo", "nncv_hip_conv_forward", "nncv_hip_conv_time",
-    "nncv_hip_matmul_f32", "nncv_hip_wino43_filter", "nncv_hip_wino43_input", "nncv_hip_wino43_gemm",
+    "nncv_hip_plan_arena", "nncv_hip_matmul_f32", "nncv_hip_wino43_filter", "nncv_hip_wino43_input", "nncv_hip_wino43_gemm",
     "nncv_hip_wino43_output", "nncv_hip_maxpool3x3s2", "nncv_hip_global_avgpool",
 ]
 
@@ -81,6 +81,8 @@ def lib():
         L.nncv_hip_conv_forward.argtypes = [vp, vp, i, i, i, i, vp, vp, vp]
         L.nncv_hip_conv_time.argtypes = [vp, vp, i, i, i, vp, vp, i, vp, P(ctypes.c_float)]
         L.nncv_hip_matmul_f32.argtypes = [vp, vp, vp, i, i, i, vp]
+        L.nncv_hip_plan_arena.argtypes = [i, P(i), P(i), P(ctypes.c_uint64), ctypes.c_uint64, P(ctypes.c_uint64)]
+        L.nncv_hip_plan_arena.restype = ctypes.c_uint64
         L.nncv_hip_wino43_filter.argtypes = [i, vp, vp, i, i, vp]
         L.nncv_hip_wino43_input.argtypes = [i, vp, i, vp, i, i, i, i, i, vp]
         L.nncv_hip_wino43_gemm.argtypes = [i, vp, vp, vp, i64, i, i, vp]
@@ -171,3 +173,16 @@ def batch_nchw_conv(x_padded, w, out):
     lib()._mlir_ciface_batch_nchw_conv(ctypes.byref(res), ctypes.byref(mi), ctypes.byref(mw), ctypes.byref(mo))
     assert res.aligned == mo.aligned
     return out
+
+
+def plan_arena(lives, align=1):
+    """lives: [(first_op, last_op, bytes)] -> (total, [offsets]) by nncv_hip_plan_arena."""
+    n = len(lives)
+    first = (ctypes.c_int * n)(*[l[0] for l in lives])
+    last = (ctypes.c_int * n)(*[l[1] for l in lives])
+    size = (ctypes.c_uint64 * n)(*[l[2] for l in lives])
+    off = (ctypes.c_uint64 * n)()
+    total = lib().nncv_hip_plan_arena(n, first, last, size, align, off)
+    if total == 2 ** 64 - 1:
+        raise NncvHipError(lib().nncv_hip_last_error().decode())
+    return int(total), [int(o) for o in off]

@@ -1,0 +1,26 @@
+// Offsets of the intermediate tensors of one forward pass inside a single device allocation.
+//
+// "Greedy by Size for Offset Calculation" of Pisarchyk & Lee, Efficient Memory Management for Deep
+// Neural Net Inference (arXiv 2001.03288, section 5.2) — the algorithm of the reference's
+// MemSolver::solve (src/nncv/compiler/Optimizer/MemSolver.cpp:15-47), which the reference has but
+// never wires into a pipeline.  Tensors are placed in non-increasing order of size; each goes into
+// the smallest gap, between already placed tensors whose lifetimes overlap its own, that holds
+// it, or behind the last of them.  Unlike the reference, the list of placed tensors is kept
+// sorted by offset, as the paper requires for the gap scan to be meaningful.
+#pragma once
+#include <cstddef>
+#include <vector>
+
+namespace nncv_hip {
+
+struct TensorLife {
+  int first_op, last_op;  // inclusive range of operator indices during which the tensor is live
+  size_t bytes;
+  size_t offset;          // out
+};
+
+// Fills `offset` of every record (input order is kept) and returns the arena size.  Offsets and
+// sizes are rounded up to `align` bytes (a power of two; 1 = none).
+size_t plan_offsets(std::vector<TensorLife>& tensors, size_t align);
+
+}  // namespace nncv_hip

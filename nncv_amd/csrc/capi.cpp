@@ -6,6 +6,7 @@
 #include <vector>
 
 #include "../../include/nncv_hip.h"
+#include "arena_plan.hpp"
 #include "model.hpp"
 
 using namespace nncv_hip;
@@ -572,6 +573,23 @@ int nncv_hip_conv_time(nncv_hip_conv* c, const void* in, int N, int H, int W, co
     *avg_us = ms * 1000.0f / (float)reps;
     sy.finish();
   });
+}
+
+unsigned long long nncv_hip_plan_arena(int n, const int* first_op, const int* last_op, const unsigned long long* bytes,
+                                       unsigned long long align, unsigned long long* offsets) {
+  unsigned long long total = 0;
+  const int rc = guarded([&] {
+    NNCV_REQUIRE(n >= 0 && (n == 0 || (first_op && last_op && bytes && offsets)), "null argument");
+    NNCV_REQUIRE(align >= 1 && (align & (align - 1)) == 0, "align must be a power of two");
+    std::vector<TensorLife> t((size_t)n);
+    for (int i = 0; i < n; ++i) {
+      NNCV_REQUIRE(first_op[i] <= last_op[i], "a tensor's first operator must not come after its last");
+      t[i] = TensorLife{first_op[i], last_op[i], (size_t)bytes[i], 0};
+    }
+    total = plan_offsets(t, (size_t)align);
+    for (int i = 0; i < n; ++i) offsets[i] = t[i].offset;
+  });
+  return rc == 0 ? total : ~0ull;
 }
 
 int nncv_hip_matmul_f32(const float* A, const float* B, float* C, int M, int N, int K, void* stream) {

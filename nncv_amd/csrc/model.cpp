@@ -1,5 +1,7 @@
 #include "model.hpp"
 
+#include "arena_plan.hpp"
+
 #include <cstring>
 
 namespace nncv_hip {
@@ -251,65 +253,90 @@ ResNet18::ResNet18(const void* params, long long n_elems, int dt, int algo3x3, h
 }
 
 namespace {
+// Workspace layout of one forward pass, planned with plan_offsets (arena_plan.hpp) from the
+// tensors' sizes and the operator range over which each one is live.  Operator numbering: 0 stem
+// convolution, 1 max-pool, then per BasicBlock k: 2+3k conv1, 3+3k shortcut conv, 4+3k conv2,
+// 26 average pool, 27 FC.
 struct Plan {
-  int h1, w1, h2, w2;   // after stem, after maxpool
-  size_t stem_out, act, pooled, conv_ws, total;
+  int h1, w1, h2, w2;            // after stem, after maxpool
+  size_t stem_out, pooled, cws;  // offsets
+  size_t x[9];                   // x[k] = input of block k; x[8] = network body output
+  size_t y1[8], idn[8];
+  size_t total;
 };
 }  // namespace
 
-static Plan make_plan(const ResNet18& m, const ConvLayer& stem, const std::vector<const ConvLayer*>& convs, int dt, int N,
-                      int H, int W) {
-  (void)m;
+static Plan make_plan(const ConvLayer& stem, const std::vector<const ConvLayer*>& c1s, const std::vector<const ConvLayer*>& c2s,
+                      const std::vector<const ConvLayer*>& dss, int dt, int N, int H, int W) {
   Plan p{};
   const size_t es = dtype_size(dt);
   p.h1 = stem.out_h(H); p.w1 = stem.out_w(W);
   p.h2 = (p.h1 + 2 - 3) / 2 + 1; p.w2 = (p.w1 + 2 - 3) / 2 + 1;
-  p.stem_out = align256((size_t)N * p.h1 * p.w1 * 64 * es);
-  p.act = align256((size_t)N * p.h2 * p.w2 * 64 * es);  // largest activation after the pool
-  p.pooled = align256((size_t)N * 512 * es);
-  p.conv_ws = stem.workspace_bytes(N, H, W);
-  int h = p.h2, w = p.w2;
-  for (const ConvLayer* c : convs) {
-    // every conv sees at most the post-pool resolution; sizes only shrink afterwards
-    p.conv_ws = std::max(p.conv_ws, c->workspace_bytes(N, h, w));
+  std::vector<TensorLife> t;
+  auto add = [&](int first, int last, size_t bytes) { t.push_back(TensorLife{first, last, bytes, 0}); return (int)t.size() - 1; };
+  const int i_stem = add(0, 1, (size_t)N * p.h1 * p.w1 * 64 * es);
+  size_t cws = stem.workspace_bytes(N, H, W);
+  int h = p.h2, w = p.w2, ch = 64;
+  int ix[9], iy1[8], iidn[8];
+  ix[0] = add(1, 0, 0);  // last use filled in below
+  const int nb = (int)c1s.size();
+  for (int k = 0; k < nb; ++k) {
+    const int o = 2 + 3 * k;
+    const int oh = c1s[k]->out_h(h), ow = c1s[k]->out_w(w), f = c2s[k]->desc().F;
+    cws = std::max(cws, c1s[k]->workspace_bytes(N, h, w));
+    cws = std::max(cws, c2s[k]->workspace_bytes(N, oh, ow));
+    if (dss[k]) cws = std::max(cws, dss[k]->workspace_bytes(N, h, w));
+    t[ix[k]].bytes = (size_t)N * h * w * ch * es;
+    t[ix[k]].last_op = dss[k] ? o + 1 : o + 2;  // identity shortcuts are read by conv2
+    iy1[k] = add(o, o + 2, (size_t)N * oh * ow * f * es);
+    iidn[k] = dss[k] ? add(o, o + 2, (size_t)N * oh * ow * f * es) : -1;
+    ix[k + 1] = add(o + 2, o + 3, 0);
+    h = oh; w = ow; ch = f;
   }
-  p.total = p.stem_out + 4 * p.act + p.pooled + p.conv_ws + 4096;
+  t[ix[nb]].bytes = (size_t)N * h * w * ch * es;
+  t[ix[nb]].last_op = 26;
+  const int i_pooled = add(26, 27, (size_t)N * 512 * es);
+  const int i_cws = add(0, 27, cws);
+  p.total = plan_offsets(t, 256) + 4096;
+  p.stem_out = t[i_stem].offset; p.pooled = t[i_pooled].offset; p.cws = t[i_cws].offset;
+  for (int k = 0; k <= nb; ++k) p.x[k] = t[ix[k]].offset;
+  for (int k = 0; k < nb; ++k) { p.y1[k] = t[iy1[k]].offset; p.idn[k] = iidn[k] >= 0 ? t[iidn[k]].offset : 0; }
   return p;
 }
 
-size_t ResNet18::workspace_bytes(int N, int H, int W) const {
-  std::vector<const ConvLayer*> convs;
-  for (const Block& b : blocks_) { convs.push_back(b.c1.get()); convs.push_back(b.c2.get()); if (b.ds) convs.push_back(b.ds.get()); }
-  return make_plan(*this, *stem_, convs, dt_, N, H, W).total;
+static Plan plan_of(const ConvLayer& stem, const std::vector<ResNet18::Block>& blocks, int dt, int N, int H, int W) {
+  std::vector<const ConvLayer*> c1s, c2s, dss;
+  for (const ResNet18::Block& b : blocks) { c1s.push_back(b.c1.get()); c2s.push_back(b.c2.get()); dss.push_back(b.ds.get()); }
+  NNCV_REQUIRE(c1s.size() == 8, "ResNet-18 has eight BasicBlocks");
+  return make_plan(stem, c1s, c2s, dss, dt, N, H, W);
 }
+
+size_t ResNet18::workspace_bytes(int N, int H, int W) const { return plan_of(*stem_, blocks_, dt_, N, H, W).total; }
 
 void ResNet18::forward(const void* src, int N, int H, int W, void* logits, void* ws, hipStream_t s, int tap_stage,
                        void* tap) const {
   NNCV_REQUIRE(N > 0 && H >= 32 && W >= 32, "ResNet-18: input must be at least 32x32");
-  std::vector<const ConvLayer*> convs;
-  for (const Block& b : blocks_) { convs.push_back(b.c1.get()); convs.push_back(b.c2.get()); if (b.ds) convs.push_back(b.ds.get()); }
-  const Plan p = make_plan(*this, *stem_, convs, dt_, N, H, W);
+  const Plan p = plan_of(*stem_, blocks_, dt_, N, H, W);
   char* base = static_cast<char*>(ws);
-  char* stem_out = base; base += p.stem_out;
-  char* act[4];
-  for (int i = 0; i < 4; ++i) { act[i] = base; base += p.act; }
-  char* pooled = base; base += p.pooled;
-  char* cws = base;
+  char* stem_out = base + p.stem_out;
+  char* pooled = base + p.pooled;
+  char* cws = base + p.cws;
+  char* x0 = base + p.x[0];
 
   // stem: conv7x7 s2 + BN + ReLU (Res18.mlir:118-142), then maxpool 3x3 s2 (:144-151)
-  if (!stem_->forward_stem_pool(src, N, H, W, act[0], s)) {
+  if (!stem_->forward_stem_pool(src, N, H, W, x0, s)) {
     stem_->forward(src, N, H, W, nullptr, stem_out, cws, s);
-    launch_maxpool3x3s2_nhwc(stem_out, act[0], dt_, N, p.h1, p.w1, 64, s);
+    launch_maxpool3x3s2_nhwc(stem_out, x0, dt_, N, p.h1, p.w1, 64, s);
   }
-  int cur = 0, h = p.h2, w = p.w2, nblk = 0, ch = 64;
+  int h = p.h2, w = p.w2, nblk = 0, ch = 64;
   const size_t es = dtype_size(dt_);
-  if (tap_stage == 0) NNCV_HIP_CHECK(hipMemcpyAsync(tap, act[0], (size_t)N * h * w * 64 * es, hipMemcpyDeviceToDevice, s));
+  if (tap_stage == 0) NNCV_HIP_CHECK(hipMemcpyAsync(tap, x0, (size_t)N * h * w * 64 * es, hipMemcpyDeviceToDevice, s));
   for (const Block& b : blocks_) {
     // BasicBlock (Res18.mlir:152-203, :255-320): y = relu(bn2(conv2(relu(bn1(conv1(x))))) + shortcut(x))
-    char* x = act[cur];
-    char* y1 = act[(cur + 1) & 3];
-    char* idn = act[(cur + 2) & 3];
-    char* y2 = act[(cur + 3) & 3];
+    char* x = base + p.x[nblk];
+    char* y1 = base + p.y1[nblk];
+    char* idn = base + p.idn[nblk];
+    char* y2 = base + p.x[nblk + 1];
     const int oh = b.c1->out_h(h), ow = b.c1->out_w(w);
     const void* shortcut = x;
     if (b.ds && b.c1->has_shortcut()) {
@@ -323,20 +350,20 @@ void ResNet18::forward(const void* src, int N, int H, int W, void* logits, void*
       }
     }
     b.c2->forward(y1, N, oh, ow, shortcut, y2, cws, s);
-    cur = (cur + 3) & 3;
     h = oh; w = ow;
     ch = b.c2->desc().F;
     ++nblk;
     if (nblk % 2 == 0 && tap_stage == nblk / 2)
-      NNCV_HIP_CHECK(hipMemcpyAsync(tap, act[cur], (size_t)N * h * w * ch * es, hipMemcpyDeviceToDevice, s));
+      NNCV_HIP_CHECK(hipMemcpyAsync(tap, y2, (size_t)N * h * w * ch * es, hipMemcpyDeviceToDevice, s));
   }
+  char* body_out = base + p.x[8];
   // head: global average pool (sum, one divide), FC with bias (Res18.mlir:609-628)
   static const bool split_head = getenv("NNCV_HIP_NO_HEAD_FUSION") != nullptr;
   if (!split_head) {
-    launch_avgpool_fc(act[cur], fc_w_.get(), fc_b_.as<float>(), static_cast<float*>(logits), dt_, N, h * w, 512, 1000, s);
+    launch_avgpool_fc(body_out, fc_w_.get(), fc_b_.as<float>(), static_cast<float*>(logits), dt_, N, h * w, 512, 1000, s);
     return;
   }
-  launch_global_avgpool_nhwc(act[cur], pooled, dt_, N, h * w, 512, s);
+  launch_global_avgpool_nhwc(body_out, pooled, dt_, N, h * w, 512, s);
   IgemmArgs a{};
   a.in = pooled; a.wt = fc_w_.get(); a.out = logits; a.shift = fc_b_.as<float>();
   a.N = N; a.H = 1; a.W = 1; a.C = 512; a.F = 1000; a.R = 1; a.S = 1; a.OH = 1; a.OW = 1;

@@ -74,10 +74,11 @@ class ResNet18 {
   void forward(const void* src, int N, int H, int W, void* logits, void* ws, hipStream_t s, int tap_stage = -1,
                void* tap = nullptr) const;
 
- private:
   struct Block {
     std::unique_ptr<ConvLayer> c1, c2, ds;
   };
+
+ private:
   int dt_;
   std::unique_ptr<ConvLayer> stem_;
   std::vector<Block> blocks_;

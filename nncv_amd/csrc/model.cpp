@@ -274,8 +274,10 @@ static Plan make_plan(const ConvLayer& stem, const std::vector<const ConvLayer*>
   p.h2 = (p.h1 + 2 - 3) / 2 + 1; p.w2 = (p.w1 + 2 - 3) / 2 + 1;
   std::vector<TensorLife> t;
   auto add = [&](int first, int last, size_t bytes) { t.push_back(TensorLife{first, last, bytes, 0}); return (int)t.size() - 1; };
-  const int i_stem = add(0, 1, (size_t)N * p.h1 * p.w1 * 64 * es);
-  size_t cws = stem.workspace_bytes(N, H, W);
+  // the fused stem kernel writes the pooled tensor directly: no stem output, no packed image
+  const bool fused_stem = stem.desc().relu && stem_pool_applicable(dt, N, H, W, stem.desc().F);
+  const int i_stem = add(0, 1, fused_stem ? 0 : (size_t)N * p.h1 * p.w1 * 64 * es);
+  size_t cws = fused_stem ? 0 : stem.workspace_bytes(N, H, W);
   int h = p.h2, w = p.w2, ch = 64;
   int ix[9], iy1[8], iidn[8];
   ix[0] = add(1, 0, 0);  // last use filled in below

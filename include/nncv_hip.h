@@ -115,6 +115,19 @@ int nncv_hip_conv_time(nncv_hip_conv* c, const void* in, int N, int H, int W, co
                        void* stream, float* avg_us);
 
 /* C += A.B, fp32 row-major, DEVICE pointers (K and N multiples of 4). */
+/* The reference driver's image preparation and top-1 scan on the device
+ * (examples/Res18/main.cpp:38-77 and :103-111).
+ * preprocess: hwc_u8 is a DEVICE [N,H,W,channels] 8-bit image (channels 3 or 4, the first three
+ * used); nchw_out receives [N,3,H,W] of `dtype` with x = ((u8 / 255.f) - mean[c]) / std[c], mean =
+ * {0.485, 0.456, 0.406}, std = {0.229, 0.224, 0.225}, fp32 arithmetic in that order.
+ * argmax: top1[n] = the first index of the largest of logits[n][0..F) that exceeds -100 (0 if none;
+ * NaNs never win) -- the driver's loop. classify_u8 = preprocess + forward + argmax in one call;
+ * logits [N,1000] fp32 and top1 [N] are DEVICE buffers. */
+int nncv_hip_preprocess_u8(const void* hwc_u8, int N, int H, int W, int channels, int dtype, void* nchw_out, void* stream);
+int nncv_hip_argmax(const float* logits, int N, int F, int* top1, void* stream);
+int nncv_hip_resnet18_classify_u8(nncv_hip_model* m, const void* hwc_u8, int N, int H, int W, int channels, float* logits,
+                                  int* top1, void* stream);
+
 /* Activation arena planner: "greedy by size" offset calculation of arXiv 2001.03288 sec. 5.2, the
  * algorithm of the reference's MemSolver (src/nncv/compiler/Optimizer/MemSolver.cpp:15-47; known
  * answer tests/MemSolver/test.cpp:17-37 = 124). Tensor i is live during operators

@@ -36,7 +36,8 @@ EXPORTS = [
     "nncv_hip_resnet18_create", "nncv_hip_resnet18_destroy", "nncv_hip_resnet18_forward",
     "nncv_hip_resnet18_forward_tap",
     "nncv_hip_conv_create", "nncv_hip_conv_destroy", "nncv_hip_conv_algo", "nncv_hip_conv_forward", "nncv_hip_conv_time",
-    "nncv_hip_plan_arena", "nncv_hip_matmul_f32", "nncv_hip_wino43_filter", "nncv_hip_wino43_input", "nncv_hip_wino43_gemm",
+    "nncv_hip_plan_arena", "nncv_hip_preprocess_u8", "nncv_hip_argmax", "nncv_hip_resnet18_classify_u8",
+    "nncv_hip_matmul_f32", "nncv_hip_wino43_filter", "nncv_hip_wino43_input", "nncv_hip_wino43_gemm",
     "nncv_hip_wino43_output", "nncv_hip_maxpool3x3s2", "nncv_hip_global_avgpool",
 ]
 
@@ -83,6 +84,9 @@ def lib():
         L.nncv_hip_matmul_f32.argtypes = [vp, vp, vp, i, i, i, vp]
         L.nncv_hip_plan_arena.argtypes = [i, P(i), P(i), P(ctypes.c_uint64), ctypes.c_uint64, P(ctypes.c_uint64)]
         L.nncv_hip_plan_arena.restype = ctypes.c_uint64
+        L.nncv_hip_preprocess_u8.argtypes = [vp, i, i, i, i, i, vp, vp]
+        L.nncv_hip_argmax.argtypes = [vp, i, i, vp, vp]
+        L.nncv_hip_resnet18_classify_u8.argtypes = [vp, vp, i, i, i, i, vp, vp, vp]
         L.nncv_hip_wino43_filter.argtypes = [i, vp, vp, i, i, vp]
         L.nncv_hip_wino43_input.argtypes = [i, vp, i, vp, i, i, i, i, i, vp]
         L.nncv_hip_wino43_gemm.argtypes = [i, vp, vp, vp, i64, i, i, vp]

@@ -463,6 +463,45 @@ int nncv_hip_resnet18_forward(nncv_hip_model* m, const void* src, int N, int H, 
   });
 }
 
+int nncv_hip_preprocess_u8(const void* hwc_u8, int N, int H, int W, int channels, int dtype, void* nchw_out, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(hwc_u8 && nchw_out, "null argument");
+    NNCV_REQUIRE(dtype == kF32 || dtype == kF16, "dtype must be 1 (fp32) or 2 (fp16)");
+    Context::get().init(-1);
+    Sync sy(stream);
+    launch_preprocess_u8(hwc_u8, nchw_out, dtype, N, H, W, channels, sy.s);
+    sy.finish();
+  });
+}
+
+int nncv_hip_argmax(const float* logits, int N, int F, int* top1, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(logits && top1, "null argument");
+    Context::get().init(-1);
+    Sync sy(stream);
+    launch_argmax_rows(logits, top1, N, F, sy.s);
+    sy.finish();
+  });
+}
+
+int nncv_hip_resnet18_classify_u8(nncv_hip_model* m, const void* hwc_u8, int N, int H, int W, int channels, float* logits,
+                                  int* top1, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(m && m->m && hwc_u8 && logits && top1, "null argument");
+    Context& ctx = Context::get();
+    Sync sy(stream);
+    const int dt = m->m->dtype();
+    const size_t in_b = align256((size_t)N * 3 * H * W * dtype_size(dt));
+    const size_t wsb = m->m->workspace_bytes(N, H, W);
+    ctx.arena.reserve(in_b + wsb + 2048, sy.s);
+    void* x = ctx.arena.take(in_b);
+    launch_preprocess_u8(hwc_u8, x, dt, N, H, W, channels, sy.s);
+    m->m->forward(x, N, H, W, logits, ctx.arena.take(wsb), sy.s);
+    launch_argmax_rows(logits, top1, N, 1000, sy.s);
+    sy.finish();
+  });
+}
+
 int nncv_hip_resnet18_forward_tap(nncv_hip_model* m, const void* src, int N, int H, int W, float* logits, int stage,
                                   void* tap, void* stream) {
   return guarded([&] {

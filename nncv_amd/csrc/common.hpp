@@ -134,6 +134,9 @@ void launch_global_avgpool_nhwc(const void* in, void* out, int dt, int N, int HW
 // head: global average pool + fully connected layer with bias, fp32 logits (C must be 512)
 void launch_avgpool_fc(const void* in, const void* w, const float* bias, float* out, int dt, int N, int HW, int C, int F,
                        hipStream_t s);
+// the reference driver's image preparation (u8 HWC -> normalised NCHW) and top-1 scan, on the device
+void launch_preprocess_u8(const void* src, void* dst, int dst_dt, int N, int H, int W, int channels, hipStream_t s);
+void launch_argmax_rows(const float* x, int* idx, int N, int F, hipStream_t s);
 // generic strided copy/cast between layouts: dst[n,c,h,w] (+)= (c < Csrc ? src[n,c,h,w] : 0) for c < Cdst
 void launch_relayout(const void* src, int src_dt, Strides4 ss, void* dst, int dst_dt, Strides4 ds, int N,
                      int Csrc, int Cdst, int H, int W, bool accumulate, hipStream_t s);

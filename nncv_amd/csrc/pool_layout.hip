@@ -193,6 +193,76 @@ void launch_avgpool_fc(const void* in, const void* w, const float* bias, float* 
 }
 
 // ---------------------------------------------------------------------------------------------
+// The driver's pre- and post-processing on the device (examples/Res18/main.cpp:38-77, :103-111).
+//   preprocess: 8-bit HWC image (3 or 4 interleaved channels, the first three used) ->
+//     NCHW, x = ((u8 / 255.f) - mean[c]) / std[c] with the driver's constants and its fp32
+//     operation order (two IEEE divisions), stored as fp32 or rounded once to fp16.
+//   argmax: the driver's scan `max = -100; idx = 0; if (v > max) {max = v; idx = i;}` per row:
+//     the FIRST index of the largest value above -100 (NaNs never win, index 0 if nothing does).
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void preprocess_u8_kernel(const unsigned char* __restrict__ src, T* __restrict__ dst, int N,
+                                                            int HW, int channels) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;  // one pixel each
+  if (idx >= (long long)N * HW) return;
+  const int n = (int)(idx / HW), p = (int)(idx - (long long)n * HW);
+  const unsigned char* px = src + idx * channels;
+  const float mean[3] = {0.485f, 0.456f, 0.406f}, sd[3] = {0.229f, 0.224f, 0.225f};
+#pragma unroll
+  for (int c = 0; c < 3; ++c) {
+    const float v = (float)px[c] / 255.f;
+    dst[((long long)n * 3 + c) * HW + p] = (T)((v - mean[c]) / sd[c]);
+  }
+}
+
+void launch_preprocess_u8(const void* src, void* dst, int dst_dt, int N, int H, int W, int channels, hipStream_t s) {
+  NNCV_REQUIRE(channels == 3 || channels == 4, "preprocess: 3 or 4 interleaved channels");
+  const long long work = (long long)N * H * W;
+  const long long grid = (work + 255) / 256;
+  NNCV_REQUIRE(work > 0 && grid < (1ll << 31), "preprocess: bad size");
+  ProfScope prof("preprocess_u8", 0.0, (double)work * (channels + 3.0 * dtype_size(dst_dt)), s);
+  if (dst_dt == kF16)
+    hipLaunchKernelGGL((preprocess_u8_kernel<half_t>), dim3((unsigned)grid), dim3(256), 0, s, (const unsigned char*)src, (half_t*)dst, N, H * W, channels);
+  else
+    hipLaunchKernelGGL((preprocess_u8_kernel<float>), dim3((unsigned)grid), dim3(256), 0, s, (const unsigned char*)src, (float*)dst, N, H * W, channels);
+  NNCV_HIP_CHECK(hipGetLastError());
+}
+
+__global__ __launch_bounds__(256) void argmax_rows_kernel(const float* __restrict__ x, int* __restrict__ idx_out, int F) {
+  __shared__ float smax[4];
+  __shared__ int sidx[4];
+  const float* row = x + (long long)blockIdx.x * F;
+  float best = -100.f;
+  int bi = 0x7fffffff;  // "nothing above -100 yet"
+  for (int i = threadIdx.x; i < F; i += 256) {
+    const float v = row[i];
+    if (v > best) { best = v; bi = i; }  // strided scan: equal values keep the earlier index
+  }
+  // wave, then workgroup: larger value wins, equal values -> smaller index
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) {
+    const float ov = __shfl_xor(best, d);
+    const int oi = __shfl_xor(bi, d);
+    if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) { smax[wave] = best; sidx[wave] = bi; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w)
+      if (smax[w] > best || (smax[w] == best && sidx[w] < bi)) { best = smax[w]; bi = sidx[w]; }
+    idx_out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+  }
+}
+
+void launch_argmax_rows(const float* x, int* idx, int N, int F, hipStream_t s) {
+  NNCV_REQUIRE(N > 0 && F > 0, "argmax: empty");
+  ProfScope prof("argmax_rows", 0.0, 4.0 * N * (F + 1.0), s);
+  hipLaunchKernelGGL(argmax_rows_kernel, dim3(N), dim3(256), 0, s, x, idx, F);
+  NNCV_HIP_CHECK(hipGetLastError());
+}
+
+// ---------------------------------------------------------------------------------------------
 // generic strided relayout / cast, dst (+)= src (operator-level ABI only; not on the ResNet-18 path)
 // ---------------------------------------------------------------------------------------------
 template <typename Ts, typename Td>

@@ -195,6 +195,31 @@ def resnet18_forward(x, params, tap_layer=-1):
     return (y, tap) if tap_layer >= 0 else y
 
 
+# ---- the reference driver's pre- and post-processing (examples/Res18/main.cpp), numpy ----
+def preprocess_u8(img_hwc):
+    """[N,H,W,ch>=3] uint8 -> [N,3,H,W] fp32: x = ((u8 / 255.f) - mean[c]) / std[c], every step in
+    fp32 in the driver's order (main.cpp:38 `(float)data[i] / 255.f`, :57-77 `(v - mean) / std`)."""
+    img = np.asarray(img_hwc)
+    assert img.dtype == np.uint8 and img.ndim == 4 and img.shape[3] >= 3
+    mean = np.array([0.485, 0.456, 0.406], np.float32)
+    std = np.array([0.229, 0.224, 0.225], np.float32)
+    v = img[..., :3].astype(np.float32) / np.float32(255.0)
+    v = (v - mean) / std
+    return np.ascontiguousarray(v.transpose(0, 3, 1, 2)).astype(np.float32)
+
+
+def top1_scan(logits):
+    """The driver's scan (main.cpp:103-111): max = -100.f; idx = 0; strict `>` left to right."""
+    out = []
+    for row in np.asarray(logits, np.float32):
+        best, idx = np.float32(-100.0), 0
+        for i, v in enumerate(row):
+            if v > best:
+                best, idx = v, i
+        out.append(idx)
+    return np.array(out, np.int32)
+
+
 # ---- AVX2/OpenMP restatement of the HostWParallel schedule (hostwparallel.cpp): the timed CPU baseline ----
 _HWP = None
 

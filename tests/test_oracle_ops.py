@@ -185,3 +185,20 @@ def test_hostwparallel_resnet18_matches_scalar_oracle():
     want = oracle.resnet18_forward(x, blob)
     assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
     assert got.argmax(1) == want.argmax(1)
+
+
+def test_driver_preprocess_and_top1_restatements():
+    """The numpy restatements of the driver's image preparation and top-1 scan against a plain
+    per-element Python transcription of the same formulas and against numpy's argmax."""
+    img = np.random.default_rng(1).integers(0, 256, size=(1, 5, 4, 3), dtype=np.uint8)
+    got = oracle.preprocess_u8(img)
+    mean, std = (0.485, 0.456, 0.406), (0.229, 0.224, 0.225)
+    for c in range(3):
+        for y in range(5):
+            for x in range(4):
+                v = np.float32(img[0, y, x, c]) / np.float32(255.0)
+                v = (v - np.float32(mean[c])) / np.float32(std[c])
+                assert got[0, c, y, x] == v
+    z = np.random.default_rng(2).normal(size=(4, 50)).astype(np.float32)
+    assert np.array_equal(oracle.top1_scan(z), z.argmax(1))  # no ties, all above -100
+    assert oracle.top1_scan(np.full((1, 5), -200.0, np.float32))[0] == 0

@@ -86,3 +86,83 @@ def write_resnet18(path, blob, dtype=np.float32):
         tensors.append((name, blob[off:off + k].reshape(shape)))
         off += k
     write(path, tensors, dtype)
+
+
+def load_state_dict(path):
+    """{name: ndarray} from a torch checkpoint (.pt/.pth, loaded with weights_only=True: nothing in
+    the file is executed) or a .safetensors file.  A checkpoint that wraps the tensors in a
+    "state_dict" / "model" entry is unwrapped."""
+    if path.endswith(".safetensors"):
+        from safetensors.numpy import load_file
+        return dict(load_file(path))
+    import torch
+    sd = torch.load(path, map_location="cpu", weights_only=True)
+    for key in ("state_dict", "model"):
+        if isinstance(sd, dict) and key in sd and isinstance(sd[key], dict):
+            sd = sd[key]
+    return {k: v.detach().to(torch.float32).numpy() for k, v in sd.items() if hasattr(v, "detach")}
+
+
+def resnet18_blob_from_state_dict(sd):
+    """Canonical-order flat fp32 blob from a torchvision-style ResNet-18 state_dict.  Every tensor
+    of the table must be present with the table's shape (`num_batches_tracked` and any other extra
+    entry is ignored), so a different architecture fails loudly instead of mis-binding."""
+    from . import resnet18_spec as spec
+    parts = []
+    for name, shape in spec.tensor_table():
+        if name not in sd:
+            raise KeyError("state_dict has no tensor %r" % name)
+        a = np.asarray(sd[name], np.float32)
+        if tuple(a.shape) != tuple(shape):
+            raise ValueError("%s: shape %s, expected %s" % (name, tuple(a.shape), tuple(shape)))
+        parts.append(a.reshape(-1))
+    return np.concatenate(parts)
+
+
+def dump(path, out=None):
+    """The listing MemRefFlatArray::printInfo gives (DataType.hpp:220-228: index and shape per
+    tensor), plus name, element width and the element offset a compiled object would use."""
+    import sys
+    out = out or sys.stdout
+    with open(path, "rb") as f:
+        magic, start, n = HEAD.unpack(f.read(HEAD.size))
+        if magic != MAGIC:
+            raise IOError("%s: bad magic 0x%x" % (path, magic))
+        off = 0
+        for i in range(n):
+            name, dims, *rest = INDEXER.unpack(f.read(INDEXER.size))
+            shape = list(rest[:dims])
+            width = rest[8]
+            numel = int(np.prod(shape, dtype=np.int64)) if dims else 1
+            out.write("idx: %d, shape%s, eleWidth %d, element offset %d, name %s\n"
+                      % (i, shape, width, off, name.split(b"\0", 1)[0].decode()))
+            off += numel
+        out.write("%d tensors, %d elements\n" % (n, off))
+    return off
+
+
+def main(argv=None):
+    """python -m nncv_amd.modelbin dump model.bin
+       python -m nncv_amd.modelbin from-state-dict resnet18.{pt,pth,safetensors} model.bin [--fp16]"""
+    import argparse
+    ap = argparse.ArgumentParser(prog="python -m nncv_amd.modelbin", description=main.__doc__,
+                                 formatter_class=argparse.RawDescriptionHelpFormatter)
+    sub = ap.add_subparsers(dest="cmd", required=True)
+    d = sub.add_parser("dump")
+    d.add_argument("file")
+    c = sub.add_parser("from-state-dict")
+    c.add_argument("checkpoint")
+    c.add_argument("out")
+    c.add_argument("--fp16", action="store_true", help="store IEEE half (eleWidth 2), rounded to nearest even")
+    a = ap.parse_args(argv)
+    if a.cmd == "dump":
+        dump(a.file)
+    else:
+        blob = resnet18_blob_from_state_dict(load_state_dict(a.checkpoint))
+        write_resnet18(a.out, blob, np.float16 if a.fp16 else np.float32)
+        print("wrote %s: %d elements, %s" % (a.out, blob.size, "fp16" if a.fp16 else "fp32"))
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())

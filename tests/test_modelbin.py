@@ -98,3 +98,46 @@ def test_resnet18_table():
     assert off["fc.bias"][0] == 11698112
     assert abs(spec.flops_per_image(224) / 1e9 - 3.628) < 1e-3
     assert abs(spec.flops_per_image(256) / 1e9 - 4.738) < 1e-3
+
+
+def test_producer_from_state_dict_and_dump(tmp_path):
+    """model.bin from a torch checkpoint and from a safetensors file: both equal the blob written
+    directly, fp32 byte for byte and fp16 as one rounding; extra entries are ignored, a wrong shape
+    is refused; the dump lists every tensor with the element offset a compiled object would use."""
+    import io
+    import torch
+    from safetensors.numpy import save_file
+    from nncv_amd import resnet18_spec as spec
+    blob = synth.resnet18_params()
+    sd, off = {}, 0
+    for name, shape in spec.tensor_table():
+        k = spec.numel(shape)
+        sd[name] = blob[off:off + k].reshape(shape).copy()
+        off += k
+    pt, st = str(tmp_path / "r18.pt"), str(tmp_path / "r18.safetensors")
+    tsd = {k: torch.from_numpy(v) for k, v in sd.items()}
+    tsd["bn1.num_batches_tracked"] = torch.tensor(7)
+    torch.save({"state_dict": tsd}, pt)
+    save_file(sd, st)
+    direct = str(tmp_path / "direct.bin")
+    modelbin.write_resnet18(direct, blob)
+    for src in (pt, st):
+        out = str(tmp_path / "out.bin")
+        assert modelbin.main(["from-state-dict", src, out]) == 0
+        assert open(out, "rb").read() == open(direct, "rb").read()
+        out16 = str(tmp_path / "out16.bin")
+        assert modelbin.main(["from-state-dict", src, out16, "--fp16"]) == 0
+        index, data = modelbin.read(out16, np.float16)
+        assert all(w == 2 for _, _, w in index) and np.array_equal(data, blob.astype(np.float16))
+    buf = io.StringIO()
+    assert modelbin.dump(direct, buf) == spec.NUM_ELEMENTS
+    lines = buf.getvalue().splitlines()
+    assert len(lines) == 103 and lines[0].startswith("idx: 0, shape[64, 3, 7, 7], eleWidth 4, element offset 0, name conv1.weight")
+    assert "element offset 9408, name bn1.weight" in lines[1]
+    bad = dict(sd)
+    bad["fc.weight"] = bad["fc.weight"][:, :100]
+    with pytest.raises(ValueError):
+        modelbin.resnet18_blob_from_state_dict(bad)
+    del bad["fc.weight"]
+    with pytest.raises(KeyError):
+        modelbin.resnet18_blob_from_state_dict(bad)

@@ -106,3 +106,11 @@ def test_arena_planner_known_answer_and_validity():
         peak = max(sum(up(l[2]) for l in lives if l[0] <= op <= l[1]) for op in range(40))
         assert total >= peak
         assert total <= sum(up(l[2]) for l in lives)
+
+
+def test_arena_planner_rejects_bad_input():
+    with pytest.raises(abi.NncvHipError):
+        abi.plan_arena([(3, 1, 16)])          # first operator after the last
+    with pytest.raises(abi.NncvHipError):
+        abi.plan_arena([(0, 1, 16)], align=24)  # alignment not a power of two
+    assert abi.plan_arena([]) == (0, [])

@@ -103,3 +103,20 @@ def test_cfg2_single_conv_winograd_vs_direct():
         err = max_rel(got, want)
         print("cfg2 algo", algo, "max_rel", err, flush=True)
         assert err < FP32_MAX_REL
+
+
+def test_conv_time_helper_reports_a_plausible_duration():
+    """nncv_hip_conv_time (the roofline timer of bench.py) leaves the same output as one forward
+    call and reports a per-launch time in a sane range."""
+    import ctypes
+    import torch
+    x = synth.round_fp16(synth.normal(300, (2, 64, 14, 14)))
+    w = synth.round_fp16(synth.normal(301, (64, 64, 3, 3), std=0.05))
+    layer = Conv(abi.F16, w, 1, 1, relu=True)
+    xd = dev(nhwc(x), abi.F16)
+    want = host(layer(xd, abi.NHWC))
+    out = torch.zeros((2, 14, 14, 64), dtype=torch.float16, device="cuda")
+    avg = ctypes.c_float(0.0)
+    abi.check(abi.lib().nncv_hip_conv_time(layer.h, xd.data_ptr(), 2, 14, 14, None, out.data_ptr(), 20, None, ctypes.byref(avg)))
+    assert np.array_equal(out.cpu().numpy(), want)
+    assert 1.0 < avg.value < 1000.0

@@ -97,8 +97,9 @@ int nncv_hip_resnet18_forward_tap(nncv_hip_model* m, const void* src, int N, int
                                   void* tap, void* stream);
 
 typedef struct nncv_hip_conv nncv_hip_conv;
-/* One fused conv + BN + (residual) + ReLU layer. weights: HOST FCHW of `dtype`;
- * bn: HOST gamma, beta, mean, var of `dtype`, each [F], or all NULL. */
+/* One fused conv + BN + (residual) + activation layer. weights: HOST FCHW of `dtype`;
+ * bn: HOST gamma, beta, mean, var of `dtype`, each [F], or all NULL; relu: 0 none, 1 ReLU, or any
+ * other NNCV_HIP_ACT_* code (those run on the implicit-GEMM kernels only). */
 nncv_hip_conv* nncv_hip_conv_create(int dtype, const void* weights, int F, int C, int R, int S, int stride, int pad,
                                     const void* gamma, const void* beta, const void* mean, const void* var, int relu,
                                     int algo);
@@ -150,6 +151,72 @@ int nncv_hip_wino43_output(int dtype, const void* M, void* out, int layout, int 
 /* pooling on DEVICE NHWC tensors */
 int nncv_hip_maxpool3x3s2(int dtype, const void* in, void* out, int N, int H, int W, int C, void* stream);
 int nncv_hip_global_avgpool(int dtype, const void* in, void* out, int N, int H, int W, int C, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Network graphs: the other fixtures of tests/Nets (MobileNetV3.mlir: depthwise convolution,
+ * hard-swish, squeeze-excitation; Yolov5s.mlir: SiLU, concatenation, up-sampling, 5x5 max-pool)
+ * as a list of fused operators over numbered tensors. Tensor 0 is the network input; every other
+ * tensor is the `out` of exactly one operator and is read only by later ones; the `out` of the
+ * last operator is the network output. No counterpart in the reference (its compiler bakes the
+ * graph into code); the operator vocabulary is the fixtures'.
+ * ------------------------------------------------------------------------------------------- */
+#define NNCV_HIP_OP_CONV 1        /* conv_2d_nchw_fchw (+bias) (+BatchNorm) (+ in[1] residual) + act; a Linear layer is K = 1 */
+#define NNCV_HIP_OP_DWCONV 2      /* depthwise_conv_2d_nchw_chw (+bias) (+BatchNorm) + act; K = 3 or 5 */
+#define NNCV_HIP_OP_MAXPOOL 3     /* pooling_nchw_max K x K, -inf halo of `pad` */
+#define NNCV_HIP_OP_GAVGPOOL 4    /* pooling_nchw_sum over the whole image / (H*W) -> [N,C,1,1] */
+#define NNCV_HIP_OP_SCALE 5       /* out = in[0] * in[1], in[1] of shape [N,C,1,1] */
+#define NNCV_HIP_OP_ADD 6         /* out = act(in[0] + in[1]) */
+#define NNCV_HIP_OP_ACT 7         /* out = act(in[0]) */
+#define NNCV_HIP_OP_CONCAT 8      /* out = concat over channels of in[0..3] (unused = -1) */
+#define NNCV_HIP_OP_UPSAMPLE2X 9  /* nearest-neighbour, H and W doubled */
+
+#define NNCV_HIP_ACT_NONE 0
+#define NNCV_HIP_ACT_RELU 1         /* select(x ugt 0, x, 0) */
+#define NNCV_HIP_ACT_HARDSWISH 2    /* (min(relu(x + 3), 6) / 6) * x */
+#define NNCV_HIP_ACT_HARDSIGMOID 3  /* max(0, min(1, (x + 3) / 6)) */
+#define NNCV_HIP_ACT_SILU 4         /* x * (1 / (1 + exp(-x))) */
+#define NNCV_HIP_ACT_SIGMOID 5
+
+typedef struct nncv_hip_graph_op {
+  int32_t kind;
+  int32_t in[4];   /* tensor ids, unused = -1 */
+  int32_t out;     /* tensor id */
+  int32_t F;       /* CONV: filters */
+  int32_t K, stride, pad;
+  int32_t act;
+  float eps;       /* BatchNorm epsilon (used when gamma >= 0) */
+  /* element offsets into the parameter blob, -1 = absent.  w: [F,C,K,K] (DWCONV: [C,1,K,K]);
+   * bias, gamma, beta, mean, var: [F].  y = BN(conv + bias) */
+  int64_t w, bias, gamma, beta, mean, var;
+} nncv_hip_graph_op;
+
+typedef struct nncv_hip_graph nncv_hip_graph;
+/* params: HOST pointer to n_elems elements of `dtype`. Channel counts other than the input's must
+ * be multiples of 8 (fp16) / 4 (fp32). Returns NULL on error (nncv_hip_last_error). */
+nncv_hip_graph* nncv_hip_graph_create(const nncv_hip_graph_op* ops, int n_ops, int in_channels, const void* params,
+                                      int64_t n_elems, int dtype);
+void nncv_hip_graph_destroy(nncv_hip_graph* g);
+/* shape[3] = channels, height, width of the network output for an H x W input */
+int nncv_hip_graph_output_shape(const nncv_hip_graph* g, int H, int W, int* shape);
+/* src: DEVICE NCHW [N,in_channels,H,W] of the graph's dtype; out: DEVICE NCHW fp32 of the output
+ * shape, out_elems = N*C*OH*OW (checked). */
+int nncv_hip_graph_forward(nncv_hip_graph* g, const void* src, int N, int H, int W, float* out, int64_t out_elems,
+                           void* stream);
+/* The operator list of torchvision's MobileNetV3-small as exported in tests/Nets/MobileNetV3.mlir
+ * (parameters in state_dict order without num_batches_tracked). Writes at most `cap` operators,
+ * returns their number; *n_elems receives the parameter count. _mlir_ciface_forward serves this
+ * network too when handed a params memref of that many elements. */
+int nncv_hip_mobilenetv3_small_ops(nncv_hip_graph_op* ops, int cap, int64_t* n_elems);
+
+/* Single operators of the list above on DEVICE NHWC tensors of `dtype` (for parity checks).
+ * dwconv: w is DEVICE [C,1,K,K]; scale / shift DEVICE fp32 [C] or NULL. */
+int nncv_hip_dwconv(int dtype, const void* in, const void* w, const float* scale, const float* shift, void* out, int N, int H,
+                    int W, int C, int K, int stride, int pad, int act, void* stream);
+int nncv_hip_scale_channels(int dtype, const void* x, const void* gate, void* out, int N, int HW, int C, void* stream);
+int nncv_hip_eltwise(int dtype, const void* a, const void* b, void* out, int64_t n, int act, void* stream);
+int nncv_hip_concat_slice(int dtype, const void* x, void* out, int64_t P, int C, int ldo, int c0, void* stream);
+int nncv_hip_upsample2x(int dtype, const void* x, void* out, int N, int H, int W, int C, int ldo, int c0, void* stream);
+int nncv_hip_maxpool(int dtype, const void* in, void* out, int N, int H, int W, int C, int K, int stride, int pad, void* stream);
 
 #ifdef __cplusplus
 }

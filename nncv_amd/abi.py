@@ -39,7 +39,36 @@ EXPORTS = [
     "nncv_hip_plan_arena", "nncv_hip_preprocess_u8", "nncv_hip_argmax", "nncv_hip_resnet18_classify_u8",
     "nncv_hip_matmul_f32", "nncv_hip_wino43_filter", "nncv_hip_wino43_input", "nncv_hip_wino43_gemm",
     "nncv_hip_wino43_output", "nncv_hip_maxpool3x3s2", "nncv_hip_global_avgpool",
+    "nncv_hip_graph_create", "nncv_hip_graph_destroy", "nncv_hip_graph_output_shape", "nncv_hip_graph_forward",
+    "nncv_hip_mobilenetv3_small_ops", "nncv_hip_dwconv", "nncv_hip_scale_channels", "nncv_hip_eltwise",
+    "nncv_hip_concat_slice", "nncv_hip_upsample2x", "nncv_hip_maxpool",
 ]
+
+# operator kinds / activations of nncv_hip_graph_op (include/nncv_hip.h)
+OP_CONV, OP_DWCONV, OP_MAXPOOL, OP_GAVGPOOL, OP_SCALE, OP_ADD, OP_ACT, OP_CONCAT, OP_UPSAMPLE2X = range(1, 10)
+ACT_NONE, ACT_RELU, ACT_HARDSWISH, ACT_HARDSIGMOID, ACT_SILU, ACT_SIGMOID = range(6)
+
+
+class GraphOp(ctypes.Structure):
+    _fields_ = [("kind", ctypes.c_int32), ("inputs", ctypes.c_int32 * 4), ("out", ctypes.c_int32), ("F", ctypes.c_int32),
+                ("K", ctypes.c_int32), ("stride", ctypes.c_int32), ("pad", ctypes.c_int32), ("act", ctypes.c_int32),
+                ("eps", ctypes.c_float), ("w", ctypes.c_int64), ("bias", ctypes.c_int64), ("gamma", ctypes.c_int64),
+                ("beta", ctypes.c_int64), ("mean", ctypes.c_int64), ("var", ctypes.c_int64)]
+
+
+assert ctypes.sizeof(GraphOp) == 96
+
+
+def graph_op(kind, inputs, out, F=0, K=0, stride=1, pad=0, act=ACT_NONE, eps=0.0, w=-1, bias=-1, bn=None):
+    """One nncv_hip_graph_op; bn = (gamma, beta, mean, var) element offsets."""
+    o = GraphOp()
+    o.kind, o.out, o.F, o.K, o.stride, o.pad, o.act, o.eps = kind, out, F, K, stride, pad, act, eps
+    ins = list(inputs) + [-1] * (4 - len(inputs))
+    for k in range(4):
+        o.inputs[k] = ins[k]
+    o.w, o.bias = w, bias
+    o.gamma, o.beta, o.mean, o.var = bn if bn is not None else (-1, -1, -1, -1)
+    return o
 
 _lib = None
 
@@ -93,6 +122,19 @@ def lib():
         L.nncv_hip_wino43_output.argtypes = [i, vp, vp, i, i, i, i, i, vp, vp, vp, i, vp]
         L.nncv_hip_maxpool3x3s2.argtypes = [i, vp, vp, i, i, i, i, vp]
         L.nncv_hip_global_avgpool.argtypes = [i, vp, vp, i, i, i, i, vp]
+        L.nncv_hip_graph_create.argtypes = [P(GraphOp), i, i, vp, i64, i]
+        L.nncv_hip_graph_create.restype = vp
+        L.nncv_hip_graph_destroy.argtypes = [vp]
+        L.nncv_hip_graph_destroy.restype = None
+        L.nncv_hip_graph_output_shape.argtypes = [vp, i, i, P(i)]
+        L.nncv_hip_graph_forward.argtypes = [vp, vp, i, i, i, vp, i64, vp]
+        L.nncv_hip_mobilenetv3_small_ops.argtypes = [P(GraphOp), i, P(i64)]
+        L.nncv_hip_dwconv.argtypes = [i, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, i, vp]
+        L.nncv_hip_scale_channels.argtypes = [i, vp, vp, vp, i, i, i, vp]
+        L.nncv_hip_eltwise.argtypes = [i, vp, vp, vp, i64, i, vp]
+        L.nncv_hip_concat_slice.argtypes = [i, vp, vp, i64, i, i, i, vp]
+        L.nncv_hip_upsample2x.argtypes = [i, vp, vp, i, i, i, i, i, i, vp]
+        L.nncv_hip_maxpool.argtypes = [i, vp, vp, i, i, i, i, i, i, i, vp]
         _lib = L
     return _lib
 
@@ -190,3 +232,29 @@ def plan_arena(lives, align=1):
     if total == 2 ** 64 - 1:
         raise NncvHipError(lib().nncv_hip_last_error().decode())
     return int(total), [int(o) for o in off]
+
+
+def mobilenetv3_small_ops():
+    """-> ([GraphOp], n_elems): the library's built-in operator list of MobileNetV3-small."""
+    n_elems = ctypes.c_int64()
+    n = lib().nncv_hip_mobilenetv3_small_ops(None, 0, ctypes.byref(n_elems))
+    arr = (GraphOp * n)()
+    lib().nncv_hip_mobilenetv3_small_ops(arr, n, ctypes.byref(n_elems))
+    return list(arr), int(n_elems.value)
+
+
+def graph_create(ops, in_channels, params_blob):
+    """nncv_hip_graph_create over a host blob (float32 / float16 numpy array); returns the handle."""
+    dt = F16 if params_blob.dtype == np.float16 else F32
+    arr = (GraphOp * len(ops))(*ops)
+    blob = np.ascontiguousarray(params_blob)
+    h = lib().nncv_hip_graph_create(arr, len(ops), in_channels, blob.ctypes.data, blob.size, dt)
+    if not h:
+        raise NncvHipError(lib().nncv_hip_last_error().decode())
+    return h
+
+
+def graph_output_shape(h, H, W):
+    shp = (ctypes.c_int * 3)()
+    check(lib().nncv_hip_graph_output_shape(h, H, W, shp))
+    return tuple(shp)

@@ -7,6 +7,7 @@
 
 #include "../../include/nncv_hip.h"
 #include "arena_plan.hpp"
+#include "graph.hpp"
 #include "model.hpp"
 
 using namespace nncv_hip;
@@ -195,7 +196,7 @@ ResNet18& cached_model(const void* host, long long n, int dt, hipStream_t s) {
 // instead of 24, which is what batch-1 latency is made of.  The pass contains no memset nodes.
 // NNCV_HIP_GRAPH=0 turns replay off; the event profiler bypasses it.
 struct GraphEntry {
-  const ResNet18* m;
+  const void* m;  // the ResNet18 or Graph object the launches belong to
   const void* src;
   const float* logits;
   int N, H, W;
@@ -214,7 +215,7 @@ void drop_graph(GraphEntry& e) {
   e.exec = nullptr;
   e.graph = nullptr;
 }
-void drop_graphs_of(const ResNet18* m) {
+void drop_graphs_of(const void* m) {
   auto& c = graph_cache();
   for (size_t i = 0; i < c.size();) {
     if (c[i].m == m) {
@@ -226,32 +227,34 @@ void drop_graphs_of(const ResNet18* m) {
   }
 }
 
-void forward_replay(const ResNet18& m, const void* src, int N, int H, int W, float* logits, void* ws, hipStream_t s) {
+// `run` enqueues the whole pass on `s`; `owner` identifies the model it belongs to.
+void replay(const void* owner, const std::function<void()>& run, const void* src, int N, int H, int W, const float* logits, void* ws,
+            hipStream_t s) {
   static const bool use = [] {
     const char* e = getenv("NNCV_HIP_GRAPH");
     return !e || atoi(e) != 0;
   }();
   if (!use || profiler_enabled()) {
-    m.forward(src, N, H, W, logits, ws, s);
+    run();
     return;
   }
   auto& cache = graph_cache();
   GraphEntry* hit = nullptr;
   for (auto& e : cache)
-    if (e.m == &m && e.src == src && e.logits == logits && e.N == N && e.H == H && e.W == W && e.ws == ws && e.s == s) hit = &e;
+    if (e.m == owner && e.src == src && e.logits == logits && e.N == N && e.H == H && e.W == W && e.ws == ws && e.s == s) hit = &e;
   if (!hit) {  // first sighting: run eagerly (this also performs every one-time kernel attribute set-up)
     if (cache.size() >= 16) {
       drop_graph(cache.front());
       cache.erase(cache.begin());
     }
-    cache.push_back(GraphEntry{&m, src, logits, N, H, W, ws, s, nullptr, nullptr});
-    m.forward(src, N, H, W, logits, ws, s);
+    cache.push_back(GraphEntry{owner, src, logits, N, H, W, ws, s, nullptr, nullptr});
+    run();
     return;
   }
   if (!hit->exec) {  // second sighting: capture
     NNCV_HIP_CHECK(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
     try {
-      m.forward(src, N, H, W, logits, ws, s);
+      run();
     } catch (...) {
       hipGraph_t g = nullptr;
       (void)hipStreamEndCapture(s, &g);
@@ -262,6 +265,58 @@ void forward_replay(const ResNet18& m, const void* src, int N, int H, int W, flo
     NNCV_HIP_CHECK(hipGraphInstantiate(&hit->exec, hit->graph, nullptr, nullptr, 0));
   }
   NNCV_HIP_CHECK(hipGraphLaunch(hit->exec, s));
+}
+
+void forward_replay(const ResNet18& m, const void* src, int N, int H, int W, float* logits, void* ws, hipStream_t s) {
+  replay(&m, [&] { m.forward(src, N, H, W, logits, ws, s); }, src, N, H, W, logits, ws, s);
+}
+
+// ---- the MobileNetV3 object behind the handle-less reference ABI ----------------------------
+struct CachedGraph {
+  const void* host_ptr;
+  long long n;
+  int dt;
+  uint64_t fingerprint;
+  std::unique_ptr<Graph> graph;
+};
+std::vector<CachedGraph>& graph_model_cache() {
+  static std::vector<CachedGraph> c;
+  return c;
+}
+long long mobilenetv3_elems() {
+  static const long long n = [] {
+    long long k = 0;
+    (void)mobilenetv3_small_ops(&k);
+    return k;
+  }();
+  return n;
+}
+std::unique_ptr<Graph> build_graph(const GraphOp* ops, int n_ops, int c_in, const void* host, long long n, int dt, hipStream_t s) {
+  DeviceBuffer blob((size_t)n * dtype_size(dt));
+  NNCV_HIP_CHECK(hipMemcpyAsync(blob.get(), host, blob.bytes(), hipMemcpyHostToDevice, s));
+  auto g = std::make_unique<Graph>(ops, n_ops, c_in, blob.get(), n, dt, s);
+  NNCV_HIP_CHECK(hipStreamSynchronize(s));  // the staging blob dies here
+  return g;
+}
+Graph& cached_mobilenetv3(const void* host, long long n, int dt, hipStream_t s) {
+  const uint64_t fp = fingerprint(host, n, dtype_size(dt));
+  auto& cache = graph_model_cache();
+  auto make = [&] {
+    long long k = 0;
+    const std::vector<GraphOp> ops = mobilenetv3_small_ops(&k);
+    return build_graph(ops.data(), (int)ops.size(), 3, host, n, dt, s);
+  };
+  for (auto& e : cache)
+    if (e.host_ptr == host && e.n == n && e.dt == dt) {
+      if (e.fingerprint != fp) {
+        e.graph = make();
+        e.fingerprint = fp;
+      }
+      return *e.graph;
+    }
+  if (cache.size() >= 4) cache.erase(cache.begin());
+  cache.push_back(CachedGraph{host, n, dt, fp, make()});
+  return *cache.back().graph;
 }
 
 void forward_abi(nncv_memref2d* dst, nncv_memref4d* src, void* params, int dt) {
@@ -275,10 +330,15 @@ void forward_abi(nncv_memref2d* dst, nncv_memref4d* src, void* params, int dt) {
   const int N = (int)src->sizes[0], C = (int)src->sizes[1], H = (int)src->sizes[2], W = (int)src->sizes[3];
   NNCV_REQUIRE(C == 3, "forward: input must be [N,3,H,W]");
   const char* blob = static_cast<const char*>(p->aligned) + p->offset * (intptr_t)es;
-  ResNet18& model = cached_model(blob, p->sizes[0], dt, s);
+  // Which network the object is follows from the size of its parameter array: ResNet-18
+  // (tests/Nets/Res18.mlir) or MobileNetV3-small (tests/Nets/MobileNetV3.mlir); both map
+  // [N,3,H,W] to [N,1000].
+  const bool mobilenet = p->sizes[0] == mobilenetv3_elems();
+  ResNet18* model = mobilenet ? nullptr : &cached_model(blob, p->sizes[0], dt, s);
+  Graph* graph = mobilenet ? &cached_mobilenetv3(blob, p->sizes[0], dt, s) : nullptr;
 
   const size_t in_bytes = align256((size_t)N * 3 * H * W * es), out_bytes = align256((size_t)N * 1000 * 4);
-  const size_t ws_bytes = model.workspace_bytes(N, H, W);
+  const size_t ws_bytes = mobilenet ? graph->workspace_bytes(N, H, W) : model->workspace_bytes(N, H, W);
   ctx.arena.reserve(in_bytes + out_bytes + ws_bytes + 1024, s);
   void* d_in = ctx.arena.take(in_bytes);
   float* d_out = static_cast<float*>(ctx.arena.take(out_bytes));
@@ -286,7 +346,8 @@ void forward_abi(nncv_memref2d* dst, nncv_memref4d* src, void* params, int dt) {
   // The reference object assumes identity layout and would misread a strided input
   // (DnnModelLowering.cpp:107-108); strides are honoured here instead.
   upload<4>(src->aligned, src->offset, src->sizes, src->strides, es, d_in, ctx.pin_in, s);
-  model.forward(d_in, N, H, W, d_out, ws, s);
+  if (mobilenet) graph->forward(d_in, N, H, W, d_out, ws, s);
+  else model->forward(d_in, N, H, W, d_out, ws, s);
 
   // MLIR C-interface convention: the callee allocates the result and overwrites *dst.
   void* result = nullptr;
@@ -316,11 +377,15 @@ struct nncv_hip_model_impl {
 struct nncv_hip_conv_impl {
   std::unique_ptr<ConvLayer> c;
 };
+struct nncv_hip_graph_impl {
+  std::unique_ptr<Graph> g;
+};
 
 }  // namespace
 
 struct nncv_hip_model : nncv_hip_model_impl {};
 struct nncv_hip_conv : nncv_hip_conv_impl {};
+struct nncv_hip_graph : nncv_hip_graph_impl {};
 
 extern "C" {
 
@@ -377,7 +442,7 @@ void _mlir_ciface_batch_nchw_conv(nncv_memref4d* res, nncv_memref4d* in, nncv_me
     const size_t ib = align256((size_t)N * C * H * W * 4), fb = align256((size_t)F * C * R * S * 4),
                  ob = align256((size_t)N * F * OH * OW * 4);
     ConvLayer::Desc d;
-    d.dt = kF32; d.C = C; d.F = F; d.R = R; d.S = S; d.stride = stride; d.pad = 0; d.relu = false; d.algo = kAlgoAuto;
+    d.dt = kF32; d.C = C; d.F = F; d.R = R; d.S = S; d.stride = stride; d.pad = 0; d.relu = kActNone; d.algo = kAlgoAuto;
     DeviceBuffer dF(fb);
     upload<4>(filter->aligned, filter->offset, filter->sizes, filter->strides, 4, dF.get(), ctx.pin_in, s);
     ConvLayer layer(d, dF.get(), nullptr, nullptr, nullptr, nullptr, s);
@@ -540,7 +605,7 @@ nncv_hip_conv* nncv_hip_conv_create(int dtype, const void* weights, int F, int C
       g = bn.as<char>();
     }
     ConvLayer::Desc d;
-    d.dt = dtype; d.C = C; d.F = F; d.R = R; d.S = S; d.stride = stride; d.pad = pad; d.relu = relu != 0; d.algo = algo;
+    d.dt = dtype; d.C = C; d.F = F; d.R = R; d.S = S; d.stride = stride; d.pad = pad; d.relu = relu; d.algo = algo;
     h = new nncv_hip_conv();
     try {
       h->c = std::make_unique<ConvLayer>(d, w.get(), g, g ? g + (size_t)F * es : nullptr, g ? g + (size_t)2 * F * es : nullptr,
@@ -707,6 +772,143 @@ int nncv_hip_global_avgpool(int dtype, const void* in, void* out, int N, int H, 
     Context::get().init(-1);
     Sync sy(stream);
     launch_global_avgpool_nhwc(in, out, dtype, N, H * W, C, sy.s);
+    sy.finish();
+  });
+}
+
+// ---------------------------------------------------------------------------------------------
+// Network graphs and their single operators
+// ---------------------------------------------------------------------------------------------
+nncv_hip_graph* nncv_hip_graph_create(const nncv_hip_graph_op* ops, int n_ops, int in_channels, const void* params,
+                                      int64_t n_elems, int dtype) {
+  nncv_hip_graph* h = nullptr;
+  const int rc = guarded([&] {
+    NNCV_REQUIRE(ops && params && n_ops > 0 && n_elems > 0, "null or empty argument");
+    NNCV_REQUIRE(dtype == kF32 || dtype == kF16, "dtype must be 1 (fp32) or 2 (fp16)");
+    Context& ctx = Context::get();
+    ctx.init(-1);
+    h = new nncv_hip_graph();
+    try {
+      h->g = build_graph(ops, n_ops, in_channels, params, n_elems, dtype, ctx.stream());
+    } catch (...) {
+      delete h;
+      h = nullptr;
+      throw;
+    }
+  });
+  return rc == 0 ? h : nullptr;
+}
+
+void nncv_hip_graph_destroy(nncv_hip_graph* g) {
+  if (!g) return;
+  guarded([&] {
+    (void)hipDeviceSynchronize();
+    drop_graphs_of(g->g.get());
+    delete g;
+  });
+}
+
+int nncv_hip_graph_output_shape(const nncv_hip_graph* g, int H, int W, int* shape) {
+  return guarded([&] {
+    NNCV_REQUIRE(g && g->g && shape, "null argument");
+    g->g->output_shape(H, W, &shape[0], &shape[1], &shape[2]);
+  });
+}
+
+int nncv_hip_graph_forward(nncv_hip_graph* g, const void* src, int N, int H, int W, float* out, int64_t out_elems, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(g && g->g && src && out, "null argument");
+    Context& ctx = Context::get();
+    Sync sy(stream);
+    const Graph& gr = *g->g;
+    int C, OH, OW;
+    gr.output_shape(H, W, &C, &OH, &OW);
+    NNCV_REQUIRE(out_elems == (int64_t)N * C * OH * OW, "graph: out_elems does not match the output shape");
+    const size_t wsb = gr.workspace_bytes(N, H, W);
+    ctx.arena.reserve(wsb + 1024, sy.s);
+    void* ws = ctx.arena.take(wsb);
+    replay(&gr, [&] { gr.forward(src, N, H, W, out, ws, sy.s); }, src, N, H, W, out, ws, sy.s);
+    sy.finish();
+  });
+}
+
+int nncv_hip_mobilenetv3_small_ops(nncv_hip_graph_op* ops, int cap, int64_t* n_elems) {
+  long long n = 0;
+  const std::vector<GraphOp> v = mobilenetv3_small_ops(&n);
+  if (n_elems) *n_elems = n;
+  if (ops)
+    for (int i = 0; i < cap && i < (int)v.size(); ++i) ops[i] = v[i];
+  return (int)v.size();
+}
+
+int nncv_hip_dwconv(int dtype, const void* in, const void* w, const float* scale, const float* shift, void* out, int N, int H,
+                    int W, int C, int K, int stride, int pad, int act, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(in && w && out, "null argument");
+    NNCV_REQUIRE(dtype == kF32 || dtype == kF16, "dtype must be 1 (fp32) or 2 (fp16)");
+    NNCV_REQUIRE(K == 3 || K == 5, "dwconv: kernel size must be 3 or 5");
+    NNCV_REQUIRE(N >= 1 && H >= 1 && W >= 1 && C >= 1 && stride >= 1 && pad >= 0 && H + 2 * pad >= K && W + 2 * pad >= K,
+                 "dwconv: bad geometry");
+    Context::get().init(-1);
+    Sync sy(stream);
+    DeviceBuffer wt((size_t)C * K * K * dtype_size(dtype));
+    launch_weight_dw(w, dtype, wt.get(), dtype, C, K, sy.s);
+    DwConvArgs a{};
+    a.in = in; a.wt = wt.get(); a.out = out; a.scale = scale; a.shift = shift;
+    a.N = N; a.H = H; a.W = W; a.C = C; a.K = K; a.stride = stride; a.pad = pad;
+    a.OH = (H + 2 * pad - K) / stride + 1; a.OW = (W + 2 * pad - K) / stride + 1; a.act = act;
+    launch_dwconv(a, dtype, sy.s);
+    NNCV_HIP_CHECK(hipStreamSynchronize(sy.s));  // the re-laid filter dies here
+  });
+}
+
+int nncv_hip_scale_channels(int dtype, const void* x, const void* gate, void* out, int N, int HW, int C, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(x && gate && out, "null argument");
+    Context::get().init(-1);
+    Sync sy(stream);
+    launch_scale_channels(x, gate, out, dtype, N, HW, C, sy.s);
+    sy.finish();
+  });
+}
+
+int nncv_hip_eltwise(int dtype, const void* a, const void* b, void* out, int64_t n, int act, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(a && out && n >= 0, "null argument");
+    NNCV_REQUIRE(act >= kActNone && act <= kActSigmoid, "unknown activation");
+    Context::get().init(-1);
+    Sync sy(stream);
+    launch_eltwise(a, b, out, dtype, n, act, sy.s);
+    sy.finish();
+  });
+}
+
+int nncv_hip_concat_slice(int dtype, const void* x, void* out, int64_t P, int C, int ldo, int c0, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(x && out && P >= 0, "null argument");
+    Context::get().init(-1);
+    Sync sy(stream);
+    launch_concat_slice(x, out, dtype, P, C, ldo, c0, sy.s);
+    sy.finish();
+  });
+}
+
+int nncv_hip_upsample2x(int dtype, const void* x, void* out, int N, int H, int W, int C, int ldo, int c0, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(x && out, "null argument");
+    Context::get().init(-1);
+    Sync sy(stream);
+    launch_upsample2x(x, out, dtype, N, H, W, C, ldo, c0, sy.s);
+    sy.finish();
+  });
+}
+
+int nncv_hip_maxpool(int dtype, const void* in, void* out, int N, int H, int W, int C, int K, int stride, int pad, void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(in && out, "null argument");
+    Context::get().init(-1);
+    Sync sy(stream);
+    launch_maxpool_nhwc(in, out, dtype, N, H, W, C, K, stride, pad, sy.s);
     sy.finish();
   });
 }

@@ -38,6 +38,35 @@ struct Error : std::runtime_error {
   } while (0)
 
 // ---------------------------------------------------------------------------------------------
+// Activations fused into the epilogues, written the way the reference's fixtures spell them
+// (tests/Nets/Res18.mlir:139-141 ReLU; tests/Nets/MobileNetV3.mlir:259-293 hard-swish,
+// :349-379 hard-sigmoid; Yolov5s.mlir SiLU = x * 1/(1+exp(-x))).
+// ---------------------------------------------------------------------------------------------
+enum Act : int { kActNone = 0, kActRelu = 1, kActHardSwish = 2, kActHardSigmoid = 3, kActSilu = 4, kActSigmoid = 5 };
+
+// `arith.cmpf ugt` + select: NaN is kept, everything not greater than zero becomes +0.
+__device__ __forceinline__ float relu_ugt(float x) { return (x <= 0.0f) ? 0.0f : x; }
+
+__device__ __forceinline__ float act_apply(float x, int act) {
+  switch (act) {
+    case kActRelu: return relu_ugt(x);
+    case kActHardSwish: {  // (min(relu(x + 3), 6) / 6) * x ; min is `olt` + select
+      float t = relu_ugt(x + 3.0f);
+      t = t < 6.0f ? t : 6.0f;
+      return (t / 6.0f) * x;
+    }
+    case kActHardSigmoid: {  // max(0, min(1, (x + 3) / 6)) ; `olt(1,t) ? 1 : t` then `ogt(0,m) ? 0 : m`
+      float t = (x + 3.0f) / 6.0f;
+      t = 1.0f < t ? 1.0f : t;
+      return 0.0f > t ? 0.0f : t;
+    }
+    case kActSilu: return x * (1.0f / (1.0f + expf(-x)));
+    case kActSigmoid: return 1.0f / (1.0f + expf(-x));
+    default: return x;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // Optional event timing of every launch (profiler.cpp).  `name` must be a string literal or
 // otherwise outlive the scope; flops / bytes are the ALGORITHMIC work of the launch.
 // ---------------------------------------------------------------------------------------------
@@ -73,7 +102,7 @@ struct IgemmArgs {
   const void* residual;  // same indexing as out, or null
   int N, H, W, C, F, R, S, OH, OW;
   int stride_h, stride_w, pad_h, pad_w;
-  int relu;
+  int relu;    // activation code (enum Act) applied last; 0 none, 1 ReLU
   int ldo;     // out/residual row pitch in elements
   int batch;   // grid.z
   long long in_bs, wt_bs, out_bs;  // batch strides in elements
@@ -157,7 +186,31 @@ void launch_stem_pool(const void* in, const void* wt, const float* scale, const 
                       hipStream_t s);
 // BN fold: scale = gamma / sqrt(var + eps), shift = beta - mean*scale (fp32 out)
 void launch_bn_fold(const void* gamma, const void* beta, const void* mean, const void* var, int dt, float* scale,
-                    float* shift, int C, hipStream_t s);
+                    float* shift, int C, hipStream_t s, float eps = 1e-5f);
+
+// ---------------------------------------------------------------------------------------------
+// Operators of the other network fixtures (MobileNetV3.mlir, Yolov5s.mlir), NHWC, elementwise.hip
+// ---------------------------------------------------------------------------------------------
+// linalg.depthwise_conv_2d_nchw_chw (+ zero halo of `pad`) + scale/shift + activation.
+// wt: [K][K][C] of type dt (launch_weight_dw); K in {3, 5}; C a multiple of the 16-byte vector.
+struct DwConvArgs {
+  const void* in; const void* wt; void* out; const float* scale; const float* shift;
+  int N, H, W, C, K, stride, pad, OH, OW, act;
+};
+void launch_dwconv(const DwConvArgs& a, int dt, hipStream_t s);
+// depthwise weights [C][1][K][K] (or [C][K][K]) -> [K][K][C]
+void launch_weight_dw(const void* w, int w_dt, void* dst, int dst_dt, int C, int K, hipStream_t s);
+// out[n,p,c] = x[n,p,c] * g[n,c]   (squeeze-excitation gate; MobileNetV3.mlir:380-384)
+void launch_scale_channels(const void* x, const void* g, void* out, int dt, int N, int HW, int C, hipStream_t s);
+// out = act(a (+ b));  b may be null;  n elements, n a multiple of the 16-byte vector
+void launch_eltwise(const void* a, const void* b, void* out, int dt, long long n, int act, hipStream_t s);
+// copies x [P][C] into channels [c0, c0 + C) of out [P][ldo]   (torch.cat over channels, NHWC)
+void launch_concat_slice(const void* x, void* out, int dt, long long P, int C, int ldo, int c0, hipStream_t s);
+// nearest-neighbour 2x up-sampling [N,H,W,C] -> [N,2H,2W,C], written at channel offset c0 of pitch ldo
+void launch_upsample2x(const void* x, void* out, int dt, int N, int H, int W, int C, int ldo, int c0, hipStream_t s);
+// max-pool K x K, any stride / padding (-inf halo), NHWC
+void launch_maxpool_nhwc(const void* in, void* out, int dt, int N, int H, int W, int C, int K, int stride, int pad,
+                         hipStream_t s);
 void launch_cast(const void* src, int src_dt, void* dst, int dst_dt, long long n, hipStream_t s);
 void launch_fill_f32(float* dst, float v, long long n, hipStream_t s);
 

@@ -281,7 +281,7 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   }
   __syncthreads();  // every wave is done with the patch: LDS becomes the output tiles
 
-  tile_reduce_store<OutT, WK, NI>(acc, smem + ws * WK * kTileBytes, wk, lane, obase, f0blk, a.F, ess,
+  tile_reduce_store<OutT, WK, NI, false>(acc, smem + ws * WK * kTileBytes, wk, lane, obase, f0blk, a.F, ess,
                               static_cast<const OutT*>(a.residual), static_cast<OutT*>(a.out), a.relu);
 }
 
@@ -344,7 +344,7 @@ bool conv3x3_patch_applicable(const IgemmArgs& a, int in_dt) {
   static const bool off = getenv("NNCV_HIP_NO_PATCH") != nullptr;
   const int slab = in_dt == kF16 ? 64 : 32;
   int ws, tn, th, lg;
-  return !off && a.aux_f0 == 0 && a.wt_frag && a.R == 3 && a.S == 3 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 1 && a.pad_w == 1 &&
+  return !off && a.aux_f0 == 0 && a.relu <= kActRelu && a.wt_frag && a.R == 3 && a.S == 3 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 1 && a.pad_w == 1 &&
          a.batch == 1 && a.pix_stride == 0 && a.C % slab == 0 && a.F % 8 == 0 && a.ldo == a.F &&
          (long long)a.N * a.H * a.W * a.F < (1ll << 31) && (long long)a.N * a.H * a.W < (1 << 24) && a.in_bytes < kOOBp &&
          (long long)((a.F + 63) / 64) * 64 * 9 * a.C * (long long)dtype_size(in_dt) < (1ll << 31) &&

@@ -1,0 +1,384 @@
+#include "graph.hpp"
+
+#include <algorithm>
+
+#include "arena_plan.hpp"
+
+namespace nncv_hip {
+
+namespace {
+
+int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+// shift[c] = (shift ? shift[c] : 0) + (scale ? scale[c] : 1) * bias[c]:  BN(conv + bias) folded
+// into one scale/shift pair, or a plain bias turned into the epilogue's fp32 shift.
+template <typename T>
+__global__ void fold_bias_kernel(const T* __restrict__ bias, const float* __restrict__ scale, float* __restrict__ shift, int has_shift,
+                                 int F) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= F) return;
+  const float b = (float)bias[c];
+  shift[c] = (has_shift ? shift[c] : 0.0f) + (scale ? scale[c] : 1.0f) * b;
+}
+
+const char* kind_name(int k) {
+  switch (k) {
+    case NNCV_HIP_OP_CONV: return "conv";
+    case NNCV_HIP_OP_DWCONV: return "dwconv";
+    case NNCV_HIP_OP_MAXPOOL: return "maxpool";
+    case NNCV_HIP_OP_GAVGPOOL: return "gavgpool";
+    case NNCV_HIP_OP_SCALE: return "scale";
+    case NNCV_HIP_OP_ADD: return "add";
+    case NNCV_HIP_OP_ACT: return "act";
+    case NNCV_HIP_OP_CONCAT: return "concat";
+    case NNCV_HIP_OP_UPSAMPLE2X: return "upsample2x";
+    default: return "?";
+  }
+}
+
+int n_inputs(int kind) {
+  switch (kind) {
+    case NNCV_HIP_OP_SCALE:
+    case NNCV_HIP_OP_ADD: return 2;
+    case NNCV_HIP_OP_CONCAT: return 4;
+    case NNCV_HIP_OP_CONV: return 2;  // second one (residual) optional
+    default: return 1;
+  }
+}
+
+}  // namespace
+
+Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, long long n_elems, int dt, hipStream_t s)
+    : dt_(dt), c_in_(in_channels) {
+  NNCV_REQUIRE(dt == kF32 || dt == kF16, "graph: dtype must be 1 (fp32) or 2 (fp16)");
+  NNCV_REQUIRE(ops && n > 0 && in_channels > 0, "graph: empty operator list");
+  const int vn = dt == kF16 ? 8 : 4;
+  const size_t es = dtype_size(dt);
+  const char* blob = static_cast<const char*>(params);
+
+  int max_id = 0;
+  for (int i = 0; i < n; ++i) max_id = std::max(max_id, ops[i].out);
+  NNCV_REQUIRE(max_id >= 1 && max_id <= 4 * n + 4, "graph: tensor ids out of range");
+  n_tensors_ = max_id + 1;
+  channels_.assign(n_tensors_, 0);
+  last_use_.assign(n_tensors_, -1);
+  channels_[0] = round_up(in_channels, vn);
+  nodes_.resize(n);
+
+  auto param = [&](long long off, long long count, const std::string& what) -> const void* {
+    NNCV_REQUIRE(off >= 0 && off + count <= n_elems, "graph: " + what + " lies outside the parameter blob");
+    return blob + (size_t)off * es;
+  };
+
+  for (int i = 0; i < n; ++i) {
+    const GraphOp& op = ops[i];
+    const std::string where = "graph: operator " + std::to_string(i) + " (" + kind_name(op.kind) + "): ";
+    Node& nd = nodes_[i];
+    nd.op = op;
+    NNCV_REQUIRE(op.kind >= NNCV_HIP_OP_CONV && op.kind <= NNCV_HIP_OP_UPSAMPLE2X, where + "unknown kind");
+    NNCV_REQUIRE(op.out >= 1 && op.out < n_tensors_ && channels_[op.out] == 0, where + "`out` must be a new tensor id");
+    NNCV_REQUIRE(op.act >= kActNone && op.act <= kActSigmoid, where + "unknown activation");
+    const int ni = n_inputs(op.kind);
+    for (int k = 0; k < 4; ++k) {
+      const int t = op.in[k];
+      if (k >= ni) {
+        NNCV_REQUIRE(t < 0, where + "too many inputs");
+        continue;
+      }
+      const bool optional = k > 0 && (op.kind == NNCV_HIP_OP_CONV || op.kind == NNCV_HIP_OP_CONCAT);
+      if (t < 0 && optional) continue;
+      NNCV_REQUIRE(t >= 0 && t < n_tensors_ && channels_[t] > 0, where + "input is not a tensor defined earlier");
+      last_use_[t] = i;
+    }
+    const int C = channels_[op.in[0]];
+    nd.C = C;
+    int Cout = C;
+    switch (op.kind) {
+      case NNCV_HIP_OP_CONV: {
+        NNCV_REQUIRE(op.F > 0 && op.F % vn == 0, where + "F must be a multiple of the 16-byte vector");
+        NNCV_REQUIRE(op.K >= 1 && op.K <= 11 && op.stride >= 1 && op.pad >= 0, where + "bad geometry");
+        NNCV_REQUIRE(op.in[1] < 0 || channels_[op.in[1]] == op.F, where + "residual has another channel count");
+        Cout = op.F;
+        const int Cl = op.in[0] == 0 ? c_in_ : C;  // channels the filters really have
+        const void* w = param(op.w, (long long)op.F * Cl * op.K * op.K, where + "w");
+        nd.wt.reset((size_t)op.F * op.K * op.K * C * es);
+        NNCV_HIP_CHECK(hipMemsetAsync(nd.wt.get(), 0, nd.wt.bytes(), s));
+        launch_weight_frsc(w, dt, nd.wt.get(), dt, op.F, Cl, op.K, op.K, C, s);
+        if (op.K == 3 && op.stride == 1 && op.pad == 1 && Cl == C && C % (128 / (int)es) == 0) {
+          nd.wfrag.reset((size_t)((op.F + 63) / 64) * 64 * 9 * C * es);
+          launch_weight_frag3x3(w, dt, nd.wfrag.get(), dt, op.F, C, s);
+        }
+        break;
+      }
+      case NNCV_HIP_OP_DWCONV: {
+        NNCV_REQUIRE(op.K == 3 || op.K == 5, where + "K must be 3 or 5");
+        NNCV_REQUIRE(op.stride >= 1 && op.pad >= 0, where + "bad geometry");
+        NNCV_REQUIRE(op.in[0] != 0 || c_in_ == C, where + "the network input must have whole channel vectors");
+        const void* w = param(op.w, (long long)C * op.K * op.K, where + "w");
+        nd.wt.reset((size_t)C * op.K * op.K * es);
+        launch_weight_dw(w, dt, nd.wt.get(), dt, C, op.K, s);
+        break;
+      }
+      case NNCV_HIP_OP_MAXPOOL:
+        NNCV_REQUIRE(op.K >= 1 && op.stride >= 1 && op.pad >= 0 && 2 * op.pad <= op.K, where + "bad geometry");
+        break;
+      case NNCV_HIP_OP_SCALE:
+      case NNCV_HIP_OP_ADD:
+        NNCV_REQUIRE(channels_[op.in[1]] == C, where + "operands have different channel counts");
+        break;
+      case NNCV_HIP_OP_CONCAT:
+        for (int k = 1; k < 4; ++k)
+          if (op.in[k] >= 0) Cout += channels_[op.in[k]];
+        break;
+      default: break;
+    }
+    if (op.kind == NNCV_HIP_OP_CONV || op.kind == NNCV_HIP_OP_DWCONV) {
+      const int F = Cout;
+      if (op.gamma >= 0) {
+        NNCV_REQUIRE(op.beta >= 0 && op.mean >= 0 && op.var >= 0, where + "BatchNorm needs gamma, beta, mean and var");
+        nd.scale.reset((size_t)F * 4);
+        nd.shift.reset((size_t)F * 4);
+        launch_bn_fold(param(op.gamma, F, where + "gamma"), param(op.beta, F, where + "beta"), param(op.mean, F, where + "mean"),
+                       param(op.var, F, where + "var"), dt, nd.scale.as<float>(), nd.shift.as<float>(), F, s, op.eps);
+      }
+      if (op.bias >= 0) {
+        const void* b = param(op.bias, F, where + "bias");
+        const bool had = nd.shift.get() != nullptr;
+        if (!had) nd.shift.reset((size_t)F * 4);
+        const unsigned grid = (unsigned)((F + 255) / 256);
+        if (dt == kF16)
+          hipLaunchKernelGGL((fold_bias_kernel<half_t>), dim3(grid), dim3(256), 0, s, (const half_t*)b, nd.scale.as<float>(),
+                             nd.shift.as<float>(), had ? 1 : 0, F);
+        else
+          hipLaunchKernelGGL((fold_bias_kernel<float>), dim3(grid), dim3(256), 0, s, (const float*)b, nd.scale.as<float>(),
+                             nd.shift.as<float>(), had ? 1 : 0, F);
+        NNCV_HIP_CHECK(hipGetLastError());
+      }
+    }
+    NNCV_REQUIRE(Cout % vn == 0, where + "channel count must be a multiple of the 16-byte vector");
+    channels_[op.out] = Cout;
+  }
+  for (int t = 1; t < n_tensors_; ++t) NNCV_REQUIRE(channels_[t] > 0, "graph: tensor " + std::to_string(t) + " is never produced");
+}
+
+const Graph::Plan& Graph::plan_of(int N, int H, int W) const {
+  for (const Plan& p : plans_)
+    if (p.N == N && p.H == H && p.W == W) return p;
+  NNCV_REQUIRE(N >= 1 && H >= 1 && W >= 1, "graph: empty input");
+  Plan p;
+  p.N = N; p.H = H; p.W = W;
+  p.dims.assign(n_tensors_, Dims{0, 0, 0});
+  p.dims[0] = Dims{channels_[0], H, W};
+  const int n = (int)nodes_.size();
+  for (int i = 0; i < n; ++i) {
+    const GraphOp& op = nodes_[i].op;
+    const std::string where = "graph: operator " + std::to_string(i) + " (" + kind_name(op.kind) + "): ";
+    const Dims a = p.dims[op.in[0]];
+    Dims o{channels_[op.out], a.H, a.W};
+    switch (op.kind) {
+      case NNCV_HIP_OP_CONV:
+      case NNCV_HIP_OP_DWCONV:
+      case NNCV_HIP_OP_MAXPOOL:
+        NNCV_REQUIRE(a.H + 2 * op.pad >= op.K && a.W + 2 * op.pad >= op.K, where + "image smaller than the window");
+        o.H = (a.H + 2 * op.pad - op.K) / op.stride + 1;
+        o.W = (a.W + 2 * op.pad - op.K) / op.stride + 1;
+        if (op.kind == NNCV_HIP_OP_CONV && op.in[1] >= 0)
+          NNCV_REQUIRE(p.dims[op.in[1]].H == o.H && p.dims[op.in[1]].W == o.W, where + "residual has another size");
+        break;
+      case NNCV_HIP_OP_GAVGPOOL: o.H = o.W = 1; break;
+      case NNCV_HIP_OP_SCALE:
+        NNCV_REQUIRE(p.dims[op.in[1]].H == 1 && p.dims[op.in[1]].W == 1, where + "the gate must be [N,C,1,1]");
+        break;
+      case NNCV_HIP_OP_ADD:
+        NNCV_REQUIRE(p.dims[op.in[1]].H == a.H && p.dims[op.in[1]].W == a.W, where + "operands have different sizes");
+        break;
+      case NNCV_HIP_OP_CONCAT:
+        for (int k = 1; k < 4; ++k)
+          if (op.in[k] >= 0)
+            NNCV_REQUIRE(p.dims[op.in[k]].H == a.H && p.dims[op.in[k]].W == a.W, where + "operands have different sizes");
+        break;
+      case NNCV_HIP_OP_UPSAMPLE2X: o.H = 2 * a.H; o.W = 2 * a.W; break;
+      default: break;
+    }
+    NNCV_REQUIRE((long long)N * o.H * o.W * o.C < (1ll << 31), where + "tensor too large");
+    p.dims[op.out] = o;
+  }
+  // Lifetimes in operator steps: step 0 lays the input out as NHWC, step i + 1 is operator i,
+  // step n + 1 converts the output.  A tensor is live from the step that writes it to the last
+  // step that reads it, so an operator's output never shares memory with any of its inputs.
+  std::vector<TensorLife> life(n_tensors_);
+  const size_t es = dtype_size(dt_);
+  life[0] = TensorLife{0, std::max(0, last_use_[0] + 1), (size_t)N * H * W * channels_[0] * es, 0};
+  for (int i = 0; i < n; ++i) {
+    const int t = nodes_[i].op.out;
+    const Dims d = p.dims[t];
+    life[t] = TensorLife{i + 1, std::max(i + 1, last_use_[t] + 1), (size_t)N * d.H * d.W * d.C * es, 0};
+  }
+  life[nodes_[n - 1].op.out].last_op = n + 1;
+  p.total = plan_offsets(life, 256);
+  p.offset.resize(n_tensors_);
+  for (int t = 0; t < n_tensors_; ++t) p.offset[t] = life[t].offset;
+  if (plans_.size() >= 8) plans_.erase(plans_.begin());
+  plans_.push_back(std::move(p));
+  return plans_.back();
+}
+
+void Graph::output_shape(int H, int W, int* C, int* OH, int* OW) const {
+  const Plan& p = plan_of(1, H, W);
+  const Dims d = p.dims[nodes_.back().op.out];
+  *C = d.C; *OH = d.H; *OW = d.W;
+}
+
+size_t Graph::workspace_bytes(int N, int H, int W) const { return plan_of(N, H, W).total; }
+
+void Graph::forward(const void* src, int N, int H, int W, float* out, void* ws, hipStream_t s) const {
+  const Plan& p = plan_of(N, H, W);
+  char* base = static_cast<char*>(ws);
+  auto at = [&](int t) -> void* { return base + p.offset[t]; };
+  launch_relayout(src, dt_, strides_of(kNCHW, c_in_, H, W), at(0), dt_, strides_of(kNHWC, channels_[0], H, W), N, c_in_,
+                  channels_[0], H, W, false, s);
+  for (const Node& nd : nodes_) {
+    const GraphOp& op = nd.op;
+    const Dims a = p.dims[op.in[0]], o = p.dims[op.out];
+    switch (op.kind) {
+      case NNCV_HIP_OP_CONV: {
+        IgemmArgs g{};
+        g.in = at(op.in[0]); g.wt = nd.wt.get(); g.wt_frag = nd.wfrag.get(); g.out = at(op.out);
+        g.scale = nd.scale.as<float>(); g.shift = nd.shift.as<float>();
+        g.residual = op.in[1] >= 0 ? at(op.in[1]) : nullptr;
+        g.N = N; g.H = a.H; g.W = a.W; g.C = a.C; g.F = op.F; g.R = g.S = op.K; g.OH = o.H; g.OW = o.W;
+        g.stride_h = g.stride_w = op.stride; g.pad_h = g.pad_w = op.pad;
+        g.relu = op.act; g.ldo = op.F; g.batch = 1;
+        launch_igemm(g, dt_, dt_, s);
+        break;
+      }
+      case NNCV_HIP_OP_DWCONV: {
+        DwConvArgs d{};
+        d.in = at(op.in[0]); d.wt = nd.wt.get(); d.out = at(op.out);
+        d.scale = nd.scale.as<float>(); d.shift = nd.shift.as<float>();
+        d.N = N; d.H = a.H; d.W = a.W; d.C = a.C; d.K = op.K; d.stride = op.stride; d.pad = op.pad; d.OH = o.H; d.OW = o.W;
+        d.act = op.act;
+        launch_dwconv(d, dt_, s);
+        break;
+      }
+      case NNCV_HIP_OP_MAXPOOL:
+        launch_maxpool_nhwc(at(op.in[0]), at(op.out), dt_, N, a.H, a.W, a.C, op.K, op.stride, op.pad, s);
+        break;
+      case NNCV_HIP_OP_GAVGPOOL:
+        launch_global_avgpool_nhwc(at(op.in[0]), at(op.out), dt_, N, a.H * a.W, a.C, s);
+        break;
+      case NNCV_HIP_OP_SCALE:
+        launch_scale_channels(at(op.in[0]), at(op.in[1]), at(op.out), dt_, N, a.H * a.W, a.C, s);
+        break;
+      case NNCV_HIP_OP_ADD:
+        launch_eltwise(at(op.in[0]), at(op.in[1]), at(op.out), dt_, (long long)N * a.H * a.W * a.C, op.act, s);
+        break;
+      case NNCV_HIP_OP_ACT:
+        launch_eltwise(at(op.in[0]), nullptr, at(op.out), dt_, (long long)N * a.H * a.W * a.C, op.act, s);
+        break;
+      case NNCV_HIP_OP_CONCAT: {
+        int c0 = 0;
+        for (int k = 0; k < 4; ++k) {
+          if (op.in[k] < 0) continue;
+          const int Ck = p.dims[op.in[k]].C;
+          launch_concat_slice(at(op.in[k]), at(op.out), dt_, (long long)N * o.H * o.W, Ck, o.C, c0, s);
+          c0 += Ck;
+        }
+        break;
+      }
+      case NNCV_HIP_OP_UPSAMPLE2X:
+        launch_upsample2x(at(op.in[0]), at(op.out), dt_, N, a.H, a.W, a.C, a.C, 0, s);
+        break;
+      default: fail("graph: unknown operator kind");
+    }
+  }
+  const int t = nodes_.back().op.out;
+  const Dims d = p.dims[t];
+  launch_relayout(at(t), dt_, strides_of(kNHWC, d.C, d.H, d.W), out, kF32, strides_of(kNCHW, d.C, d.H, d.W), N, d.C, d.C, d.H, d.W,
+                  false, s);
+}
+
+// ---------------------------------------------------------------------------------------------
+// MobileNetV3-small, the network of tests/Nets/MobileNetV3.mlir (torchvision's mobilenet_v3_small:
+// 52 convolutions of which 11 depthwise, 9 squeeze-excitation blocks, BatchNorm epsilon 1e-3,
+// two Linear layers).  Parameter order = state_dict order without num_batches_tracked:
+//   conv weight, then BN weight / bias / running_mean / running_var; SE fc1 weight, bias, fc2
+//   weight, bias; classifier weight, bias.
+// ---------------------------------------------------------------------------------------------
+std::vector<GraphOp> mobilenetv3_small_ops(long long* n_elems) {
+  std::vector<GraphOp> ops;
+  long long off = 0;
+  int next = 1;
+  const float eps = 1e-3f;
+  auto blank = [](int kind) {
+    GraphOp o{};
+    o.kind = kind;
+    o.in[0] = o.in[1] = o.in[2] = o.in[3] = -1;
+    o.w = o.bias = o.gamma = o.beta = o.mean = o.var = -1;
+    return o;
+  };
+  // conv / dwconv followed by BatchNorm
+  auto conv_bn = [&](int in, int C, int F, int K, int stride, bool depthwise, int act, int residual) {
+    GraphOp o = blank(depthwise ? NNCV_HIP_OP_DWCONV : NNCV_HIP_OP_CONV);
+    o.in[0] = in; o.in[1] = residual; o.out = next++;
+    o.F = F; o.K = K; o.stride = stride; o.pad = (K - 1) / 2; o.act = act; o.eps = eps;
+    o.w = off; off += (long long)F * (depthwise ? 1 : C) * K * K;
+    o.gamma = off; off += F;
+    o.beta = off; off += F;
+    o.mean = off; off += F;
+    o.var = off; off += F;
+    ops.push_back(o);
+    return o.out;
+  };
+  // 1x1 convolution / Linear with bias
+  auto fc = [&](int in, int C, int F, int act) {
+    GraphOp o = blank(NNCV_HIP_OP_CONV);
+    o.in[0] = in; o.out = next++;
+    o.F = F; o.K = 1; o.stride = 1; o.pad = 0; o.act = act;
+    o.w = off; off += (long long)F * C;
+    o.bias = off; off += F;
+    ops.push_back(o);
+    return o.out;
+  };
+  auto simple = [&](int kind, int a, int b) {
+    GraphOp o = blank(kind);
+    o.in[0] = a; o.in[1] = b; o.out = next++;
+    ops.push_back(o);
+    return o.out;
+  };
+  auto make_divisible8 = [](int v) {  // torchvision _make_divisible(v, 8)
+    int nv = std::max(8, (v + 4) / 8 * 8);
+    if (nv * 10 < 9 * v) nv += 8;
+    return nv;
+  };
+
+  int x = conv_bn(0, 3, 16, 3, 2, false, kActHardSwish, -1);
+  struct Cfg { int cin, k, exp, cout, se, hs, stride; };
+  const Cfg cfgs[11] = {{16, 3, 16, 16, 1, 0, 2},  {16, 3, 72, 24, 0, 0, 2},  {24, 3, 88, 24, 0, 0, 1},  {24, 5, 96, 40, 1, 1, 2},
+                        {40, 5, 240, 40, 1, 1, 1}, {40, 5, 240, 40, 1, 1, 1}, {40, 5, 120, 48, 1, 1, 1}, {48, 5, 144, 48, 1, 1, 1},
+                        {48, 5, 288, 96, 1, 1, 2}, {96, 5, 576, 96, 1, 1, 1}, {96, 5, 576, 96, 1, 1, 1}};
+  for (const Cfg& c : cfgs) {
+    const int act = c.hs ? kActHardSwish : kActRelu;
+    const int block_in = x;
+    int y = x;
+    if (c.exp != c.cin) y = conv_bn(y, c.cin, c.exp, 1, 1, false, act, -1);
+    y = conv_bn(y, c.exp, c.exp, c.k, c.stride, true, act, -1);
+    if (c.se) {
+      const int sq = make_divisible8(c.exp / 4);
+      int g = simple(NNCV_HIP_OP_GAVGPOOL, y, -1);
+      g = fc(g, c.exp, sq, kActRelu);
+      g = fc(g, sq, c.exp, kActHardSigmoid);
+      y = simple(NNCV_HIP_OP_SCALE, y, g);
+    }
+    const bool res = c.stride == 1 && c.cin == c.cout;
+    x = conv_bn(y, c.exp, c.cout, 1, 1, false, kActNone, res ? block_in : -1);
+  }
+  x = conv_bn(x, 96, 576, 1, 1, false, kActHardSwish, -1);
+  x = simple(NNCV_HIP_OP_GAVGPOOL, x, -1);
+  x = fc(x, 576, 1024, kActHardSwish);
+  x = fc(x, 1024, 1000, kActNone);
+  if (n_elems) *n_elems = off;
+  return ops;
+}
+
+}  // namespace nncv_hip

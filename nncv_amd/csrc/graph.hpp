@@ -1,0 +1,60 @@
+// A network as a list of operators over numbered NHWC tensors: what a compiled object for the
+// reference's other fixtures (tests/Nets/MobileNetV3.mlir, Yolov5s.mlir) is made of once BatchNorm
+// is folded and the elementwise tails are fused into their producers.  The reference has no such
+// object at run time -- its compiler bakes the graph into straight-line code -- so the description
+// is this library's own; its vocabulary is the fixtures' (conv_2d_nchw_fchw,
+// depthwise_conv_2d_nchw_chw, pooling_nchw_max / _sum, concat, the activation generics).
+#pragma once
+#include <memory>
+#include <vector>
+
+#include "../../include/nncv_hip.h"
+#include "runtime.hpp"
+
+namespace nncv_hip {
+
+typedef nncv_hip_graph_op GraphOp;
+
+class Graph {
+ public:
+  // ops: n operators in execution order.  Tensor 0 is the network input (NCHW, in_channels
+  // channels); every other tensor is the `out` of exactly one operator and may only be read by
+  // later ones.  The `out` of the last operator is the network output.
+  // params_dev: flat device blob of n_elems elements of type dt that the operators' offsets index.
+  Graph(const GraphOp* ops, int n, int in_channels, const void* params_dev, long long n_elems, int dt, hipStream_t s);
+  int dtype() const { return dt_; }
+  int in_channels() const { return c_in_; }
+  int num_ops() const { return (int)nodes_.size(); }
+  // channels / height / width of the network output for an H x W input
+  void output_shape(int H, int W, int* C, int* OH, int* OW) const;
+  size_t workspace_bytes(int N, int H, int W) const;
+  // src: NCHW [N,in_channels,H,W] of type dt; out: NCHW fp32 of the output shape (both device)
+  void forward(const void* src, int N, int H, int W, float* out, void* ws, hipStream_t s) const;
+
+ private:
+  struct Node {
+    GraphOp op;
+    int C = 0;  // channels of in[0] as stored (the network input is padded to a whole vector)
+    DeviceBuffer wt, wfrag, scale, shift;
+  };
+  struct Dims { int C, H, W; };
+  struct Plan {
+    int N, H, W;
+    std::vector<Dims> dims;      // per tensor
+    std::vector<size_t> offset;  // per tensor, in the workspace (tensor 0: its NHWC copy)
+    size_t total;
+  };
+  const Plan& plan_of(int N, int H, int W) const;
+
+  int dt_, c_in_, n_tensors_ = 0;
+  std::vector<Node> nodes_;
+  std::vector<int> channels_;  // per tensor, as stored
+  std::vector<int> last_use_;  // per tensor: index of the last operator that reads it
+  mutable std::vector<Plan> plans_;
+};
+
+// The operator list and parameter count of torchvision's MobileNetV3-small as exported in
+// tests/Nets/MobileNetV3.mlir (parameters in state_dict order without num_batches_tracked).
+std::vector<GraphOp> mobilenetv3_small_ops(long long* n_elems);
+
+}  // namespace nncv_hip

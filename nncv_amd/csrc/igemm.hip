@@ -60,10 +60,6 @@ struct Vec4<half_t> {
   typedef half4 type;
 };
 
-// ReLU with the predicate of the reference (`arith.cmpf ugt`, tests/Nets/Res18.mlir:139-141):
-// NaN is kept, everything not greater than zero becomes +0.
-__device__ __forceinline__ float relu_ugt(float x) { return (x <= 0.0f) ? 0.0f : x; }
-
 constexpr int kThreads = 256;
 constexpr int kChunksPerStep = 4;                   // 16-byte chunks per row per K step
 constexpr int kRowBytes = (kChunksPerStep + 1) * 16;  // LDS row pitch: 64 B payload + 16 B pad
@@ -201,9 +197,12 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(const IgemmArgs a) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) y[e] += (float)rv[e];
         }
-        if (a.relu) {
+        if (a.relu == kActRelu) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) y[e] = relu_ugt(y[e]);
+        } else if (a.relu) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) y[e] = act_apply(y[e], a.relu);
         }
         V4 ov;
 #pragma unroll

@@ -34,8 +34,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, unsig
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
 }
 
-// ReLU with the reference's predicate (`arith.cmpf ugt`, tests/Nets/Res18.mlir:139-141): NaN stays.
-__device__ __forceinline__ float relu_ugt(float x) { return (x <= 0.0f) ? 0.0f : x; }
+using ::nncv_hip::relu_ugt;
 
 // x / d for 0 <= x < 2^24 and 1 <= d, given inv = 1.0f / d computed on the host: one float
 // multiply and a +-1 correction instead of the integer-divide expansion (which costs more VALU
@@ -101,7 +100,8 @@ struct EpiScale {
 
 // NI = 1: the wave tile is 64 slots x 32 channels (acc[0] only); the LDS tile keeps its 64-channel
 // rows and the lanes of the upper 32 channels simply store nothing.
-template <typename OutT, int NG, int NI = 2>
+// ACT = false compiles only the ReLU form of the activation (the register-tight patch kernel).
+template <typename OutT, int NG, int NI = 2, bool ACT = true>
 __device__ __forceinline__ void tile_reduce_store(const floatx16 (&acc)[2][2], unsigned char* tile, int g, int lane,
                                                   const int (&rowoff)[2], int f0, int F, const EpiScale<OutT>& ss,
                                                   const OutT* res, OutT* out, int relu) {
@@ -168,9 +168,12 @@ __device__ __forceinline__ void tile_reduce_store(const floatx16 (&acc)[2][2], u
 #pragma unroll
       for (int e = 0; e < FPL; ++e) y[e] += (float)rv[it][e];
     }
-    if (relu) {
+    if (relu == kActRelu) {
 #pragma unroll
       for (int e = 0; e < FPL; ++e) y[e] = relu_ugt(y[e]);
+    } else if (ACT && relu) {
+#pragma unroll
+      for (int e = 0; e < FPL; ++e) y[e] = act_apply(y[e], relu);
     }
     VO ov;
 #pragma unroll

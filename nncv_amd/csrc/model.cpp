@@ -21,9 +21,10 @@ ConvLayer::ConvLayer(const Desc& d, const void* w, const void* gamma, const void
     : d_(d) {
   NNCV_REQUIRE(d.dt == kF32 || d.dt == kF16, "conv: dtype must be f32 or f16");
   NNCV_REQUIRE(d.C > 0 && d.F > 0 && d.R > 0 && d.S > 0 && d.stride > 0 && d.pad >= 0, "conv: bad geometry");
+  NNCV_REQUIRE(d.relu >= kActNone && d.relu <= kActSigmoid, "conv: unknown activation");
   const int ce = d.dt == kF16 ? 8 : 4;
   const size_t es = dtype_size(d.dt);
-  const bool wino_ok = !d.stem && d.R == 3 && d.S == 3 && d.stride == 1 && d.C % ce == 0 && d.F % 4 == 0;
+  const bool wino_ok = !d.stem && d.relu <= kActRelu && d.R == 3 && d.S == 3 && d.stride == 1 && d.C % ce == 0 && d.F % 4 == 0;
   int algo = d.algo;
   if (algo == kAlgoAuto) algo = env_algo3x3();
   // default: the direct form for both types.  In fp16 F(4,3) costs about 10x the rounding error;
@@ -114,7 +115,7 @@ void ConvLayer::forward(const void* in, int N, int H, int W, const void* residua
 }
 
 bool ConvLayer::forward_stem_pool(const void* in, int N, int H, int W, void* pooled_out, hipStream_t s) const {
-  if (!d_.stem || !d_.relu || !stem_pool_applicable(d_.dt, N, H, W, d_.F)) return false;
+  if (!d_.stem || d_.relu != kActRelu || !stem_pool_applicable(d_.dt, N, H, W, d_.F)) return false;
   launch_stem_pool(in, wt_shift_.get(), scale_.as<float>(), shift_.as<float>(), pooled_out, N, H, W, s);
   return true;
 }
@@ -275,7 +276,7 @@ static Plan make_plan(const ConvLayer& stem, const std::vector<const ConvLayer*>
   std::vector<TensorLife> t;
   auto add = [&](int first, int last, size_t bytes) { t.push_back(TensorLife{first, last, bytes, 0}); return (int)t.size() - 1; };
   // the fused stem kernel writes the pooled tensor directly: no stem output, no packed image
-  const bool fused_stem = stem.desc().relu && stem_pool_applicable(dt, N, H, W, stem.desc().F);
+  const bool fused_stem = stem.desc().relu == kActRelu && stem_pool_applicable(dt, N, H, W, stem.desc().F);
   const int i_stem = add(0, 1, fused_stem ? 0 : (size_t)N * p.h1 * p.w1 * 64 * es);
   size_t cws = fused_stem ? 0 : stem.workspace_bytes(N, H, W);
   int h = p.h2, w = p.w2, ch = 64;

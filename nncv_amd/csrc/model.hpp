@@ -21,7 +21,7 @@ class ConvLayer {
   struct Desc {
     int dt = kF32;  // element type of activations and weights
     int C = 0, F = 0, R = 0, S = 0, stride = 1, pad = 0;
-    bool relu = false;
+    int relu = 0;  // activation applied last (enum Act); 1 = ReLU
     int algo = kAlgoAuto;
     bool stem = false;  // 7x7 s2 p3 over 3 channels read from NCHW (pixel-pair packing)
   };
@@ -58,7 +58,7 @@ class ConvLayer {
   DeviceBuffer wt_, wfrag_, U_, scale_, shift_, wt_shift_;
   DeviceBuffer wt_cat_, scale_cat_, shift_cat_;  // this layer's filters followed by the fused shortcut's
   int aux_F_ = 0;
-  bool aux_relu_ = false;
+  int aux_relu_ = 0;
   double aux_flops_per_pixel_ = 0.0;
 };
 

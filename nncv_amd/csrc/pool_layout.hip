@@ -439,10 +439,10 @@ void launch_stem_weight(const void* w, int w_dt, void* dst, int dst_dt, int F, i
 //   r = 1/sqrt(var + (float)1e-5) ; scale = gamma * r ; shift = beta - mean * scale
 // evaluated in fp64 and rounded once, so the fold adds less than one fp32 ulp to each factor.
 template <typename T>
-__global__ void bn_fold_kernel(const T* g, const T* b, const T* m, const T* v, float* scale, float* shift, int C) {
+__global__ void bn_fold_kernel(const T* g, const T* b, const T* m, const T* v, float* scale, float* shift, int C, float eps_f) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= C) return;
-  const double eps = (double)(float)1e-5;
+  const double eps = (double)eps_f;  // the reference truncates its f64 epsilon to f32 first
   const double r = 1.0 / sqrt((double)(float)v[c] + eps);
   const double sc = (double)(float)g[c] * r;
   scale[c] = (float)sc;
@@ -450,12 +450,12 @@ __global__ void bn_fold_kernel(const T* g, const T* b, const T* m, const T* v, f
 }
 
 void launch_bn_fold(const void* g, const void* b, const void* m, const void* v, int dt, float* scale, float* shift, int C,
-                    hipStream_t s) {
+                    hipStream_t s, float eps) {
   const unsigned grid = (unsigned)((C + 255) / 256);
   if (dt == kF16)
-    hipLaunchKernelGGL((bn_fold_kernel<half_t>), dim3(grid), dim3(256), 0, s, (const half_t*)g, (const half_t*)b, (const half_t*)m, (const half_t*)v, scale, shift, C);
+    hipLaunchKernelGGL((bn_fold_kernel<half_t>), dim3(grid), dim3(256), 0, s, (const half_t*)g, (const half_t*)b, (const half_t*)m, (const half_t*)v, scale, shift, C, eps);
   else
-    hipLaunchKernelGGL((bn_fold_kernel<float>), dim3(grid), dim3(256), 0, s, (const float*)g, (const float*)b, (const float*)m, (const float*)v, scale, shift, C);
+    hipLaunchKernelGGL((bn_fold_kernel<float>), dim3(grid), dim3(256), 0, s, (const float*)g, (const float*)b, (const float*)m, (const float*)v, scale, shift, C, eps);
   NNCV_HIP_CHECK(hipGetLastError());
 }
 

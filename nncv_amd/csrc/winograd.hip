@@ -32,7 +32,6 @@ struct Pair<half_t> {
   typedef half_t type __attribute__((ext_vector_type(2)));
 };
 
-__device__ __forceinline__ float relu_ugt(float x) { return (x <= 0.0f) ? 0.0f : x; }
 
 // rows of B^T applied to a 6-vector
 __device__ __forceinline__ void bt6(const float d[6], float o[6]) {

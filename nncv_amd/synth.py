@@ -100,6 +100,34 @@ def resnet18_params(seed_base=3100):
     return blob
 
 
+def mobilenetv3_params(seed_base=6100):
+    """Flat fp32 parameter blob of MobileNetV3-small in the canonical order (mobilenetv3_spec).
+
+    conv / Linear weights: Kaiming normal, std = sqrt(2/fan_in) (fan_in = K*K for depthwise filters);
+    conv / Linear biases N(0, 0.1); BN as in resnet18_params.  Tensor k uses seed seed_base + k."""
+    from . import mobilenetv3_spec as m
+    parts = []
+    for k, (name, shape) in enumerate(m.tensor_table()):
+        seed = seed_base + k
+        if len(shape) >= 2:
+            fan_in = int(np.prod(shape[1:]))
+            a = normal(seed, shape, std=float(np.sqrt(2.0 / fan_in)))
+        elif name.endswith("running_var"):
+            a = uniform(seed, shape, 0.5, 1.5)
+        elif name.endswith("running_mean"):
+            a = normal(seed, shape, std=0.1)
+        elif name.endswith(".weight"):  # BN gamma
+            a = uniform(seed, shape, 0.5, 1.5)
+        elif name.endswith(".bias"):  # BN beta, squeeze-excitation and classifier biases
+            a = normal(seed, shape, std=0.1)
+        else:
+            raise AssertionError(name)
+        parts.append(a.reshape(-1))
+    blob = np.concatenate(parts)
+    assert blob.size == m.NUM_ELEMENTS
+    return blob
+
+
 def cfg3_input():
     return uniform(3000, (1, 3, 256, 256), 0.0, 1.0)
 

@@ -195,6 +195,174 @@ def resnet18_forward(x, params, tap_layer=-1):
     return (y, tap) if tap_layer >= 0 else y
 
 
+# ---- operators of tests/Nets/MobileNetV3.mlir and Yolov5s.mlir, numpy (fp32 like the fixtures) ----
+def batchnorm_eps(x, gamma, beta, mean, var, eps):
+    """(x - mean) * rsqrt(var + f32(eps)) * gamma + beta, op by op (MobileNetV3.mlir:249-258)."""
+    x = _c(x)
+    sh = (1, -1) + (1,) * (x.ndim - 2)
+    r = (np.float32(1.0) / np.sqrt(_c(var) + np.float32(eps))).astype(np.float32)
+    return (((x - _c(mean).reshape(sh)) * r.reshape(sh)) * _c(gamma).reshape(sh) + _c(beta).reshape(sh)).astype(np.float32)
+
+
+def depthwise_conv2d_nchw_chw(x_padded, w, stride=1):
+    """linalg.depthwise_conv_2d_nchw_chw (MobileNetV3.mlir:290): out[n,c,oh,ow] += x[n,c,oh*s+kh,ow*s+kw] * w[c,kh,kw],
+    accumulated over (kh, kw) in loop order, separate multiply and add."""
+    x_padded, w = _c(x_padded), _c(w)
+    N, C, H, W = x_padded.shape
+    if w.ndim == 4:
+        w = w.reshape(w.shape[0], w.shape[2], w.shape[3])  # tensor.collapse_shape of [C,1,K,K] (:289)
+    assert w.shape[0] == C
+    K1, K2 = w.shape[1:]
+    OH, OW = (H - K1) // stride + 1, (W - K2) // stride + 1
+    y = np.zeros((N, C, OH, OW), np.float32)
+    for kh in range(K1):
+        for kw in range(K2):
+            win = x_padded[:, :, kh:kh + stride * (OH - 1) + 1:stride, kw:kw + stride * (OW - 1) + 1:stride]
+            y = y + win * w[None, :, kh, kw, None, None]
+    return y
+
+
+def hardswish(x):
+    """(min(relu_ugt(x + 3), 6) / 6) * x, the generics of MobileNetV3.mlir:259-293; the min is `olt` + select."""
+    x = _c(x)
+    t = relu(x + np.float32(3.0))
+    t = np.where(t < np.float32(6.0), t, np.float32(6.0)).astype(np.float32)
+    return ((t / np.float32(6.0)) * x).astype(np.float32)
+
+
+def hardsigmoid(x):
+    """max(0, min(1, (x + 3) / 6)) as MobileNetV3.mlir:349-379 spells it: olt(1, t) ? 1 : t, then ogt(0, m) ? 0 : m."""
+    x = _c(x)
+    t = ((x + np.float32(3.0)) / np.float32(6.0)).astype(np.float32)
+    m = np.where(np.float32(1.0) < t, np.float32(1.0), t)
+    return np.where(np.float32(0.0) > m, np.float32(0.0), m).astype(np.float32)
+
+
+def sigmoid(x):
+    """1 / (exp(-x) + 1)  (Yolov5s.mlir:158-165)"""
+    x = _c(x)
+    return (np.float32(1.0) / (np.exp(-x) + np.float32(1.0))).astype(np.float32)
+
+
+def silu(x):
+    """sigmoid(x) * x  (Yolov5s.mlir:158-171)"""
+    return (sigmoid(x) * _c(x)).astype(np.float32)
+
+
+ACTIVATIONS = {0: _c, 1: relu, 2: hardswish, 3: hardsigmoid, 4: silu, 5: sigmoid}
+
+
+def maxpool_nchw(x, k, stride, pad):
+    """linalg.pooling_nchw_max over a -inf halo (Yolov5s.mlir SPPF: 5x5 stride 1 pad 2)."""
+    xp = pad_nchw(x, pad, -np.inf) if pad else _c(x)
+    N, C, H, W = xp.shape
+    OH, OW = (H - k) // stride + 1, (W - k) // stride + 1
+    y = np.full((N, C, OH, OW), -np.inf, np.float32)
+    lib().orc_maxpool_nchw(xp, y, N, C, H, W, k, k, stride, stride)
+    return y
+
+
+def upsample2x_nearest(x):
+    """out[n,c,y,x] = in[n,c,y // 2,x // 2]  (the index arithmetic + tensor.extract generics of Yolov5s.mlir)"""
+    return _c(x).repeat(2, axis=2).repeat(2, axis=3)
+
+
+def mobilenetv3_forward(x, tensors, taps=None):
+    """MobileNetV3-small as tests/Nets/MobileNetV3.mlir computes it.  x [N,3,H,W] fp32; tensors: {name: ndarray} with
+    torchvision state_dict names (nncv_amd.mobilenetv3_spec.tensor_table) -> logits [N,1000].
+    `taps`, when a list, receives the NCHW output of every bottleneck block."""
+    from nncv_amd import mobilenetv3_spec as spec
+    T = tensors
+    eps = spec.BN_EPS
+
+    def bn(y, p):
+        return batchnorm_eps(y, T[p + ".weight"], T[p + ".bias"], T[p + ".running_mean"], T[p + ".running_var"], eps)
+
+    def conv(y, name, stride=1, pad=0):
+        return conv2d_nchw_fchw(pad_nchw(y, pad) if pad else y, T[name + ".weight"], stride)
+
+    def conv_bias(y, name):  # the bias initialises the accumulator (:331-335)
+        w = _c(T[name + ".weight"])
+        w = w.reshape(w.shape[0], w.shape[1], 1, 1)
+        init = np.broadcast_to(_c(T[name + ".bias"]).reshape(1, -1, 1, 1), (y.shape[0], w.shape[0], 1, 1))
+        return conv2d_nchw_fchw(y, w, 1, out=init)
+
+    y = hardswish(bn(conv(x, "features.0.0", 2, 1), "features.0.1"))
+    for i, (cin, k, exp, cout, se, hs, stride) in enumerate(spec.BNECK, start=1):
+        p = "features.%d.block" % i
+        act = hardswish if hs else relu
+        block_in, j = y, 0
+        if exp != cin:
+            y = act(bn(conv(y, "%s.%d.0" % (p, j)), "%s.%d.1" % (p, j)))
+            j += 1
+        y = act(bn(depthwise_conv2d_nchw_chw(pad_nchw(y, (k - 1) // 2), T["%s.%d.0.weight" % (p, j)], stride), "%s.%d.1" % (p, j)))
+        j += 1
+        if se:
+            N, C, H, W = y.shape
+            g = global_avgpool(y).reshape(N, C, 1, 1)  # pooling_nchw_sum, then one divf by H*W (:322-328)
+            g = relu(conv_bias(g, "%s.%d.fc1" % (p, j)))
+            g = hardsigmoid(conv_bias(g, "%s.%d.fc2" % (p, j)))
+            y = (g * y).astype(np.float32)
+            j += 1
+        y = bn(conv(y, "%s.%d.0" % (p, j)), "%s.%d.1" % (p, j))
+        if stride == 1 and cin == cout:
+            y = (y + block_in).astype(np.float32)
+        if taps is not None:
+            taps.append(y)
+    y = hardswish(bn(conv(y, "features.12.0"), "features.12.1"))
+    N, C = y.shape[:2]
+    y = global_avgpool(y)
+    y = hardswish(fc(y, T["classifier.0.weight"], T["classifier.0.bias"]))
+    return fc(y, T["classifier.3.weight"], T["classifier.3.bias"])
+
+
+def run_graph(ops, x, blob, in_channels):
+    """Evaluates a list of nncv_hip_graph_op-like records (attributes kind, inputs, out, F, K, stride, pad, act, eps,
+    w, bias, gamma, beta, mean, var) with the operator restatements above; NCHW fp32.  Checker for the graph executor."""
+    blob = _c(blob)
+    vals = {0: _c(x)}
+    for o in ops:
+        ins = [t for t in o.inputs if t >= 0]
+        a = vals[ins[0]]
+        act = ACTIVATIONS[o.act]
+        if o.kind in (1, 2):
+            C = a.shape[1]
+            if o.kind == 1:
+                F = o.F
+                w = blob[o.w:o.w + F * C * o.K * o.K].reshape(F, C, o.K, o.K)
+                y = conv2d_nchw_fchw(pad_nchw(a, o.pad) if o.pad else a, w, o.stride)
+            else:
+                F = C
+                w = blob[o.w:o.w + C * o.K * o.K].reshape(C, o.K, o.K)
+                y = depthwise_conv2d_nchw_chw(pad_nchw(a, o.pad) if o.pad else a, w, o.stride)
+            if o.bias >= 0:
+                y = (y + blob[o.bias:o.bias + F].reshape(1, F, 1, 1)).astype(np.float32)
+            if o.gamma >= 0:
+                y = batchnorm_eps(y, blob[o.gamma:o.gamma + F], blob[o.beta:o.beta + F], blob[o.mean:o.mean + F],
+                                  blob[o.var:o.var + F], o.eps)
+            if o.kind == 1 and len(ins) > 1:
+                y = (y + vals[ins[1]]).astype(np.float32)
+            y = act(y)
+        elif o.kind == 3:
+            y = maxpool_nchw(a, o.K, o.stride, o.pad)
+        elif o.kind == 4:
+            y = global_avgpool(a).reshape(a.shape[0], a.shape[1], 1, 1)
+        elif o.kind == 5:
+            y = (vals[ins[1]] * a).astype(np.float32)
+        elif o.kind == 6:
+            y = act((a + vals[ins[1]]).astype(np.float32))
+        elif o.kind == 7:
+            y = act(a)
+        elif o.kind == 8:
+            y = np.concatenate([vals[t] for t in ins], axis=1)
+        elif o.kind == 9:
+            y = upsample2x_nearest(a)
+        else:
+            raise ValueError("unknown operator kind %d" % o.kind)
+        vals[o.out] = _c(y)
+    return vals[ops[-1].out]
+
+
 # ---- the reference driver's pre- and post-processing (examples/Res18/main.cpp), numpy ----
 def preprocess_u8(img_hwc):
     """[N,H,W,ch>=3] uint8 -> [N,3,H,W] fp32: x = ((u8 / 255.f) - mean[c]) / std[c], every step in

@@ -131,3 +131,27 @@ class Model:
 
     def __del__(self):
         self.close()
+
+
+class Graph:
+    """nncv_hip_graph_* handle over an operator list and a host parameter blob."""
+
+    def __init__(self, ops, in_channels, blob, dt):
+        self.dt = dt
+        self.h = abi.graph_create(ops, in_channels, np.ascontiguousarray(blob, abi.np_dtype(dt)))
+
+    def __call__(self, x_dev):
+        N, C, H, W = x_dev.shape
+        c, oh, ow = abi.graph_output_shape(self.h, H, W)
+        out = torch.empty((N, c, oh, ow), dtype=torch.float32, device="cuda")
+        torch.cuda.synchronize()
+        abi.check(abi.lib().nncv_hip_graph_forward(self.h, x_dev.data_ptr(), N, H, W, out.data_ptr(), out.numel(), None))
+        return out
+
+    def close(self):
+        if self.h and abi is not None:
+            abi.lib().nncv_hip_graph_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        self.close()

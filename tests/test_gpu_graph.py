@@ -1,0 +1,296 @@
+"""Operators of the reference's other fixtures (MobileNetV3.mlir, Yolov5s.mlir) and the graph
+executor built from them, on the GPU through the C ABI, against the oracle."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from nncv_amd import abi, synth
+from nncv_amd import mobilenetv3_spec as spec
+from gpu_util import Conv, Graph, dev, empty, host, nchw, nhwc, max_rel, rel_l2, FP32_MAX_REL, FP16_REL_L2
+
+pytestmark = pytest.mark.gpu
+
+ACTS = [abi.ACT_NONE, abi.ACT_RELU, abi.ACT_HARDSWISH, abi.ACT_HARDSIGMOID, abi.ACT_SILU, abi.ACT_SIGMOID]
+
+
+def r16(a):
+    return synth.round_fp16(a)
+
+
+# ---------------------------------------------------------------------------------------------
+# single operators
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dt", [abi.F32, abi.F16])
+@pytest.mark.parametrize("k,stride,shape", [(3, 1, (2, 24, 13, 17)), (3, 2, (1, 16, 64, 64)), (5, 1, (3, 40, 9, 11)),
+                                            (5, 2, (2, 96, 32, 31)), (5, 1, (1, 576, 8, 8)), (3, 2, (1, 8, 5, 4))])
+def test_dwconv_vs_oracle(dt, k, stride, shape):
+    N, C, H, W = shape
+    pad = (k - 1) // 2
+    x = synth.normal(7000 + k, shape)
+    w = synth.normal(7001 + k, (C, 1, k, k), std=0.4)
+    scale = synth.uniform(7002, (C,), 0.5, 1.5)
+    shift = synth.normal(7003, (C,), std=0.2)
+    if dt == abi.F16:
+        x, w = r16(x), r16(w)
+    conv = oracle.depthwise_conv2d_nchw_chw(oracle.pad_nchw(x, pad), w, stride)
+    OH, OW = conv.shape[2:]
+    xd, wd, sd, hd = dev(nhwc(x), dt), dev(w, dt), dev(scale), dev(shift)
+    for act, affine in [(abi.ACT_NONE, False), (abi.ACT_HARDSWISH, True), (abi.ACT_RELU, True)]:
+        want = conv * scale.reshape(1, C, 1, 1) + shift.reshape(1, C, 1, 1) if affine else conv
+        want = oracle.ACTIVATIONS[act](want.astype(np.float32))
+        out = empty((N, OH, OW, C), dt)
+        print("dwconv", dt, k, stride, shape, act, affine, flush=True)
+        abi.check(abi.lib().nncv_hip_dwconv(dt, xd.data_ptr(), wd.data_ptr(), sd.data_ptr() if affine else None,
+                                            hd.data_ptr() if affine else None, out.data_ptr(), N, H, W, C, k, stride,
+                                            pad, act, None))
+        got = nchw(host(out))
+        if dt == abi.F32:
+            assert max_rel(got, want) < FP32_MAX_REL
+        else:
+            assert rel_l2(got, want) < 2e-3  # one rounding of the result to half
+
+
+def test_dwconv_rejects_bad_arguments():
+    x = empty((1, 4, 4, 12), abi.F16)
+    L = abi.lib()
+    assert L.nncv_hip_dwconv(abi.F16, x.data_ptr(), x.data_ptr(), None, None, x.data_ptr(), 1, 4, 4, 12, 3, 1, 1, 0, None) != 0
+    assert b"multiple" in L.nncv_hip_last_error()  # 12 channels are not whole 16-byte vectors of halves
+    assert L.nncv_hip_dwconv(abi.F16, x.data_ptr(), x.data_ptr(), None, None, x.data_ptr(), 1, 4, 4, 16, 4, 1, 1, 0, None) != 0
+    assert L.nncv_hip_dwconv(abi.F16, x.data_ptr(), x.data_ptr(), None, None, x.data_ptr(), 1, 2, 2, 16, 5, 1, 0, 0, None) != 0
+
+
+@pytest.mark.parametrize("dt", [abi.F32, abi.F16])
+def test_eltwise_activations_and_add(dt):
+    special = np.float32([-3, 3, 0, -0.0, 6, -6, np.inf, -np.inf, np.nan, 1e-8, -1e-8, 2.999, -2.999])
+    a = np.concatenate([synth.normal(7100, (4083,), std=3.0), special]).astype(np.float32)
+    b = synth.normal(7101, a.shape, std=1.0)
+    if dt == abi.F16:
+        a, b = r16(a), r16(b)
+    ad, bd = dev(a, dt), dev(b, dt)
+    for act in ACTS:
+        for add in (False, True):
+            want = oracle.ACTIVATIONS[act]((a + b).astype(np.float32) if add else a)
+            out = empty(a.shape, dt)
+            abi.check(abi.lib().nncv_hip_eltwise(dt, ad.data_ptr(), bd.data_ptr() if add else None, out.data_ptr(), a.size, act, None))
+            got = host(out)
+            if dt == abi.F16:
+                want = r16(want)
+            nan = np.isnan(want)
+            assert np.array_equal(np.isnan(got), nan), (act, add)
+            fin = np.isfinite(want)
+            assert np.array_equal(got[~fin & ~nan], want[~fin & ~nan]), (act, add)
+            tol = 2e-3 if dt == abi.F16 else 2e-6
+            assert np.abs(got[fin] - want[fin]).max() <= tol * max(1.0, np.abs(want[fin]).max()), (act, add)
+            if act in (abi.ACT_NONE, abi.ACT_RELU, abi.ACT_HARDSIGMOID) and not add and dt == abi.F32:
+                assert np.array_equal(got[fin], want[fin])  # no transcendental, no product: bit exact
+
+
+@pytest.mark.parametrize("dt", [abi.F32, abi.F16])
+def test_scale_concat_upsample_maxpool(dt):
+    N, H, W, C = 2, 7, 5, 24
+    x = synth.normal(7200, (N, C, H, W))
+    g = synth.uniform(7201, (N, C), 0.0, 1.0)
+    if dt == abi.F16:
+        x, g = r16(x), r16(g)
+    xd = dev(nhwc(x), dt)
+    L = abi.lib()
+    # squeeze-excitation gate
+    out, gd = empty((N, H, W, C), dt), dev(g, dt)
+    abi.check(L.nncv_hip_scale_channels(dt, xd.data_ptr(), gd.data_ptr(), out.data_ptr(), N, H * W, C, None))
+    want = g.reshape(N, C, 1, 1) * x
+    assert np.array_equal(nchw(host(out)), r16(want) if dt == abi.F16 else want)
+    # concat of [x, y] into 24 + 16 channels, then a 2x up-sampled copy into another slice
+    y = synth.normal(7202, (N, 16, H, W))
+    y = r16(y) if dt == abi.F16 else y
+    cat = torch.zeros((N, H, W, 40), dtype=xd.dtype, device="cuda")
+    abi.check(L.nncv_hip_concat_slice(dt, xd.data_ptr(), cat.data_ptr(), N * H * W, 24, 40, 0, None))
+    yd = dev(nhwc(y), dt)
+    abi.check(L.nncv_hip_concat_slice(dt, yd.data_ptr(), cat.data_ptr(), N * H * W, 16, 40, 24, None))
+    assert np.array_equal(nchw(host(cat)), np.concatenate([x, y], axis=1))
+    up = torch.zeros((N, 2 * H, 2 * W, 40), dtype=xd.dtype, device="cuda")
+    abi.check(L.nncv_hip_upsample2x(dt, xd.data_ptr(), up.data_ptr(), N, H, W, 24, 40, 16, None))
+    got = nchw(host(up))
+    assert np.array_equal(got[:, 16:], oracle.upsample2x_nearest(x)) and not got[:, :16].any()
+    # max-pool windows of the fixtures: SPPF 5x5 s1 p2, the ResNet 3x3 s2 p1, a plain 2x2 s2
+    for k, s, p in [(5, 1, 2), (3, 2, 1), (2, 2, 0)]:
+        want = oracle.maxpool_nchw(x, k, s, p)
+        out = empty((N, want.shape[2], want.shape[3], C), dt)
+        abi.check(L.nncv_hip_maxpool(dt, xd.data_ptr(), out.data_ptr(), N, H, W, C, k, s, p, None))
+        assert np.array_equal(nchw(host(out)), want)
+    assert L.nncv_hip_concat_slice(dt, xd.data_ptr(), cat.data_ptr(), N * H * W, 24, 40, 20, None) != 0  # 20 + 24 > 40
+
+
+@pytest.mark.parametrize("dt", [abi.F32, abi.F16])
+@pytest.mark.parametrize("C,F,k,stride,H", [(96, 576, 1, 1, 8), (64, 64, 3, 1, 20), (40, 240, 1, 1, 16), (64, 128, 3, 2, 21)])
+def test_conv_with_fused_activations(dt, C, F, k, stride, H):
+    """hard-swish / SiLU / hard-sigmoid in the epilogue of the MFMA kernels (fast and generic tiles)."""
+    x = synth.normal(7300, (2, C, H, H))
+    w = synth.normal(7301, (F, C, k, k), std=float(np.sqrt(2.0 / (C * k * k))))
+    bn = (synth.uniform(7302, (F,), 0.5, 1.5), synth.normal(7303, (F,), std=0.1), synth.normal(7304, (F,), std=0.1),
+          synth.uniform(7305, (F,), 0.5, 1.5))
+    if dt == abi.F16:
+        x, w = r16(x), r16(w)
+        bn = tuple(r16(b) for b in bn)
+    pad = (k - 1) // 2
+    pre = oracle.batchnorm(oracle.conv2d_nchw_fchw(oracle.pad_nchw(x, pad) if pad else x, w, stride), *bn)
+    xd = dev(nhwc(x), dt)
+    for act in (abi.ACT_HARDSWISH, abi.ACT_SILU, abi.ACT_HARDSIGMOID):
+        conv = Conv(dt, w, stride, pad, bn=bn, relu=act, algo=abi.ALGO_IGEMM)
+        print("conv+act", dt, C, F, k, stride, H, act, flush=True)
+        got = nchw(host(conv(xd, abi.NHWC)))
+        want = oracle.ACTIVATIONS[act](pre)
+        if dt == abi.F32:
+            assert max_rel(got, want) < FP32_MAX_REL
+        else:
+            assert rel_l2(got, want) < FP16_REL_L2
+        conv.close()
+
+
+# ---------------------------------------------------------------------------------------------
+# MobileNetV3-small through the graph executor
+# ---------------------------------------------------------------------------------------------
+@pytest.fixture(scope="module")
+def blob():
+    return synth.mobilenetv3_params()
+
+
+def tensors_of(blob):
+    return {name: blob[o:o + spec.numel(shape)].reshape(shape) for name, (o, shape) in spec.offsets().items()}
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 64, 64), (1, 3, 256, 256), (3, 3, 100, 77)])
+def test_mobilenetv3_fp32(blob, shape):
+    ops, n = abi.mobilenetv3_small_ops()
+    g = Graph(ops, 3, blob, abi.F32)
+    assert abi.graph_output_shape(g.h, shape[2], shape[3]) == (1000, 1, 1)
+    x = synth.uniform(7400, shape, 0.0, 1.0)
+    print("mobilenetv3 fp32", shape, flush=True)
+    got = host(g(dev(x))).reshape(shape[0], 1000)
+    want = oracle.mobilenetv3_forward(x, tensors_of(blob))
+    err = max_rel(got, want)
+    print("logits max_rel", err, flush=True)
+    assert err < FP32_MAX_REL
+    assert np.array_equal(got.argmax(1), want.argmax(1))
+    g.close()
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 64, 64), (32, 3, 224, 224)])
+def test_mobilenetv3_fp16(blob, shape):
+    b16 = r16(blob)
+    ops, n = abi.mobilenetv3_small_ops()
+    g = Graph(ops, 3, b16, abi.F16)
+    x = r16(synth.uniform(7401, shape, 0.0, 1.0))
+    print("mobilenetv3 fp16", shape, flush=True)
+    xd = dev(x, abi.F16)
+    got = host(g(xd)).reshape(shape[0], 1000)
+    want = oracle.mobilenetv3_forward(x, tensors_of(b16))
+    err = rel_l2(got, want)
+    print("logits rel_l2", err, flush=True)
+    assert err < FP16_REL_L2
+    assert np.array_equal(got.argmax(1), want.argmax(1))
+    # later calls replay a captured HIP graph: every replay must reproduce the eager result, with
+    # unrelated eager work and synchronisations in between
+    for it in range(4):
+        scratch = torch.randn(1 << 20, device="cuda").sum().item()
+        again = host(g(xd)).reshape(shape[0], 1000)
+        assert np.array_equal(again, got), it
+    g.close()
+
+
+def test_mobilenetv3_through_reference_abi(blob):
+    """_mlir_ciface_forward recognises the network by the size of the params memref (host memory in,
+    malloc'd [N,1000] out), as a program linked against the object for MobileNetV3.mlir would call it."""
+    x = synth.uniform(7402, (1, 3, 256, 256), 0.0, 1.0)
+    got = abi.forward(x, blob.copy())
+    want = oracle.mobilenetv3_forward(x, tensors_of(blob))
+    assert got.shape == (1, 1000)
+    assert max_rel(got, want) < FP32_MAX_REL
+    assert np.array_equal(got.argmax(1), want.argmax(1))
+
+
+# ---------------------------------------------------------------------------------------------
+# executor: the YOLOv5-style operators, and what it refuses
+# ---------------------------------------------------------------------------------------------
+def small_net(C=16):
+    """conv(SiLU) -> [5x5 max-pool x2, concat] -> conv 1x1 -> stride-2 conv -> upsample -> concat with the skip ->
+    conv + residual add -> sigmoid: every operator kind the MobileNetV3 list does not use."""
+    sizes, ops = [], []
+
+    def take(n):
+        off = sum(sizes)
+        sizes.append(n)
+        return off
+
+    def conv(i, o, cin, F, k, stride, act, res=-1, bias=True, bn=False):
+        w = take(F * cin * k * k)
+        b = take(F) if bias else -1
+        bnp = tuple(take(F) for _ in range(4)) if bn else None
+        ops.append(abi.graph_op(abi.OP_CONV, [i, res], o, F=F, K=k, stride=stride, pad=(k - 1) // 2, act=act, eps=1e-3, w=w,
+                                bias=b, bn=bnp))
+
+    conv(0, 1, 3, C, 3, 1, abi.ACT_SILU, bn=True)
+    ops.append(abi.graph_op(abi.OP_MAXPOOL, [1], 2, K=5, stride=1, pad=2))
+    ops.append(abi.graph_op(abi.OP_MAXPOOL, [2], 3, K=5, stride=1, pad=2))
+    ops.append(abi.graph_op(abi.OP_CONCAT, [1, 2, 3], 4))
+    conv(4, 5, 3 * C, C, 1, 1, abi.ACT_SILU)
+    conv(5, 6, C, 2 * C, 3, 2, abi.ACT_SILU, bias=False, bn=True)
+    ops.append(abi.graph_op(abi.OP_UPSAMPLE2X, [6], 7))
+    ops.append(abi.graph_op(abi.OP_CONCAT, [7, 5], 8))
+    conv(8, 9, 3 * C, C, 3, 1, abi.ACT_NONE, res=5)
+    ops.append(abi.graph_op(abi.OP_ADD, [9, 1], 10, act=abi.ACT_RELU))
+    ops.append(abi.graph_op(abi.OP_ACT, [10], 11, act=abi.ACT_SIGMOID))
+    n = sum(sizes)
+    blob = synth.normal(7500, (n,), std=0.15)
+    for o in ops:  # variances must be positive
+        if o.var >= 0:
+            blob[o.var:o.var + o.F] = synth.uniform(7501, (o.F,), 0.5, 1.5)
+    return ops, blob
+
+
+@pytest.mark.parametrize("dt", [abi.F32, abi.F16])
+def test_executor_on_yolo_style_operators(dt):
+    ops, blob = small_net()
+    x = synth.normal(7502, (2, 3, 20, 12))
+    if dt == abi.F16:
+        blob, x = r16(blob), r16(x)
+    g = Graph(ops, 3, blob, dt)
+    assert abi.graph_output_shape(g.h, 20, 12) == (16, 20, 12)
+    got = host(g(dev(x, dt)))
+    want = oracle.run_graph(ops, x, blob, 3)
+    assert got.shape == want.shape
+    if dt == abi.F32:
+        assert max_rel(got, want) < FP32_MAX_REL
+    else:
+        assert rel_l2(got, want) < FP16_REL_L2
+    # an odd-sized image cannot be up-sampled back onto its skip connection: refused with a message
+    out = torch.empty(2 * 16 * 21 * 12, device="cuda")
+    assert abi.lib().nncv_hip_graph_forward(g.h, out.data_ptr(), 2, 21, 12, out.data_ptr(), out.numel(), None) != 0
+    assert b"different sizes" in abi.lib().nncv_hip_last_error()
+    g.close()
+
+
+def test_graph_create_refuses_malformed_lists():
+    ops, blob = small_net()
+
+    def refused(bad, blob=blob, cin=3):
+        with pytest.raises(abi.NncvHipError) as e:
+            abi.graph_create(bad, cin, blob)
+        return str(e.value)
+
+    def clone(i, **kw):
+        c = [abi.GraphOp.from_buffer_copy(o) for o in ops]
+        for k, v in kw.items():
+            setattr(c[i], k, v)
+        return c
+
+    assert "defined earlier" in refused(clone(1, inputs=(ctypes.c_int32 * 4)(9, -1, -1, -1)))  # reads a later tensor
+    assert "new tensor id" in refused(clone(2, out=2))                                          # writes a tensor twice
+    assert "unknown kind" in refused(clone(3, kind=42))
+    assert "outside the parameter blob" in refused(clone(4, w=blob.size - 3))
+    assert "multiple" in refused(clone(4, F=10))                                                # 10 floats are not whole 16-byte vectors
+    assert "K must be 3 or 5" in refused(clone(1, kind=abi.OP_DWCONV, K=7, w=0))
+    assert "unknown activation" in refused(clone(10, act=9))
+    assert "channel" in refused(clone(8, inputs=(ctypes.c_int32 * 4)(8, 6, -1, -1)))            # residual with 2C channels

@@ -1,0 +1,186 @@
+"""The MobileNetV3 / YOLOv5 operator restatements of the oracle, pinned against torch CPU library
+routines (float64), the network's published parameter count and the structure of the reference's
+fixture tests/Nets/MobileNetV3.mlir; and the library's built-in operator list against the
+independently written Python one."""
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+from nncv_amd import abi, synth
+from nncv_amd import mobilenetv3_spec as spec
+
+FIXTURE = "/root/reference/tests/Nets/MobileNetV3.mlir"
+
+
+def close(got, want, tol=2e-6):
+    want = np.asarray(want, np.float64)
+    return np.abs(np.asarray(got, np.float64) - want).max() <= tol * max(np.abs(want).max(), 1.0)
+
+
+def tensors_of(blob):
+    out = {}
+    for name, (o, shape) in spec.offsets().items():
+        out[name] = blob[o:o + spec.numel(shape)].reshape(shape)
+    return out
+
+
+def torch_mobilenetv3(x, T):
+    """torchvision.models.mobilenet_v3_small.forward composed of float64 functional ops."""
+    P = lambda n: torch.from_numpy(np.asarray(T[n], np.float64))
+
+    def bn(y, p):
+        return F.batch_norm(y, P(p + ".running_mean"), P(p + ".running_var"), P(p + ".weight"), P(p + ".bias"), False, 0.0,
+                            float(np.float32(1e-3)))
+
+    y = torch.from_numpy(x.astype(np.float64))
+    y = F.hardswish(bn(F.conv2d(y, P("features.0.0.weight"), stride=2, padding=1), "features.0.1"))
+    taps = []
+    for i, (cin, k, exp, cout, se, hs, stride) in enumerate(spec.BNECK, start=1):
+        p = "features.%d.block" % i
+        act = F.hardswish if hs else F.relu
+        inp, j = y, 0
+        if exp != cin:
+            y = act(bn(F.conv2d(y, P("%s.%d.0.weight" % (p, j))), "%s.%d.1" % (p, j)))
+            j += 1
+        y = act(bn(F.conv2d(y, P("%s.%d.0.weight" % (p, j)), stride=stride, padding=(k - 1) // 2, groups=exp), "%s.%d.1" % (p, j)))
+        j += 1
+        if se:
+            g = F.adaptive_avg_pool2d(y, 1)
+            g = F.relu(F.conv2d(g, P("%s.%d.fc1.weight" % (p, j)), P("%s.%d.fc1.bias" % (p, j))))
+            g = F.hardsigmoid(F.conv2d(g, P("%s.%d.fc2.weight" % (p, j)), P("%s.%d.fc2.bias" % (p, j))))
+            y = g * y
+            j += 1
+        y = bn(F.conv2d(y, P("%s.%d.0.weight" % (p, j))), "%s.%d.1" % (p, j))
+        if stride == 1 and cin == cout:
+            y = y + inp
+        taps.append(y.numpy())
+    y = F.hardswish(bn(F.conv2d(y, P("features.12.0.weight")), "features.12.1"))
+    y = torch.flatten(F.adaptive_avg_pool2d(y, 1), 1)
+    y = F.hardswish(F.linear(y, P("classifier.0.weight"), P("classifier.0.bias")))
+    return F.linear(y, P("classifier.3.weight"), P("classifier.3.bias")).numpy(), taps
+
+
+def test_tensor_table_counts():
+    t = spec.tensor_table()
+    assert len(t) == spec.NUM_TENSORS == 210
+    assert sum(spec.numel(s) for _, s in t) == spec.NUM_ELEMENTS
+    stats = sum(spec.numel(s) for n, s in t if "running_" in n)
+    # torchvision documents 2 542 856 parameters for mobilenet_v3_small
+    assert spec.NUM_ELEMENTS - stats == 2542856
+    assert len(set(n for n, _ in t)) == len(t)
+    # the squeeze widths the fixture holds (tensor<8x16x1x1>, <24x96x1x1>, <64x240x1x1>, <32x120x1x1>, <40x144x1x1> ...)
+    assert [spec.squeeze_channels(e) for e in (16, 96, 240, 120, 144, 288, 576)] == [8, 24, 64, 32, 40, 72, 144]
+
+
+@pytest.mark.skipif(not os.path.exists(FIXTURE), reason="reference checkout not present")
+def test_conv_table_matches_the_reference_fixture():
+    text = open(FIXTURE).read()
+    assert text.count("dense_resource<__elided__>") == spec.NUM_TENSORS
+    assert "arith.constant 1.000000e-03 : f64" in text  # BatchNorm epsilon
+    pat = re.compile(r"linalg\.(conv_2d_nchw_fchw|depthwise_conv_2d_nchw_chw) \{dilations = dense<1> : vector<2xi64>, "
+                     r"strides = dense<(\d+)> : vector<2xi64>\} ins\(%\w+, %\w+ : tensor<1x(\d+)x(\d+)x(\d+)xf32>, "
+                     r"tensor<([0-9x]+)xf32>\)")
+    got = []
+    for m in pat.finditer(text):
+        kind = "dw" if m.group(1).startswith("depthwise") else "conv"
+        stride, c, hp = int(m.group(2)), int(m.group(3)), int(m.group(4))
+        wshape = [int(v) for v in m.group(6).split("x")]
+        k = wshape[-1]
+        f = wshape[0]
+        got.append((kind, c, f, k, stride, hp - 2 * ((k - 1) // 2)))  # the fixture's input is already padded
+    assert got == spec.conv_table(256)
+    assert len(got) == 52 and sum(1 for g in got if g[0] == "dw") == 11
+
+
+def test_builtin_operator_list_equals_the_python_one():
+    ops, n_elems = abi.mobilenetv3_small_ops()
+    mine = spec.graph_ops()
+    assert n_elems == spec.NUM_ELEMENTS and len(ops) == len(mine)
+    for a, b in zip(ops, mine):
+        for name, _ in abi.GraphOp._fields_:
+            va, vb = getattr(a, name), getattr(b, name)
+            if name == "inputs":
+                va, vb = list(va), list(vb)
+            assert va == vb or (name == "eps" and abs(va - vb) < 1e-9), (name, va, vb, a.out)
+
+
+@pytest.mark.parametrize("k,stride", [(3, 1), (3, 2), (5, 1), (5, 2)])
+def test_depthwise_conv_vs_torch(k, stride):
+    rng = np.random.default_rng(k * 10 + stride)
+    x = rng.normal(0, 1, (2, 24, 13, 17)).astype(np.float32)
+    w = rng.normal(0, 0.3, (24, 1, k, k)).astype(np.float32)
+    pad = (k - 1) // 2
+    want = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(w).double(), stride=stride, padding=pad, groups=24).numpy()
+    got = oracle.depthwise_conv2d_nchw_chw(oracle.pad_nchw(x, pad), w, stride)
+    assert got.shape == want.shape and close(got, want)
+    # a transposed filter or swapped stride must not pass
+    assert not close(oracle.depthwise_conv2d_nchw_chw(oracle.pad_nchw(x, pad), np.swapaxes(w, 2, 3).copy(), stride), want, 1e-3)
+
+
+def test_activations_vs_torch_and_special_values():
+    x = np.concatenate([np.linspace(-8, 8, 4001), [-3.0, 3.0, 0.0, -0.0, 6.0, -6.0]]).astype(np.float32)
+    xt = torch.from_numpy(x).double()
+    assert close(oracle.hardswish(x), F.hardswish(xt).numpy())
+    assert close(oracle.hardsigmoid(x), F.hardsigmoid(xt).numpy())
+    assert close(oracle.silu(x), F.silu(xt).numpy())
+    assert close(oracle.sigmoid(x), torch.sigmoid(xt).numpy())
+    # closed forms: saturation and the knees
+    assert oracle.hardswish(np.float32([-3, -4, 3, 7, 0])).tolist() == [0.0, 0.0, 3.0, 7.0, 0.0]
+    assert oracle.hardsigmoid(np.float32([-3, -9, 3, 9, 0])).tolist() == [0.0, 0.0, 1.0, 1.0, 0.5]
+    # the fixture's predicates: NaN passes through both, infinities saturate
+    assert np.isnan(oracle.hardswish(np.float32([np.nan]))[0]) and np.isnan(oracle.hardsigmoid(np.float32([np.nan]))[0])
+    assert oracle.hardsigmoid(np.float32([np.inf, -np.inf])).tolist() == [1.0, 0.0]
+    assert oracle.hardswish(np.float32([np.inf]))[0] == np.inf
+
+
+def test_batchnorm_eps_vs_torch():
+    rng = np.random.default_rng(5)
+    x = rng.normal(0, 2, (2, 16, 5, 7)).astype(np.float32)
+    g, b, m = (rng.normal(0, 1, 16).astype(np.float32) for _ in range(3))
+    v = rng.uniform(1e-4, 2, 16).astype(np.float32)  # small variances make the epsilon matter
+    want = F.batch_norm(torch.from_numpy(x).double(), torch.from_numpy(m).double(), torch.from_numpy(v).double(),
+                        torch.from_numpy(g).double(), torch.from_numpy(b).double(), False, 0.0, float(np.float32(1e-3))).numpy()
+    assert close(oracle.batchnorm_eps(x, g, b, m, v, 1e-3), want, 1e-5)
+    assert not close(oracle.batchnorm_eps(x, g, b, m, v, 1e-5), want, 1e-3)
+
+
+def test_pool_upsample_vs_torch():
+    rng = np.random.default_rng(6)
+    x = rng.normal(0, 1, (2, 8, 11, 9)).astype(np.float32)
+    xt = torch.from_numpy(x)
+    assert np.array_equal(oracle.maxpool_nchw(x, 5, 1, 2), F.max_pool2d(xt, 5, 1, 2).numpy())
+    assert np.array_equal(oracle.maxpool_nchw(x, 3, 2, 1), F.max_pool2d(xt, 3, 2, 1).numpy())
+    assert np.array_equal(oracle.maxpool_nchw(x, 2, 2, 0), F.max_pool2d(xt, 2, 2, 0).numpy())
+    assert np.array_equal(oracle.upsample2x_nearest(x), F.interpolate(xt, scale_factor=2, mode="nearest").numpy())
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 64, 64), (1, 3, 96, 72)])
+def test_mobilenetv3_oracle_vs_torch(shape):
+    blob = synth.mobilenetv3_params()
+    T = tensors_of(blob)
+    x = synth.uniform(6000, shape, 0.0, 1.0)
+    taps = []
+    got = oracle.mobilenetv3_forward(x, T, taps)
+    want, want_taps = torch_mobilenetv3(x, T)
+    assert got.shape == (shape[0], 1000)
+    for a, b in zip(taps, want_taps):
+        assert a.shape == b.shape and close(a, b, 2e-5)
+    assert close(got, want, 2e-5)
+    assert np.array_equal(got.argmax(1), want.argmax(1))
+    # the operator-list evaluator (what the graph executor is checked against) says the same
+    got2 = oracle.run_graph(spec.graph_ops(), x, blob, 3).reshape(shape[0], 1000)
+    assert close(got2, want, 2e-5)
+
+
+def test_mobilenetv3_oracle_batch_independent():
+    blob = synth.mobilenetv3_params()
+    T = tensors_of(blob)
+    x = synth.uniform(6001, (3, 3, 64, 64), 0.0, 1.0)
+    full = oracle.mobilenetv3_forward(x, T)
+    one = oracle.mobilenetv3_forward(x[1:2], T)
+    assert np.array_equal(full[1:2], one)

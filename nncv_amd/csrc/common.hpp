@@ -202,6 +202,14 @@ void launch_dwconv(const DwConvArgs& a, int dt, hipStream_t s);
 void launch_weight_dw(const void* w, int w_dt, void* dst, int dst_dt, int C, int K, hipStream_t s);
 // out[n,p,c] = x[n,p,c] * g[n,c]   (squeeze-excitation gate; MobileNetV3.mlir:380-384)
 void launch_scale_channels(const void* x, const void* g, void* out, int dt, int N, int HW, int C, hipStream_t s);
+// Whole squeeze-excitation block: out = x * act2(W2 . act1(W1 . mean_hw(x) + b1) + b2), one launch.
+// w1 [SQ][C], w2 [C][SQ] of type dt; b1, b2 fp32.
+struct SeArgs {
+  const void* x; const void* w1; const float* b1; const void* w2; const float* b2; void* out;
+  int N, HW, C, SQ, act1, act2;
+};
+bool se_block_applicable(int dt, int HW, int C, int SQ);
+void launch_se_block(const SeArgs& a, int dt, hipStream_t s);
 // out = act(a (+ b));  b may be null;  n elements, n a multiple of the 16-byte vector
 void launch_eltwise(const void* a, const void* b, void* out, int dt, long long n, int act, hipStream_t s);
 // copies x [P][C] into channels [c0, c0 + C) of out [P][ldo]   (torch.cat over channels, NHWC)

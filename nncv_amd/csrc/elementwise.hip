@@ -38,74 +38,126 @@ inline unsigned grid_for(long long work) {
 }  // namespace
 
 // ---------------------------------------------------------------------------------------------
-// Depthwise convolution.  One thread = one output pixel x one channel group; the K*K input
-// vectors it needs are shared with its neighbours through L1/L2 (the maps of the MobileNet
-// stages are at most a few MB).  fp32 accumulation in (kh, kw) order like the reference's loop
-// nest; scale/shift (folded BatchNorm) and the activation are applied before the one rounding.
+// Depthwise convolution.  One thread = OXT horizontally adjacent output pixels x one channel
+// group: per filter row it loads the (OXT-1)*S + K input vectors the strip needs once and each
+// filter tap once, instead of K*K of both per output pixel -- the kernel is bound by the number of
+// vector-memory instructions, not by HBM (the maps of the MobileNet stages are a few MB and the
+// halo reuse between neighbouring threads is served by L1/L2).  fp32 accumulation in (kh, kw)
+// order like the reference's loop nest; scale/shift (folded BatchNorm) and the activation are
+// applied before the one rounding.
 // ---------------------------------------------------------------------------------------------
-template <typename T, int K>
-__global__ __launch_bounds__(256) void dwconv_kernel(const DwConvArgs a) {
+template <typename T, int K, int S, int OXT>
+__global__ __launch_bounds__(128) void dwconv_kernel(const DwConvArgs a, int strips) {
   constexpr int VN = V16<T>::n;
+  constexpr int LW = (OXT - 1) * S + K;  // input pixels one strip touches per filter row
   typedef typename V16<T>::type V;
   const int CG = a.C / VN;
   const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= (long long)a.N * a.OH * a.OW * CG) return;
+  if (idx >= (long long)a.N * a.OH * strips * CG) return;
   const int cg = (int)(idx % CG);
   long long p = idx / CG;
-  const int ox = (int)(p % a.OW);
-  p /= a.OW;
+  const int sx = (int)(p % strips);
+  p /= strips;
   const int oy = (int)(p % a.OH);
   const int n = (int)(p / a.OH);
+  const int ox0 = sx * OXT;
   const T* in = static_cast<const T*>(a.in) + (long long)n * a.H * a.W * a.C + cg * VN;
   const T* wt = static_cast<const T*>(a.wt) + cg * VN;
-  float acc[VN];
+  const int ix0 = ox0 * S - a.pad;
+  float acc[OXT][VN];
 #pragma unroll
-  for (int e = 0; e < VN; ++e) acc[e] = 0.0f;
+  for (int j = 0; j < OXT; ++j)
+#pragma unroll
+    for (int e = 0; e < VN; ++e) acc[j][e] = 0.0f;
+  // Every load is unconditional from a clamped address and zeroed afterwards when it lies in the
+  // halo: no control flow in the tap loops, so the loads of all rows can be in flight together.
 #pragma unroll
   for (int r = 0; r < K; ++r) {
-    const int iy = oy * a.stride - a.pad + r;
-    if ((unsigned)iy >= (unsigned)a.H) continue;
+    const int iy = oy * S - a.pad + r;
+    const bool rok = (unsigned)iy < (unsigned)a.H;
+    const T* row = in + (long long)min(max(iy, 0), a.H - 1) * a.W * a.C;
+    V x[LW];
+#pragma unroll
+    for (int q = 0; q < LW; ++q) {
+      const int ix = ix0 + q;
+      const bool ok = rok && (unsigned)ix < (unsigned)a.W;
+      x[q] = *reinterpret_cast<const V*>(row + (long long)min(max(ix, 0), a.W - 1) * a.C);
+      if (!ok) {
+#pragma unroll
+        for (int e = 0; e < VN; ++e) x[q][e] = (T)0.0f;
+      }
+    }
 #pragma unroll
     for (int s = 0; s < K; ++s) {
-      const int ix = ox * a.stride - a.pad + s;
-      if ((unsigned)ix >= (unsigned)a.W) continue;
-      const V x = *reinterpret_cast<const V*>(in + ((long long)iy * a.W + ix) * a.C);
       const V w = *reinterpret_cast<const V*>(wt + (r * K + s) * a.C);
 #pragma unroll
-      for (int e = 0; e < VN; ++e) acc[e] += (float)x[e] * (float)w[e];
+      for (int j = 0; j < OXT; ++j)
+#pragma unroll
+        for (int e = 0; e < VN; ++e) acc[j][e] += (float)x[j * S + s][e] * (float)w[e];
     }
   }
-  V o;
+  float sc[VN], sh[VN];
 #pragma unroll
   for (int e = 0; e < VN; ++e) {
-    float y = acc[e];
-    if (a.scale) y *= a.scale[cg * VN + e];
-    if (a.shift) y += a.shift[cg * VN + e];
-    o[e] = (T)act_apply(y, a.act);
+    sc[e] = a.scale ? a.scale[cg * VN + e] : 1.0f;
+    sh[e] = a.shift ? a.shift[cg * VN + e] : 0.0f;
   }
-  *reinterpret_cast<V*>(static_cast<T*>(a.out) + (((long long)n * a.OH + oy) * a.OW + ox) * a.C + cg * VN) = o;
+  T* out = static_cast<T*>(a.out) + (((long long)n * a.OH + oy) * a.OW) * a.C + cg * VN;
+#pragma unroll
+  for (int j = 0; j < OXT; ++j) {
+    if (ox0 + j >= a.OW) break;
+    V o;
+#pragma unroll
+    for (int e = 0; e < VN; ++e) o[e] = (T)act_apply(acc[j][e] * sc[e] + sh[e], a.act);
+    *reinterpret_cast<V*>(out + (long long)(ox0 + j) * a.C) = o;
+  }
+}
+
+template <typename T, int K, int S, int OXT>
+static void launch_dwconv_oxt(const DwConvArgs& a, hipStream_t s) {
+  const int strips = (a.OW + OXT - 1) / OXT;
+  const long long work = (long long)a.N * a.OH * strips * (a.C / V16<T>::n);
+  const long long grid = (work + 127) / 128;
+  NNCV_REQUIRE(grid >= 1 && grid < (1ll << 31), "dwconv: grid out of range");
+  hipLaunchKernelGGL((dwconv_kernel<T, K, S, OXT>), dim3((unsigned)grid), dim3(128), 0, s, a, strips);
+}
+
+// A lane-FMA is all the arithmetic there is (a wave retires one per 4 cycles), so the launch is as
+// long as the FMA chain of one thread unless there are many waves per CU to interleave.  Strips
+// of 4 or 2 outputs per thread save vector loads, but only pay once the grid is large enough to
+// fill the machine with them (256 CUs x 8 waves).
+template <typename T, int K, int S>
+static void launch_dwconv_cfg(const DwConvArgs& a, hipStream_t s) {
+  const long long vecs = (long long)a.N * a.OH * (a.C / V16<T>::n);
+  auto waves = [&](int oxt) { return vecs * ((a.OW + oxt - 1) / oxt) / 64; };
+  if (waves(4) >= 2048 && !(K == 5 && S == 2)) launch_dwconv_oxt<T, K, S, 4>(a, s);
+  else if (waves(2) >= 2048) launch_dwconv_oxt<T, K, S, 2>(a, s);
+  else launch_dwconv_oxt<T, K, S, 1>(a, s);
 }
 
 void launch_dwconv(const DwConvArgs& a, int dt, hipStream_t s) {
   const int vn = dt == kF16 ? 8 : 4;
   NNCV_REQUIRE(a.K == 3 || a.K == 5, "dwconv: kernel size must be 3 or 5");
+  NNCV_REQUIRE(a.stride == 1 || a.stride == 2, "dwconv: stride must be 1 or 2");
   NNCV_REQUIRE(a.C % vn == 0, "dwconv: C must be a multiple of the 16-byte vector");
-  NNCV_REQUIRE(a.stride >= 1 && a.pad >= 0 && a.N >= 1 && a.H >= 1 && a.W >= 1, "dwconv: bad geometry");
+  NNCV_REQUIRE(a.pad >= 0 && a.N >= 1 && a.H >= 1 && a.W >= 1, "dwconv: bad geometry");
   NNCV_REQUIRE(a.OH == (a.H + 2 * a.pad - a.K) / a.stride + 1 && a.OW == (a.W + 2 * a.pad - a.K) / a.stride + 1 && a.OH >= 1 &&
                    a.OW >= 1,
                "dwconv: output size does not match input/filter/stride/pad");
-  const long long work = (long long)a.N * a.OH * a.OW * (a.C / vn);
-  const unsigned grid = grid_for(work);
   const double px_in = (double)a.N * a.H * a.W, px_out = (double)a.N * a.OH * a.OW;
   ProfScope prof(a.K == 3 ? "dwconv3x3" : "dwconv5x5", 2.0 * px_out * a.C * a.K * a.K,
                  (double)dtype_size(dt) * a.C * (px_in + px_out + a.K * a.K), s);
-#define LAUNCH(T, KK) hipLaunchKernelGGL((dwconv_kernel<T, KK>), dim3(grid), dim3(256), 0, s, a)
-  if (dt == kF16) {
-    if (a.K == 3) LAUNCH(half_t, 3); else LAUNCH(half_t, 5);
-  } else {
-    if (a.K == 3) LAUNCH(float, 3); else LAUNCH(float, 5);
+  const int sel = (dt == kF16 ? 0 : 4) + (a.K == 3 ? 0 : 2) + (a.stride == 1 ? 0 : 1);
+  switch (sel) {
+    case 0: launch_dwconv_cfg<half_t, 3, 1>(a, s); break;
+    case 1: launch_dwconv_cfg<half_t, 3, 2>(a, s); break;
+    case 2: launch_dwconv_cfg<half_t, 5, 1>(a, s); break;
+    case 3: launch_dwconv_cfg<half_t, 5, 2>(a, s); break;
+    case 4: launch_dwconv_cfg<float, 3, 1>(a, s); break;
+    case 5: launch_dwconv_cfg<float, 3, 2>(a, s); break;
+    case 6: launch_dwconv_cfg<float, 5, 1>(a, s); break;
+    default: launch_dwconv_cfg<float, 5, 2>(a, s); break;
   }
-#undef LAUNCH
   NNCV_HIP_CHECK(hipGetLastError());
 }
 
@@ -163,6 +215,161 @@ void launch_scale_channels(const void* x, const void* g, void* out, int dt, int 
   else
     hipLaunchKernelGGL((scale_channels_kernel<float>), dim3(grid_for(total)), dim3(256), 0, s, (const float*)x, (const float*)g,
                        (float*)out, total, HW * CG, CG);
+  NNCV_HIP_CHECK(hipGetLastError());
+}
+
+// ---------------------------------------------------------------------------------------------
+// Squeeze-excitation block in one launch (MobileNetV3.mlir:322-384): global average pool, 1x1
+// convolution + bias + act1 (C -> SQ), 1x1 convolution + bias + act2 (SQ -> C), and the gate
+// multiplied back onto the input.  One workgroup per image: its activation (at most a few
+// hundred KB in these networks) is read twice, the second time out of L2, and nothing but the
+// gated result is written.  The pooled vector, the squeezed vector and the gate stay in fp32 in
+// LDS -- they are never rounded to the storage type.  1024 threads and batched loads, because
+// with one workgroup per image the launch is as long as its longest chain of dependent loads.
+// ---------------------------------------------------------------------------------------------
+constexpr int kSeMaxC = 1024, kSeMaxSq = 256, kSeThreads = 1024;
+
+template <typename T>
+__global__ __launch_bounds__(kSeThreads) void se_block_kernel(const SeArgs a) {
+  constexpr int VN = V16<T>::n;
+  constexpr int NT = kSeThreads, NW = NT / 64;
+  typedef typename V16<T>::type V;
+  __shared__ float part[NT * VN];
+  __shared__ float mean[kSeMaxC];
+  __shared__ float hid[kSeMaxSq];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n = blockIdx.x;
+  const int CG = a.C / VN;
+  const T* __restrict__ x = static_cast<const T*>(a.x) + (long long)n * a.HW * a.C;
+
+  // 1. pool: thread = (pixel phase pp, channel group cg), eight loads in flight
+  const int ppb = NT / CG;  // CG <= 256
+  const int pp = tid / CG, cg = tid - pp * CG;
+  if (pp < ppb) {
+    float acc[VN];
+#pragma unroll
+    for (int e = 0; e < VN; ++e) acc[e] = 0.0f;
+    constexpr int U = 8;
+    for (int p = pp; p < a.HW; p += U * ppb) {
+      V v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = *reinterpret_cast<const V*>(x + (long long)min(p + u * ppb, a.HW - 1) * a.C + cg * VN);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (p + u * ppb < a.HW) {
+#pragma unroll
+          for (int e = 0; e < VN; ++e) acc[e] += (float)v[u][e];
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < VN; ++e) part[tid * VN + e] = acc[e];
+  }
+  __syncthreads();
+  // the ppb partial rows (C floats each, row q at part[q * C]) are folded in two steps so that a
+  // narrow tensor (C = 16: 512 rows) is not one thread's chain of 512 dependent LDS reads
+  const int GA = min(ppb, max(1, NT / a.C));
+  {
+    const int g = tid / a.C, c = tid - g * a.C;
+    if (g < GA) {
+      float s = 0.0f;
+#pragma unroll 8
+      for (int q = g; q < ppb; q += GA) s += part[q * a.C + c];
+      part[g * a.C + c] = s;  // row g is read by this thread only
+    }
+  }
+  __syncthreads();
+  for (int c = tid; c < a.C; c += NT) {
+    float s = 0.0f;
+#pragma unroll 8
+    for (int q = 0; q < GA; ++q) s += part[q * a.C + c];
+    mean[c] = s / (float)a.HW;
+  }
+  __syncthreads();
+
+  // 2. squeeze: a wave takes four outputs at a time, lanes along C
+  const T* __restrict__ w1 = static_cast<const T*>(a.w1);
+  constexpr int JB = 4;
+  for (int j0 = wave; j0 < a.SQ; j0 += NW * JB) {
+    float s[JB];
+#pragma unroll
+    for (int b = 0; b < JB; ++b) s[b] = 0.0f;
+    for (int v = lane; v < CG; v += 64) {
+      V w[JB];
+#pragma unroll
+      for (int b = 0; b < JB; ++b) w[b] = *reinterpret_cast<const V*>(w1 + (long long)min(j0 + b * NW, a.SQ - 1) * a.C + v * VN);
+#pragma unroll
+      for (int b = 0; b < JB; ++b)
+#pragma unroll
+        for (int e = 0; e < VN; ++e) s[b] += mean[v * VN + e] * (float)w[b][e];
+    }
+#pragma unroll
+    for (int b = 0; b < JB; ++b) {
+#pragma unroll
+      for (int o = 32; o >= 1; o >>= 1) s[b] += __shfl_xor(s[b], o);
+      const int j = j0 + b * NW;
+      if (lane == 0 && j < a.SQ) hid[j] = act_apply(s[b] + a.b1[j], a.act1);
+    }
+  }
+  __syncthreads();
+
+  // 3. excite: one thread per channel, six filter vectors in flight; the gate overwrites the means
+  const T* __restrict__ w2 = static_cast<const T*>(a.w2);
+  const int SG = a.SQ / VN;
+  for (int c = tid; c < a.C; c += NT) {
+    float s = 0.0f;
+    constexpr int U = 6;
+    for (int v0 = 0; v0 < SG; v0 += U) {
+      V w[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) w[u] = *reinterpret_cast<const V*>(w2 + (long long)c * a.SQ + min(v0 + u, SG - 1) * VN);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (v0 + u < SG) {
+#pragma unroll
+          for (int e = 0; e < VN; ++e) s += hid[(v0 + u) * VN + e] * (float)w[u][e];
+        }
+    }
+    mean[c] = act_apply(s + a.b2[c], a.act2);
+  }
+  __syncthreads();
+
+  // 4. gate the image, four vectors in flight per thread
+  T* __restrict__ out = static_cast<T*>(a.out) + (long long)n * a.HW * a.C;
+  const int total = a.HW * CG;
+  constexpr int UG = 4;
+  for (int i0 = tid; i0 < total; i0 += UG * NT) {
+    V xv[UG];
+#pragma unroll
+    for (int u = 0; u < UG; ++u) xv[u] = *reinterpret_cast<const V*>(x + (long long)min(i0 + u * NT, total - 1) * VN);
+#pragma unroll
+    for (int u = 0; u < UG; ++u) {
+      const int i = i0 + u * NT;
+      if (i < total) {
+        const int g = i % CG;
+        V o;
+#pragma unroll
+        for (int e = 0; e < VN; ++e) o[e] = (T)(mean[g * VN + e] * (float)xv[u][e]);
+        *reinterpret_cast<V*>(out + (long long)i * VN) = o;
+      }
+    }
+  }
+}
+
+bool se_block_applicable(int dt, int HW, int C, int SQ) {
+  const int vn = dt == kF16 ? 8 : 4;
+  return C % vn == 0 && SQ % vn == 0 && C / vn <= 256 && C <= kSeMaxC && SQ <= kSeMaxSq && HW >= 1 &&
+         (long long)HW * C < (1ll << 31);
+}
+
+void launch_se_block(const SeArgs& a, int dt, hipStream_t s) {
+  NNCV_REQUIRE(se_block_applicable(dt, a.HW, a.C, a.SQ), "se_block: shape not covered");
+  NNCV_REQUIRE(a.N >= 1 && a.b1 && a.b2, "se_block: bad arguments");
+  const double es = (double)dtype_size(dt);
+  ProfScope prof("se_block", 4.0 * a.N * a.C * a.SQ + 2.0 * a.N * a.HW * a.C, es * (2.0 * a.N * a.HW * a.C + 2.0 * a.C * a.SQ), s);
+  if (dt == kF16)
+    hipLaunchKernelGGL((se_block_kernel<half_t>), dim3(a.N), dim3(kSeThreads), 0, s, a);
+  else
+    hipLaunchKernelGGL((se_block_kernel<float>), dim3(a.N), dim3(kSeThreads), 0, s, a);
   NNCV_HIP_CHECK(hipGetLastError());
 }
 

@@ -159,6 +159,26 @@ Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, lon
     channels_[op.out] = Cout;
   }
   for (int t = 1; t < n_tensors_; ++t) NNCV_REQUIRE(channels_[t] > 0, "graph: tensor " + std::to_string(t) + " is never produced");
+
+  // squeeze-excitation blocks
+  static const bool no_se = getenv("NNCV_HIP_NO_SE_FUSION") != nullptr;
+  std::vector<int> readers(n_tensors_, 0);
+  for (int i = 0; i < n; ++i)
+    for (int k = 0; k < 4; ++k)
+      if (ops[i].in[k] >= 0) ++readers[ops[i].in[k]];
+  auto plain_fc = [&](const GraphOp& o, int in) {
+    return o.kind == NNCV_HIP_OP_CONV && o.K == 1 && o.stride == 1 && o.pad == 0 && o.in[0] == in && o.in[1] < 0 && o.bias >= 0 &&
+           o.gamma < 0 && readers[in] == 1;
+  };
+  for (int i = 0; !no_se && i + 3 < n; ++i) {
+    const GraphOp &p0 = ops[i], &f1 = ops[i + 1], &f2 = ops[i + 2], &sc = ops[i + 3];
+    if (p0.kind != NNCV_HIP_OP_GAVGPOOL || p0.in[0] == 0 || !plain_fc(f1, p0.out) || !plain_fc(f2, f1.out)) continue;
+    if (sc.kind != NNCV_HIP_OP_SCALE || sc.in[0] != p0.in[0] || sc.in[1] != f2.out || readers[f2.out] != 1) continue;
+    if (f2.F != channels_[p0.in[0]] || !se_block_applicable(dt, 1, f2.F, f1.F)) continue;
+    nodes_[i].se_head = true;
+    nodes_[i + 1].skip = nodes_[i + 2].skip = nodes_[i + 3].skip = true;
+    i += 3;
+  }
 }
 
 const Graph::Plan& Graph::plan_of(int N, int H, int W) const {
@@ -237,9 +257,20 @@ void Graph::forward(const void* src, int N, int H, int W, float* out, void* ws, 
   auto at = [&](int t) -> void* { return base + p.offset[t]; };
   launch_relayout(src, dt_, strides_of(kNCHW, c_in_, H, W), at(0), dt_, strides_of(kNHWC, channels_[0], H, W), N, c_in_,
                   channels_[0], H, W, false, s);
-  for (const Node& nd : nodes_) {
+  for (size_t i = 0; i < nodes_.size(); ++i) {
+    const Node& nd = nodes_[i];
     const GraphOp& op = nd.op;
     const Dims a = p.dims[op.in[0]], o = p.dims[op.out];
+    if (nd.skip) continue;
+    if (nd.se_head) {
+      const Node &f1 = nodes_[i + 1], &f2 = nodes_[i + 2];
+      SeArgs e{};
+      e.x = at(op.in[0]); e.w1 = f1.wt.get(); e.b1 = f1.shift.as<float>(); e.w2 = f2.wt.get(); e.b2 = f2.shift.as<float>();
+      e.out = at(nodes_[i + 3].op.out);
+      e.N = N; e.HW = a.H * a.W; e.C = a.C; e.SQ = f1.op.F; e.act1 = f1.op.act; e.act2 = f2.op.act;
+      launch_se_block(e, dt_, s);
+      continue;
+    }
     switch (op.kind) {
       case NNCV_HIP_OP_CONV: {
         IgemmArgs g{};

@@ -99,9 +99,70 @@ __global__ __launch_bounds__(256) void global_avgpool_kernel(const T* __restrict
   }
 }
 
+// Whole-vector form for C % (16 bytes) == 0: a workgroup owns one image x up to 32 channel
+// groups; its threads split into pixel phases x channel groups, keep four 16-byte loads in
+// flight each, and meet in LDS.  Same arithmetic (fp32 sums, one divide).
+template <typename T>
+__global__ __launch_bounds__(256) void global_avgpool_vec_kernel(const T* __restrict__ in, T* __restrict__ out, int HW, int C,
+                                                                 int cgb) {
+  constexpr int VN = Vec16<T>::n;
+  typedef typename Vec16<T>::type V;
+  __shared__ float part[256 * VN];
+  const int tid = threadIdx.x, n = blockIdx.y;
+  const int CG = C / VN;
+  const int g0 = blockIdx.x * cgb;
+  const int ng = min(cgb, CG - g0);  // channel groups of this workgroup
+  const int ppb = 256 / ng;
+  const int pp = tid / ng, cg = g0 + (tid - pp * ng);
+  const T* x = in + (long long)n * HW * C + cg * VN;
+  float acc[VN];
+#pragma unroll
+  for (int e = 0; e < VN; ++e) acc[e] = 0.0f;
+  if (pp < ppb) {
+    int p = pp;
+    for (; p + 3 * ppb < HW; p += 4 * ppb) {
+      V v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const V*>(x + (long long)(p + u * ppb) * C);
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int e = 0; e < VN; ++e) acc[e] += (float)v[u][e];
+    }
+    for (; p < HW; p += ppb) {
+      const V v = *reinterpret_cast<const V*>(x + (long long)p * C);
+#pragma unroll
+      for (int e = 0; e < VN; ++e) acc[e] += (float)v[e];
+    }
+#pragma unroll
+    for (int e = 0; e < VN; ++e) part[tid * VN + e] = acc[e];
+  }
+  __syncthreads();
+  if (tid < ng * VN) {
+    const int g = tid / VN, e = tid % VN;
+    float s = 0.0f;
+    for (int q = 0; q < ppb; ++q) s += part[(q * ng + g) * VN + e];
+    out[(long long)n * C + (g0 + g) * VN + e] = (T)(s / (float)HW);
+  }
+}
+
 void launch_global_avgpool_nhwc(const void* in, void* out, int dt, int N, int HW, int C, hipStream_t s) {
-  dim3 grid((C + 63) / 64, N);
   ProfScope prof("global_avgpool", 0.0, (double)dtype_size(dt) * N * C * (HW + 1.0), s);
+  const int vn = dt == kF16 ? 8 : 4;
+  if (C % vn == 0) {
+    const int CG = C / vn;
+    // fewer channel groups per workgroup when that is what it takes to give every CU one
+    int cgb = 32;
+    while (cgb > 2 && (long long)((CG + cgb - 1) / cgb) * N < 256) cgb >>= 1;
+    dim3 grid((CG + cgb - 1) / cgb, N);
+    if (dt == kF16)
+      hipLaunchKernelGGL((global_avgpool_vec_kernel<half_t>), grid, dim3(256), 0, s, (const half_t*)in, (half_t*)out, HW, C, cgb);
+    else
+      hipLaunchKernelGGL((global_avgpool_vec_kernel<float>), grid, dim3(256), 0, s, (const float*)in, (float*)out, HW, C, cgb);
+    NNCV_HIP_CHECK(hipGetLastError());
+    return;
+  }
+  dim3 grid((C + 63) / 64, N);
   if (dt == kF16)
     hipLaunchKernelGGL((global_avgpool_kernel<half_t>), grid, dim3(256), 0, s, (const half_t*)in, (half_t*)out, HW, C);
   else

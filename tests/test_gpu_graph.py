@@ -294,3 +294,34 @@ def test_graph_create_refuses_malformed_lists():
     assert "K must be 3 or 5" in refused(clone(1, kind=abi.OP_DWCONV, K=7, w=0))
     assert "unknown activation" in refused(clone(10, act=9))
     assert "channel" in refused(clone(8, inputs=(ctypes.c_int32 * 4)(8, 6, -1, -1)))            # residual with 2C channels
+
+
+@pytest.mark.parametrize("dt", [abi.F32, abi.F16])
+@pytest.mark.parametrize("C,SQ,H,W,N", [(16, 8, 56, 56, 2), (576, 144, 7, 7, 3), (240, 64, 14, 14, 1), (96, 24, 5, 3, 2)])
+def test_squeeze_excitation_block(dt, C, SQ, H, W, N):
+    """pool -> fc + ReLU -> fc + hard-sigmoid -> gate, which the executor runs as one launch."""
+    sizes, ops = [], []
+
+    def take(n):
+        off = sum(sizes)
+        sizes.append(n)
+        return off
+
+    ops.append(abi.graph_op(abi.OP_ACT, [0], 1, act=abi.ACT_NONE, stride=0))
+    ops.append(abi.graph_op(abi.OP_GAVGPOOL, [1], 2, stride=0))
+    ops.append(abi.graph_op(abi.OP_CONV, [2], 3, F=SQ, K=1, act=abi.ACT_RELU, w=take(SQ * C), bias=take(SQ)))
+    ops.append(abi.graph_op(abi.OP_CONV, [3], 4, F=C, K=1, act=abi.ACT_HARDSIGMOID, w=take(C * SQ), bias=take(C)))
+    ops.append(abi.graph_op(abi.OP_SCALE, [1, 4], 5, stride=0))
+    blob = synth.normal(7600, (sum(sizes),), std=0.3)
+    x = synth.normal(7601, (N, C, H, W))
+    if dt == abi.F16:
+        blob, x = r16(blob), r16(x)
+    g = Graph(ops, C, blob, dt)
+    print("se block", dt, C, SQ, H, W, N, flush=True)
+    got = host(g(dev(x, dt)))
+    want = oracle.run_graph(ops, x, blob, C)
+    if dt == abi.F32:
+        assert max_rel(got, want) < FP32_MAX_REL
+    else:
+        assert rel_l2(got, want) < 2e-3
+    g.close()

@@ -169,6 +169,13 @@ int nncv_hip_global_avgpool(int dtype, const void* in, void* out, int N, int H, 
 #define NNCV_HIP_OP_ACT 7         /* out = act(in[0]) */
 #define NNCV_HIP_OP_CONCAT 8      /* out = concat over channels of in[0..3] (unused = -1) */
 #define NNCV_HIP_OP_UPSAMPLE2X 9  /* nearest-neighbour, H and W doubled */
+/* YOLOv5 Detect decode (tests/Nets/Yolov5s.mlir:1348-1448), only as the LAST operator: in[0..2] are the
+ * head tensors of up to three levels, each with K * F channels (K anchors per level, F = 5 + classes
+ * values per anchor). w: anchors [levels,K,2] in units of the level's stride, bias: strides [levels].
+ * s = sigmoid(head); xy = (2 s + grid - 0.5) * stride; wh = (2 s)^2 * anchor * stride; the rest is s.
+ * Network output: [N, sum_l K*H_l*W_l, F] fp32, boxes ordered (level, anchor, y, x); reported by
+ * nncv_hip_graph_output_shape as channels = boxes, height = F, width = 1. */
+#define NNCV_HIP_OP_YOLO_DETECT 10
 
 #define NNCV_HIP_ACT_NONE 0
 #define NNCV_HIP_ACT_RELU 1         /* select(x ugt 0, x, 0) */
@@ -191,8 +198,10 @@ typedef struct nncv_hip_graph_op {
 } nncv_hip_graph_op;
 
 typedef struct nncv_hip_graph nncv_hip_graph;
-/* params: HOST pointer to n_elems elements of `dtype`. Channel counts other than the input's must
- * be multiples of 8 (fp16) / 4 (fp32). Returns NULL on error (nncv_hip_last_error). */
+/* params: HOST pointer to n_elems elements of `dtype`. Channel counts that are not multiples of 8
+ * (fp16) / 4 (fp32) are allowed for the network input and for convolution outputs that feed only
+ * convolutions, YOLO_DETECT or the network output (they are stored padded). Returns NULL on error
+ * (nncv_hip_last_error). */
 nncv_hip_graph* nncv_hip_graph_create(const nncv_hip_graph_op* ops, int n_ops, int in_channels, const void* params,
                                       int64_t n_elems, int dtype);
 void nncv_hip_graph_destroy(nncv_hip_graph* g);

@@ -45,7 +45,7 @@ EXPORTS = [
 ]
 
 # operator kinds / activations of nncv_hip_graph_op (include/nncv_hip.h)
-OP_CONV, OP_DWCONV, OP_MAXPOOL, OP_GAVGPOOL, OP_SCALE, OP_ADD, OP_ACT, OP_CONCAT, OP_UPSAMPLE2X = range(1, 10)
+OP_CONV, OP_DWCONV, OP_MAXPOOL, OP_GAVGPOOL, OP_SCALE, OP_ADD, OP_ACT, OP_CONCAT, OP_UPSAMPLE2X, OP_YOLO_DETECT = range(1, 11)
 ACT_NONE, ACT_RELU, ACT_HARDSWISH, ACT_HARDSIGMOID, ACT_SILU, ACT_SIGMOID = range(6)
 
 

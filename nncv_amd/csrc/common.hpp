@@ -219,6 +219,13 @@ void launch_upsample2x(const void* x, void* out, int dt, int N, int H, int W, in
 // max-pool K x K, any stride / padding (-inf halo), NHWC
 void launch_maxpool_nhwc(const void* in, void* out, int dt, int N, int H, int W, int C, int K, int stride, int pad,
                          hipStream_t s);
+// YOLOv5 Detect decode of one level: head [N,H,W,ldc] (A*F used channels, anchor-major) ->
+// out[n][box0 + (a*H + y)*W + x][0..F) fp32, rows of `boxes_total` boxes per image.
+// anchor_wh: A (w, h) pairs already multiplied by the stride.
+struct DetectArgs {
+  const void* head; float* out; int N, H, W, A, F, ldc; long long box0, boxes_total; float stride; float anchor_wh[8];
+};
+void launch_yolo_detect(const DetectArgs& a, int dt, hipStream_t s);
 void launch_cast(const void* src, int src_dt, void* dst, int dst_dt, long long n, hipStream_t s);
 void launch_fill_f32(float* dst, float v, long long n, hipStream_t s);
 

@@ -518,4 +518,49 @@ void launch_maxpool_nhwc(const void* in, void* out, int dt, int N, int H, int W,
   NNCV_HIP_CHECK(hipGetLastError());
 }
 
+// ---------------------------------------------------------------------------------------------
+// YOLOv5 Detect decode, one level (Yolov5s.mlir:1348-1448): expand [N,A*F,H,W] to [N,A,H,W,F],
+// sigmoid, xy = (2 s + (x, y) - 0.5) * stride, wh = (2 s)^2 * anchor (powf(., 2) is the square),
+// everything else the sigmoid itself; boxes ordered (anchor, y, x).  One thread per output value,
+// F fastest, so both the NHWC read (F consecutive channels of one anchor) and the fp32 write are
+// contiguous runs of F elements.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void yolo_detect_kernel(const DetectArgs a) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long per_img = (long long)a.A * a.H * a.W * a.F;
+  if (idx >= per_img * a.N) return;
+  const int n = (int)(idx / per_img);
+  long long r = idx - n * per_img;
+  const int k = (int)(r % a.F);
+  r /= a.F;
+  const int x = (int)(r % a.W);
+  r /= a.W;
+  const int y = (int)(r % a.H);
+  const int an = (int)(r / a.H);
+  const T* head = static_cast<const T*>(a.head);
+  const float v = (float)head[(((long long)n * a.H + y) * a.W + x) * a.ldc + an * a.F + k];
+  const float sg = 1.0f / (expf(-v) + 1.0f);
+  float o = sg;
+  if (k < 2) {
+    const float g = (float)(k == 0 ? x : y) - 0.5f;
+    o = (sg * 2.0f + g) * a.stride;
+  } else if (k < 4) {
+    const float t = sg * 2.0f;
+    o = (t * t) * a.anchor_wh[an * 2 + (k - 2)];
+  }
+  a.out[((long long)n * a.boxes_total + a.box0 + ((long long)an * a.H + y) * a.W + x) * a.F + k] = o;
+}
+
+void launch_yolo_detect(const DetectArgs& a, int dt, hipStream_t s) {
+  NNCV_REQUIRE(a.A >= 1 && a.A <= 4 && a.F >= 5 && a.A * a.F <= a.ldc && a.N >= 1 && a.H >= 1 && a.W >= 1, "yolo_detect: bad shape");
+  const long long work = (long long)a.N * a.A * a.H * a.W * a.F;
+  ProfScope prof("yolo_detect", 0.0, (double)work * (dtype_size(dt) + 4.0), s);
+  if (dt == kF16)
+    hipLaunchKernelGGL((yolo_detect_kernel<half_t>), dim3(grid_for(work)), dim3(256), 0, s, a);
+  else
+    hipLaunchKernelGGL((yolo_detect_kernel<float>), dim3(grid_for(work)), dim3(256), 0, s, a);
+  NNCV_HIP_CHECK(hipGetLastError());
+}
+
 }  // namespace nncv_hip

@@ -32,6 +32,7 @@ const char* kind_name(int k) {
     case NNCV_HIP_OP_ACT: return "act";
     case NNCV_HIP_OP_CONCAT: return "concat";
     case NNCV_HIP_OP_UPSAMPLE2X: return "upsample2x";
+    case NNCV_HIP_OP_YOLO_DETECT: return "yolo_detect";
     default: return "?";
   }
 }
@@ -41,6 +42,7 @@ int n_inputs(int kind) {
     case NNCV_HIP_OP_SCALE:
     case NNCV_HIP_OP_ADD: return 2;
     case NNCV_HIP_OP_CONCAT: return 4;
+    case NNCV_HIP_OP_YOLO_DETECT: return 3;
     case NNCV_HIP_OP_CONV: return 2;  // second one (residual) optional
     default: return 1;
   }
@@ -61,8 +63,10 @@ Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, lon
   NNCV_REQUIRE(max_id >= 1 && max_id <= 4 * n + 4, "graph: tensor ids out of range");
   n_tensors_ = max_id + 1;
   channels_.assign(n_tensors_, 0);
+  logical_.assign(n_tensors_, 0);
   last_use_.assign(n_tensors_, -1);
   channels_[0] = round_up(in_channels, vn);
+  logical_[0] = in_channels;
   nodes_.resize(n);
 
   auto param = [&](long long off, long long count, const std::string& what) -> const void* {
@@ -75,7 +79,8 @@ Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, lon
     const std::string where = "graph: operator " + std::to_string(i) + " (" + kind_name(op.kind) + "): ";
     Node& nd = nodes_[i];
     nd.op = op;
-    NNCV_REQUIRE(op.kind >= NNCV_HIP_OP_CONV && op.kind <= NNCV_HIP_OP_UPSAMPLE2X, where + "unknown kind");
+    NNCV_REQUIRE(op.kind >= NNCV_HIP_OP_CONV && op.kind <= NNCV_HIP_OP_YOLO_DETECT, where + "unknown kind");
+    NNCV_REQUIRE(op.kind != NNCV_HIP_OP_YOLO_DETECT || i == n - 1, where + "must be the last operator");
     NNCV_REQUIRE(op.out >= 1 && op.out < n_tensors_ && channels_[op.out] == 0, where + "`out` must be a new tensor id");
     NNCV_REQUIRE(op.act >= kActNone && op.act <= kActSigmoid, where + "unknown activation");
     const int ni = n_inputs(op.kind);
@@ -85,26 +90,36 @@ Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, lon
         NNCV_REQUIRE(t < 0, where + "too many inputs");
         continue;
       }
-      const bool optional = k > 0 && (op.kind == NNCV_HIP_OP_CONV || op.kind == NNCV_HIP_OP_CONCAT);
+      const bool optional =
+          k > 0 && (op.kind == NNCV_HIP_OP_CONV || op.kind == NNCV_HIP_OP_CONCAT || op.kind == NNCV_HIP_OP_YOLO_DETECT);
       if (t < 0 && optional) continue;
       NNCV_REQUIRE(t >= 0 && t < n_tensors_ && channels_[t] > 0, where + "input is not a tensor defined earlier");
       last_use_[t] = i;
     }
     const int C = channels_[op.in[0]];
     nd.C = C;
-    int Cout = C;
+    int Cout = C;       // logical channels of the result
+    int Cstored = -1;   // stored channels when they differ
+    // Only convolutions (which know the real count from their filters), the Detect decode and the
+    // network output may read a tensor that is stored with padding channels.
+    if (op.kind != NNCV_HIP_OP_CONV && op.kind != NNCV_HIP_OP_YOLO_DETECT)
+      for (int k = 0; k < ni; ++k)
+        if (op.in[k] >= 0)
+          NNCV_REQUIRE(logical_[op.in[k]] == channels_[op.in[k]],
+                       where + "channel count of an input must be a multiple of the 16-byte vector");
     switch (op.kind) {
       case NNCV_HIP_OP_CONV: {
-        NNCV_REQUIRE(op.F > 0 && op.F % vn == 0, where + "F must be a multiple of the 16-byte vector");
+        NNCV_REQUIRE(op.F > 0, where + "F must be positive");
         NNCV_REQUIRE(op.K >= 1 && op.K <= 11 && op.stride >= 1 && op.pad >= 0, where + "bad geometry");
-        NNCV_REQUIRE(op.in[1] < 0 || channels_[op.in[1]] == op.F, where + "residual has another channel count");
+        NNCV_REQUIRE(op.in[1] < 0 || logical_[op.in[1]] == op.F, where + "residual has another channel count");
         Cout = op.F;
-        const int Cl = op.in[0] == 0 ? c_in_ : C;  // channels the filters really have
+        Cstored = round_up(op.F, vn);
+        const int Cl = logical_[op.in[0]];  // channels the filters really have
         const void* w = param(op.w, (long long)op.F * Cl * op.K * op.K, where + "w");
-        nd.wt.reset((size_t)op.F * op.K * op.K * C * es);
+        nd.wt.reset((size_t)Cstored * op.K * op.K * C * es);
         NNCV_HIP_CHECK(hipMemsetAsync(nd.wt.get(), 0, nd.wt.bytes(), s));
         launch_weight_frsc(w, dt, nd.wt.get(), dt, op.F, Cl, op.K, op.K, C, s);
-        if (op.K == 3 && op.stride == 1 && op.pad == 1 && Cl == C && C % (128 / (int)es) == 0) {
+        if (op.K == 3 && op.stride == 1 && op.pad == 1 && Cl == C && Cstored == op.F && C % (128 / (int)es) == 0) {
           nd.wfrag.reset((size_t)((op.F + 63) / 64) * 64 * 9 * C * es);
           launch_weight_frag3x3(w, dt, nd.wfrag.get(), dt, op.F, C, s);
         }
@@ -113,7 +128,6 @@ Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, lon
       case NNCV_HIP_OP_DWCONV: {
         NNCV_REQUIRE(op.K == 3 || op.K == 5, where + "K must be 3 or 5");
         NNCV_REQUIRE(op.stride >= 1 && op.pad >= 0, where + "bad geometry");
-        NNCV_REQUIRE(op.in[0] != 0 || c_in_ == C, where + "the network input must have whole channel vectors");
         const void* w = param(op.w, (long long)C * op.K * op.K, where + "w");
         nd.wt.reset((size_t)C * op.K * op.K * es);
         launch_weight_dw(w, dt, nd.wt.get(), dt, C, op.K, s);
@@ -130,21 +144,53 @@ Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, lon
         for (int k = 1; k < 4; ++k)
           if (op.in[k] >= 0) Cout += channels_[op.in[k]];
         break;
+      case NNCV_HIP_OP_YOLO_DETECT: {
+        NNCV_REQUIRE(op.K >= 1 && op.K <= 4 && op.F >= 5, where + "K anchors (1..4) of F >= 5 values each");
+        int levels = 0;
+        for (int k = 0; k < 3; ++k)
+          if (op.in[k] >= 0) {
+            NNCV_REQUIRE(k == levels, where + "levels must be in[0], in[1], ... without gaps");
+            NNCV_REQUIRE(logical_[op.in[k]] == op.K * op.F, where + "a head must have K * F channels");
+            ++levels;
+          }
+        // anchors and strides are tiny and needed as kernel arguments: read them back once
+        const void* an = param(op.w, (long long)levels * op.K * 2, where + "anchors");
+        const void* st = param(op.bias, levels, where + "strides");
+        std::vector<float> anchors((size_t)levels * op.K * 2), strides(levels);
+        DeviceBuffer tmp((anchors.size() + strides.size()) * 4);
+        launch_cast(an, dt, tmp.get(), kF32, (long long)anchors.size(), s);
+        launch_cast(st, dt, tmp.as<float>() + anchors.size(), kF32, levels, s);
+        NNCV_HIP_CHECK(hipMemcpyAsync(anchors.data(), tmp.get(), anchors.size() * 4, hipMemcpyDeviceToHost, s));
+        NNCV_HIP_CHECK(hipMemcpyAsync(strides.data(), tmp.as<float>() + anchors.size(), strides.size() * 4, hipMemcpyDeviceToHost, s));
+        NNCV_HIP_CHECK(hipStreamSynchronize(s));
+        detect_stride_ = strides;
+        detect_anchor_wh_.resize(anchors.size());
+        for (int l = 0; l < levels; ++l)
+          for (int q = 0; q < op.K * 2; ++q) detect_anchor_wh_[l * op.K * 2 + q] = anchors[l * op.K * 2 + q] * strides[l];
+        Cout = op.F;
+        Cstored = op.F;
+        break;
+      }
       default: break;
     }
     if (op.kind == NNCV_HIP_OP_CONV || op.kind == NNCV_HIP_OP_DWCONV) {
-      const int F = Cout;
+      const int F = Cout, Fs = Cstored > 0 ? Cstored : Cout;
       if (op.gamma >= 0) {
         NNCV_REQUIRE(op.beta >= 0 && op.mean >= 0 && op.var >= 0, where + "BatchNorm needs gamma, beta, mean and var");
-        nd.scale.reset((size_t)F * 4);
-        nd.shift.reset((size_t)F * 4);
+        nd.scale.reset((size_t)Fs * 4);
+        nd.shift.reset((size_t)Fs * 4);
+        launch_fill_f32(nd.scale.as<float>(), 0.0f, Fs, s);
+        launch_fill_f32(nd.shift.as<float>(), 0.0f, Fs, s);
         launch_bn_fold(param(op.gamma, F, where + "gamma"), param(op.beta, F, where + "beta"), param(op.mean, F, where + "mean"),
                        param(op.var, F, where + "var"), dt, nd.scale.as<float>(), nd.shift.as<float>(), F, s, op.eps);
       }
       if (op.bias >= 0) {
         const void* b = param(op.bias, F, where + "bias");
         const bool had = nd.shift.get() != nullptr;
-        if (!had) nd.shift.reset((size_t)F * 4);
+        if (!had) {
+          nd.shift.reset((size_t)Fs * 4);
+          launch_fill_f32(nd.shift.as<float>(), 0.0f, Fs, s);
+        }
         const unsigned grid = (unsigned)((F + 255) / 256);
         if (dt == kF16)
           hipLaunchKernelGGL((fold_bias_kernel<half_t>), dim3(grid), dim3(256), 0, s, (const half_t*)b, nd.scale.as<float>(),
@@ -155,8 +201,11 @@ Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, lon
         NNCV_HIP_CHECK(hipGetLastError());
       }
     }
-    NNCV_REQUIRE(Cout % vn == 0, where + "channel count must be a multiple of the 16-byte vector");
-    channels_[op.out] = Cout;
+    if (Cstored < 0) Cstored = Cout;
+    NNCV_REQUIRE(Cstored % vn == 0 || op.kind == NNCV_HIP_OP_YOLO_DETECT,
+                 where + "channel count must be a multiple of the 16-byte vector");
+    channels_[op.out] = Cstored;
+    logical_[op.out] = Cout;
   }
   for (int t = 1; t < n_tensors_; ++t) NNCV_REQUIRE(channels_[t] > 0, "graph: tensor " + std::to_string(t) + " is never produced");
 
@@ -218,6 +267,14 @@ const Graph::Plan& Graph::plan_of(int N, int H, int W) const {
             NNCV_REQUIRE(p.dims[op.in[k]].H == a.H && p.dims[op.in[k]].W == a.W, where + "operands have different sizes");
         break;
       case NNCV_HIP_OP_UPSAMPLE2X: o.H = 2 * a.H; o.W = 2 * a.W; break;
+      case NNCV_HIP_OP_YOLO_DETECT: {  // [N, boxes, F]: reported as channels = boxes, height = F, width = 1
+        long long boxes = 0;
+        for (int k = 0; k < 3; ++k)
+          if (op.in[k] >= 0) boxes += (long long)op.K * p.dims[op.in[k]].H * p.dims[op.in[k]].W;
+        NNCV_REQUIRE(boxes * op.F * N < (1ll << 31), where + "tensor too large");
+        o.C = (int)boxes; o.H = op.F; o.W = 1;
+        break;
+      }
       default: break;
     }
     NNCV_REQUIRE((long long)N * o.H * o.W * o.C < (1ll << 31), where + "tensor too large");
@@ -233,6 +290,7 @@ const Graph::Plan& Graph::plan_of(int N, int H, int W) const {
     const int t = nodes_[i].op.out;
     const Dims d = p.dims[t];
     life[t] = TensorLife{i + 1, std::max(i + 1, last_use_[t] + 1), (size_t)N * d.H * d.W * d.C * es, 0};
+    if (nodes_[i].op.kind == NNCV_HIP_OP_YOLO_DETECT) life[t].bytes = 256;  // written straight to the caller's buffer
   }
   life[nodes_[n - 1].op.out].last_op = n + 1;
   p.total = plan_offsets(life, 256);
@@ -245,8 +303,10 @@ const Graph::Plan& Graph::plan_of(int N, int H, int W) const {
 
 void Graph::output_shape(int H, int W, int* C, int* OH, int* OW) const {
   const Plan& p = plan_of(1, H, W);
-  const Dims d = p.dims[nodes_.back().op.out];
-  *C = d.C; *OH = d.H; *OW = d.W;
+  const int t = nodes_.back().op.out;
+  const Dims d = p.dims[t];
+  *C = nodes_.back().op.kind == NNCV_HIP_OP_YOLO_DETECT ? d.C : logical_[t];
+  *OH = d.H; *OW = d.W;
 }
 
 size_t Graph::workspace_bytes(int N, int H, int W) const { return plan_of(N, H, W).total; }
@@ -277,9 +337,11 @@ void Graph::forward(const void* src, int N, int H, int W, float* out, void* ws, 
         g.in = at(op.in[0]); g.wt = nd.wt.get(); g.wt_frag = nd.wfrag.get(); g.out = at(op.out);
         g.scale = nd.scale.as<float>(); g.shift = nd.shift.as<float>();
         g.residual = op.in[1] >= 0 ? at(op.in[1]) : nullptr;
-        g.N = N; g.H = a.H; g.W = a.W; g.C = a.C; g.F = op.F; g.R = g.S = op.K; g.OH = o.H; g.OW = o.W;
+        // padding filters (zero rows, zero scale/shift) are computed like any other: o.C >= op.F
+        g.N = N; g.H = a.H; g.W = a.W; g.C = a.C; g.F = o.C; g.R = g.S = op.K; g.OH = o.H; g.OW = o.W;
         g.stride_h = g.stride_w = op.stride; g.pad_h = g.pad_w = op.pad;
-        g.relu = op.act; g.ldo = op.F; g.batch = 1;
+        g.relu = op.act; g.ldo = o.C; g.batch = 1;
+        g.alg_flops = 2.0 * N * o.H * o.W * op.F * (double)op.K * op.K * logical_[op.in[0]];
         launch_igemm(g, dt_, dt_, s);
         break;
       }
@@ -320,12 +382,27 @@ void Graph::forward(const void* src, int N, int H, int W, float* out, void* ws, 
       case NNCV_HIP_OP_UPSAMPLE2X:
         launch_upsample2x(at(op.in[0]), at(op.out), dt_, N, a.H, a.W, a.C, a.C, 0, s);
         break;
+      case NNCV_HIP_OP_YOLO_DETECT: {
+        long long box0 = 0;
+        for (int k = 0; k < 3 && op.in[k] >= 0; ++k) {
+          const Dims h = p.dims[op.in[k]];
+          DetectArgs d{};
+          d.head = at(op.in[k]); d.out = out; d.N = N; d.H = h.H; d.W = h.W; d.A = op.K; d.F = op.F; d.ldc = h.C;
+          d.box0 = box0; d.boxes_total = o.C; d.stride = detect_stride_[k];
+          for (int q = 0; q < op.K * 2; ++q) d.anchor_wh[q] = detect_anchor_wh_[k * op.K * 2 + q];
+          launch_yolo_detect(d, dt_, s);
+          box0 += (long long)op.K * h.H * h.W;
+        }
+        break;
+      }
       default: fail("graph: unknown operator kind");
     }
   }
+  if (nodes_.back().op.kind == NNCV_HIP_OP_YOLO_DETECT) return;  // already in the caller's buffer, fp32
   const int t = nodes_.back().op.out;
   const Dims d = p.dims[t];
-  launch_relayout(at(t), dt_, strides_of(kNHWC, d.C, d.H, d.W), out, kF32, strides_of(kNCHW, d.C, d.H, d.W), N, d.C, d.C, d.H, d.W,
+  const int Cl = logical_[t];
+  launch_relayout(at(t), dt_, strides_of(kNHWC, d.C, d.H, d.W), out, kF32, strides_of(kNCHW, Cl, d.H, d.W), N, Cl, Cl, d.H, d.W,
                   false, s);
 }
 

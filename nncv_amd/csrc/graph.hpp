@@ -52,7 +52,9 @@ class Graph {
 
   int dt_, c_in_, n_tensors_ = 0;
   std::vector<Node> nodes_;
-  std::vector<int> channels_;  // per tensor, as stored
+  std::vector<int> channels_;  // per tensor, as stored (padded to a whole 16-byte vector)
+  std::vector<int> logical_;   // per tensor, as the network defines it
+  std::vector<float> detect_anchor_wh_, detect_stride_;  // YOLO_DETECT: host copies of anchors * stride, strides
   std::vector<int> last_use_;  // per tensor: index of the last operator that reads it
   mutable std::vector<Plan> plans_;
 };

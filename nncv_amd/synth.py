@@ -128,6 +128,29 @@ def mobilenetv3_params(seed_base=6100):
     return blob
 
 
+def yolov5s_params(seed_base=8100):
+    """Flat fp32 parameter blob of YOLOv5s in the canonical order (yolov5s_spec).  Convolution weights
+    Kaiming normal std = sqrt(2/fan_in) (the BatchNorm is already fused in this network's table), biases
+    N(0, 0.1) -- the three Detect biases N(0, 1) so that the decoded boxes spread over their range --,
+    anchors and strides the published yolov5s.yaml values."""
+    from . import yolov5s_spec as y
+    parts = []
+    for k, (name, shape) in enumerate(y.tensor_table()):
+        seed = seed_base + k
+        if name == "model.24.anchors":
+            a = np.array([[v / y.STRIDES[l] for v in y.ANCHORS_PX[l]] for l in range(3)], np.float32).reshape(shape)
+        elif name == "model.24.stride":
+            a = np.array(y.STRIDES, np.float32)
+        elif len(shape) == 4:
+            a = normal(seed, shape, std=float(np.sqrt(2.0 / int(np.prod(shape[1:])))))
+        else:
+            a = normal(seed, shape, std=1.0 if name.startswith("model.24.") else 0.1)
+        parts.append(a.reshape(-1))
+    blob = np.concatenate(parts)
+    assert blob.size == y.NUM_ELEMENTS
+    return blob
+
+
 def cfg3_input():
     return uniform(3000, (1, 3, 256, 256), 0.0, 1.0)
 

@@ -267,6 +267,27 @@ def upsample2x_nearest(x):
     return _c(x).repeat(2, axis=2).repeat(2, axis=3)
 
 
+def yolo_detect(heads, anchors, strides, A, F):
+    """YOLOv5 Detect decode as Yolov5s.mlir:1348-1448 (and :1449-1662 for the other levels) spells it.
+    heads: NCHW [N, A*F, H_l, W_l] per level; anchors [L, A, 2] in units of the stride; strides [L]
+    -> [N, sum_l A*H_l*W_l, F], boxes ordered (level, anchor, y, x)."""
+    anchors, strides = _c(anchors), _c(strides)
+    outs = []
+    for l, h in enumerate(heads):
+        h = _c(h)
+        N, _, H, W = h.shape
+        p = h.reshape(N, A, F, H, W).transpose(0, 1, 3, 4, 2)            # expand_shape + permuting generic
+        s = sigmoid(p)
+        gx = np.arange(W, dtype=np.float32) + np.float32(0.0)             # linalg.index + 0 (:1358-1366)
+        gy = np.arange(H, dtype=np.float32) + np.float32(0.0)
+        grid = np.stack(np.broadcast_arrays(gx[None, :], gy[:, None]), axis=-1) - np.float32(0.5)  # (x, y) - 0.5
+        ag = (anchors[l] * strides[l]).astype(np.float32).reshape(1, A, 1, 1, 2)                    # anchors * stride
+        xy = ((s[..., 0:2] * np.float32(2.0) + grid.reshape(1, 1, H, W, 2)) * strides[l]).astype(np.float32)
+        wh = (np.power(s[..., 2:4] * np.float32(2.0), np.float32(2.0)) * ag).astype(np.float32)     # math.powf(., 2)
+        outs.append(np.concatenate([xy, wh, s[..., 4:]], axis=-1).reshape(N, A * H * W, F))
+    return np.concatenate(outs, axis=1)
+
+
 def mobilenetv3_forward(x, tensors, taps=None):
     """MobileNetV3-small as tests/Nets/MobileNetV3.mlir computes it.  x [N,3,H,W] fp32; tensors: {name: ndarray} with
     torchvision state_dict names (nncv_amd.mobilenetv3_spec.tensor_table) -> logits [N,1000].
@@ -316,10 +337,13 @@ def mobilenetv3_forward(x, tensors, taps=None):
     return fc(y, T["classifier.3.weight"], T["classifier.3.bias"])
 
 
-def run_graph(ops, x, blob, in_channels):
+def run_graph(ops, x, blob, in_channels, conv=None):
     """Evaluates a list of nncv_hip_graph_op-like records (attributes kind, inputs, out, F, K, stride, pad, act, eps,
-    w, bias, gamma, beta, mean, var) with the operator restatements above; NCHW fp32.  Checker for the graph executor."""
+    w, bias, gamma, beta, mean, var) with the operator restatements above; NCHW fp32.  Checker for the graph executor.  `conv(x, w, stride, pad)`
+    replaces the scalar convolution (e.g. hwp_conv2d, the OpenMP x AVX2 restatement, for large images)."""
     blob = _c(blob)
+    if conv is None:
+        conv = lambda a, w, stride, pad: conv2d_nchw_fchw(pad_nchw(a, pad) if pad else a, w, stride)
     vals = {0: _c(x)}
     for o in ops:
         ins = [t for t in o.inputs if t >= 0]
@@ -330,7 +354,7 @@ def run_graph(ops, x, blob, in_channels):
             if o.kind == 1:
                 F = o.F
                 w = blob[o.w:o.w + F * C * o.K * o.K].reshape(F, C, o.K, o.K)
-                y = conv2d_nchw_fchw(pad_nchw(a, o.pad) if o.pad else a, w, o.stride)
+                y = conv(a, w, o.stride, o.pad)
             else:
                 F = C
                 w = blob[o.w:o.w + C * o.K * o.K].reshape(C, o.K, o.K)
@@ -357,6 +381,9 @@ def run_graph(ops, x, blob, in_channels):
             y = np.concatenate([vals[t] for t in ins], axis=1)
         elif o.kind == 9:
             y = upsample2x_nearest(a)
+        elif o.kind == 10:
+            L = len(ins)
+            y = yolo_detect([vals[t] for t in ins], blob[o.w:o.w + L * o.K * 2].reshape(L, o.K, 2), blob[o.bias:o.bias + L], o.K, o.F)
         else:
             raise ValueError("unknown operator kind %d" % o.kind)
         vals[o.out] = _c(y)

@@ -290,7 +290,7 @@ def test_graph_create_refuses_malformed_lists():
     assert "new tensor id" in refused(clone(2, out=2))                                          # writes a tensor twice
     assert "unknown kind" in refused(clone(3, kind=42))
     assert "outside the parameter blob" in refused(clone(4, w=blob.size - 3))
-    assert "multiple" in refused(clone(4, F=10))                                                # 10 floats are not whole 16-byte vectors
+    assert "multiple" in refused(clone(0, F=10))                                                # a max-pool cannot read 10 (stored 12) channels
     assert "K must be 3 or 5" in refused(clone(1, kind=abi.OP_DWCONV, K=7, w=0))
     assert "unknown activation" in refused(clone(10, act=9))
     assert "channel" in refused(clone(8, inputs=(ctypes.c_int32 * 4)(8, 6, -1, -1)))            # residual with 2C channels

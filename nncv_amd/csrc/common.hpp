@@ -43,6 +43,9 @@ struct Error : std::runtime_error {
 // :349-379 hard-sigmoid; Yolov5s.mlir SiLU = x * 1/(1+exp(-x))).
 // ---------------------------------------------------------------------------------------------
 enum Act : int { kActNone = 0, kActRelu = 1, kActHardSwish = 2, kActHardSigmoid = 3, kActSilu = 4, kActSigmoid = 5 };
+// flag on the activation code of a convolution epilogue: the residual is added after the activation
+// (a YOLOv5 Bottleneck, x + SiLU(conv)) instead of before it (a ResNet BasicBlock, ReLU(conv + x))
+constexpr int kActResidualAfter = 0x100;
 
 // `arith.cmpf ugt` + select: NaN is kept, everything not greater than zero becomes +0.
 __device__ __forceinline__ float relu_ugt(float x) { return (x <= 0.0f) ? 0.0f : x; }
@@ -102,7 +105,7 @@ struct IgemmArgs {
   const void* residual;  // same indexing as out, or null
   int N, H, W, C, F, R, S, OH, OW;
   int stride_h, stride_w, pad_h, pad_w;
-  int relu;    // activation code (enum Act) applied last; 0 none, 1 ReLU
+  int relu;    // activation code (enum Act), optionally | kActResidualAfter; 0 none, 1 ReLU
   int ldo;     // out/residual row pitch in elements
   int batch;   // grid.z
   long long in_bs, wt_bs, out_bs;  // batch strides in elements
@@ -212,13 +215,17 @@ bool se_block_applicable(int dt, int HW, int C, int SQ);
 void launch_se_block(const SeArgs& a, int dt, hipStream_t s);
 // out = act(a (+ b));  b may be null;  n elements, n a multiple of the 16-byte vector
 void launch_eltwise(const void* a, const void* b, void* out, int dt, long long n, int act, hipStream_t s);
+// the same over [P][C] tensors with row pitches lda / ldb / ldo (elements): slices of wider tensors
+void launch_eltwise_pitched(const void* a, int lda, const void* b, int ldb, void* out, int ldo, int dt, long long P, int C, int act,
+                            hipStream_t s);
 // copies x [P][C] into channels [c0, c0 + C) of out [P][ldo]   (torch.cat over channels, NHWC)
-void launch_concat_slice(const void* x, void* out, int dt, long long P, int C, int ldo, int c0, hipStream_t s);
+// (ldi: row pitch of x, 0 = C)
+void launch_concat_slice(const void* x, void* out, int dt, long long P, int C, int ldo, int c0, hipStream_t s, int ldi = 0);
 // nearest-neighbour 2x up-sampling [N,H,W,C] -> [N,2H,2W,C], written at channel offset c0 of pitch ldo
-void launch_upsample2x(const void* x, void* out, int dt, int N, int H, int W, int C, int ldo, int c0, hipStream_t s);
+void launch_upsample2x(const void* x, void* out, int dt, int N, int H, int W, int C, int ldo, int c0, hipStream_t s, int ldi = 0);
 // max-pool K x K, any stride / padding (-inf halo), NHWC
 void launch_maxpool_nhwc(const void* in, void* out, int dt, int N, int H, int W, int C, int K, int stride, int pad,
-                         hipStream_t s);
+                         hipStream_t s, int ldi = 0, int ldo = 0);  // pixel pitches of in / out, 0 = C
 // YOLOv5 Detect decode of one level: head [N,H,W,ldc] (A*F used channels, anchor-major) ->
 // out[n][box0 + (a*H + y)*W + x][0..F) fp32, rows of `boxes_total` boxes per image.
 // anchor_wh: A (w, h) pairs already multiplied by the stride.

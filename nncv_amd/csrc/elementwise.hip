@@ -374,42 +374,55 @@ void launch_se_block(const SeArgs& a, int dt, hipStream_t s) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// out = act(a + b)
+// out = act(a + b) over [P][C] tensors whose rows may sit inside wider ones (row pitches lda, ldb,
+// ldo in elements): a tensor that is one input of a channel concatenation lives in its slice of the
+// concatenated tensor.
 // ---------------------------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void eltwise_kernel(const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ out,
-                                                      long long nvec, int act) {
+                                                      long long nvec, int CG, int lda, int ldb, int ldo, int act) {
   constexpr int VN = V16<T>::n;
   typedef typename V16<T>::type V;
   const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= nvec) return;
-  const V av = *reinterpret_cast<const V*>(a + idx * VN);
+  const long long p = idx / CG;
+  const int c = (int)(idx - p * CG) * VN;
+  const V av = *reinterpret_cast<const V*>(a + p * lda + c);
   float y[VN];
 #pragma unroll
   for (int e = 0; e < VN; ++e) y[e] = (float)av[e];
   if (b) {
-    const V bv = *reinterpret_cast<const V*>(b + idx * VN);
+    const V bv = *reinterpret_cast<const V*>(b + p * ldb + c);
 #pragma unroll
     for (int e = 0; e < VN; ++e) y[e] += (float)bv[e];
   }
   V o;
 #pragma unroll
   for (int e = 0; e < VN; ++e) o[e] = (T)act_apply(y[e], act);
-  *reinterpret_cast<V*>(out + idx * VN) = o;
+  *reinterpret_cast<V*>(out + p * ldo + c) = o;
+}
+
+void launch_eltwise_pitched(const void* a, int lda, const void* b, int ldb, void* out, int ldo, int dt, long long P, int C, int act,
+                            hipStream_t s) {
+  const int vn = dt == kF16 ? 8 : 4;
+  NNCV_REQUIRE(C % vn == 0 && lda % vn == 0 && ldb % vn == 0 && ldo % vn == 0 && lda >= C && ldo >= C && (!b || ldb >= C),
+               "eltwise: channel count and pitches must be multiples of the 16-byte vector");
+  const long long n = P * C;
+  if (n == 0) return;
+  ProfScope prof(b ? "eltwise_add" : "eltwise_act", (double)n, (double)dtype_size(dt) * n * (b ? 3 : 2), s);
+  if (dt == kF16)
+    hipLaunchKernelGGL((eltwise_kernel<half_t>), dim3(grid_for(n / vn)), dim3(256), 0, s, (const half_t*)a, (const half_t*)b,
+                       (half_t*)out, n / vn, C / vn, lda, ldb, ldo, act);
+  else
+    hipLaunchKernelGGL((eltwise_kernel<float>), dim3(grid_for(n / vn)), dim3(256), 0, s, (const float*)a, (const float*)b,
+                       (float*)out, n / vn, C / vn, lda, ldb, ldo, act);
+  NNCV_HIP_CHECK(hipGetLastError());
 }
 
 void launch_eltwise(const void* a, const void* b, void* out, int dt, long long n, int act, hipStream_t s) {
   const int vn = dt == kF16 ? 8 : 4;
   NNCV_REQUIRE(n % vn == 0, "eltwise: element count must be a multiple of the 16-byte vector");
-  if (n == 0) return;
-  ProfScope prof(b ? "eltwise_add" : "eltwise_act", (double)n, (double)dtype_size(dt) * n * (b ? 3 : 2), s);
-  if (dt == kF16)
-    hipLaunchKernelGGL((eltwise_kernel<half_t>), dim3(grid_for(n / vn)), dim3(256), 0, s, (const half_t*)a, (const half_t*)b,
-                       (half_t*)out, n / vn, act);
-  else
-    hipLaunchKernelGGL((eltwise_kernel<float>), dim3(grid_for(n / vn)), dim3(256), 0, s, (const float*)a, (const float*)b,
-                       (float*)out, n / vn, act);
-  NNCV_HIP_CHECK(hipGetLastError());
+  launch_eltwise_pitched(a, vn, b, vn, out, vn, dt, n / vn, vn, act, s);  // a dense tensor is [n / vn][vn]
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -417,28 +430,29 @@ void launch_eltwise(const void* a, const void* b, void* out, int dt, long long n
 // up-sampling written straight into such a slice; both move raw 16-byte vectors.
 // ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void concat_slice_kernel(const uint4* __restrict__ x, uint4* __restrict__ out, long long total,
-                                                           int CG, int ldg, int g0) {
+                                                           int CG, int ldig, int ldg, int g0) {
   const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const long long p = idx / CG;
   const int cg = (int)(idx % CG);
-  out[p * ldg + g0 + cg] = x[idx];
+  out[p * ldg + g0 + cg] = x[p * ldig + cg];
 }
 
-void launch_concat_slice(const void* x, void* out, int dt, long long P, int C, int ldo, int c0, hipStream_t s) {
+void launch_concat_slice(const void* x, void* out, int dt, long long P, int C, int ldo, int c0, hipStream_t s, int ldi) {
   const int vn = dt == kF16 ? 8 : 4;
-  NNCV_REQUIRE(C % vn == 0 && ldo % vn == 0 && c0 % vn == 0 && c0 >= 0 && c0 + C <= ldo,
+  if (ldi == 0) ldi = C;
+  NNCV_REQUIRE(C % vn == 0 && ldo % vn == 0 && c0 % vn == 0 && c0 >= 0 && c0 + C <= ldo && ldi % vn == 0 && ldi >= C,
                "concat: channel counts and offset must be multiples of the 16-byte vector");
   const long long total = P * (C / vn);
   if (total == 0) return;
   ProfScope prof("concat_slice", 0.0, 2.0 * dtype_size(dt) * P * C, s);
   hipLaunchKernelGGL(concat_slice_kernel, dim3(grid_for(total)), dim3(256), 0, s, (const uint4*)x, (uint4*)out, total, C / vn,
-                     ldo / vn, c0 / vn);
+                     ldi / vn, ldo / vn, c0 / vn);
   NNCV_HIP_CHECK(hipGetLastError());
 }
 
 __global__ __launch_bounds__(256) void upsample2x_kernel(const uint4* __restrict__ x, uint4* __restrict__ out, long long total,
-                                                         int H, int W, int CG, int ldg, int g0) {
+                                                         int H, int W, int CG, int ldig, int ldg, int g0) {
   const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;  // over output vectors
   if (idx >= total) return;
   const int cg = (int)(idx % CG);
@@ -447,18 +461,19 @@ __global__ __launch_bounds__(256) void upsample2x_kernel(const uint4* __restrict
   p /= 2 * W;
   const int oy = (int)(p % (2 * H));
   const long long n = p / (2 * H);
-  out[((n * 2 * H + oy) * 2 * W + ox) * ldg + g0 + cg] = x[((n * H + (oy >> 1)) * W + (ox >> 1)) * CG + cg];
+  out[((n * 2 * H + oy) * 2 * W + ox) * ldg + g0 + cg] = x[((n * H + (oy >> 1)) * W + (ox >> 1)) * ldig + cg];
 }
 
-void launch_upsample2x(const void* x, void* out, int dt, int N, int H, int W, int C, int ldo, int c0, hipStream_t s) {
+void launch_upsample2x(const void* x, void* out, int dt, int N, int H, int W, int C, int ldo, int c0, hipStream_t s, int ldi) {
   const int vn = dt == kF16 ? 8 : 4;
-  NNCV_REQUIRE(C % vn == 0 && ldo % vn == 0 && c0 % vn == 0 && c0 >= 0 && c0 + C <= ldo,
+  if (ldi == 0) ldi = C;
+  NNCV_REQUIRE(C % vn == 0 && ldo % vn == 0 && c0 % vn == 0 && c0 >= 0 && c0 + C <= ldo && ldi % vn == 0 && ldi >= C,
                "upsample: channel counts and offset must be multiples of the 16-byte vector");
   const long long total = (long long)N * 4 * H * W * (C / vn);
   if (total == 0) return;
   ProfScope prof("upsample2x", 0.0, 5.0 * dtype_size(dt) * N * H * W * C, s);
   hipLaunchKernelGGL(upsample2x_kernel, dim3(grid_for(total)), dim3(256), 0, s, (const uint4*)x, (uint4*)out, total, H, W, C / vn,
-                     ldo / vn, c0 / vn);
+                     ldi / vn, ldo / vn, c0 / vn);
   NNCV_HIP_CHECK(hipGetLastError());
 }
 
@@ -468,7 +483,7 @@ void launch_upsample2x(const void* x, void* out, int dt, int N, int H, int W, in
 // ---------------------------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void maxpool_kernel(const T* __restrict__ in, T* __restrict__ out, int N, int H, int W, int C,
-                                                      int K, int stride, int pad, int OH, int OW) {
+                                                      int K, int stride, int pad, int OH, int OW, int ldi, int ldo) {
   constexpr int VN = V16<T>::n;
   typedef typename V16<T>::type V;
   const int CG = C / VN;
@@ -489,7 +504,7 @@ __global__ __launch_bounds__(256) void maxpool_kernel(const T* __restrict__ in, 
     for (int q = 0; q < K; ++q) {
       const int ix = ox * stride - pad + q;
       if ((unsigned)ix >= (unsigned)W) continue;
-      const V v = *reinterpret_cast<const V*>(in + (((long long)n * H + iy) * W + ix) * C + cg * VN);
+      const V v = *reinterpret_cast<const V*>(in + (((long long)n * H + iy) * W + ix) * ldi + cg * VN);
 #pragma unroll
       for (int e = 0; e < VN; ++e) m[e] = max_nan(m[e], (float)v[e]);
     }
@@ -497,13 +512,16 @@ __global__ __launch_bounds__(256) void maxpool_kernel(const T* __restrict__ in, 
   V o;
 #pragma unroll
   for (int e = 0; e < VN; ++e) o[e] = (T)m[e];
-  *reinterpret_cast<V*>(out + (((long long)n * OH + oy) * OW + ox) * C + cg * VN) = o;
+  *reinterpret_cast<V*>(out + (((long long)n * OH + oy) * OW + ox) * ldo + cg * VN) = o;
 }
 
 void launch_maxpool_nhwc(const void* in, void* out, int dt, int N, int H, int W, int C, int K, int stride, int pad,
-                         hipStream_t s) {
+                         hipStream_t s, int ldi, int ldo) {
   const int vn = dt == kF16 ? 8 : 4;
-  NNCV_REQUIRE(C % vn == 0, "maxpool: C must be a multiple of the 16-byte vector");
+  if (ldi == 0) ldi = C;
+  if (ldo == 0) ldo = C;
+  NNCV_REQUIRE(C % vn == 0 && ldi % vn == 0 && ldo % vn == 0 && ldi >= C && ldo >= C,
+               "maxpool: C and the pitches must be multiples of the 16-byte vector");
   NNCV_REQUIRE(K >= 1 && stride >= 1 && pad >= 0 && 2 * pad <= K && H + 2 * pad >= K && W + 2 * pad >= K, "maxpool: bad geometry");
   const int OH = (H + 2 * pad - K) / stride + 1, OW = (W + 2 * pad - K) / stride + 1;
   const long long work = (long long)N * OH * OW * (C / vn);
@@ -511,10 +529,10 @@ void launch_maxpool_nhwc(const void* in, void* out, int dt, int N, int H, int W,
   ProfScope prof("maxpool", 0.0, (double)dtype_size(dt) * N * C * ((double)H * W + (double)OH * OW), s);
   if (dt == kF16)
     hipLaunchKernelGGL((maxpool_kernel<half_t>), dim3(grid_for(work)), dim3(256), 0, s, (const half_t*)in, (half_t*)out, N, H, W, C,
-                       K, stride, pad, OH, OW);
+                       K, stride, pad, OH, OW, ldi, ldo);
   else
     hipLaunchKernelGGL((maxpool_kernel<float>), dim3(grid_for(work)), dim3(256), 0, s, (const float*)in, (float*)out, N, H, W, C, K,
-                       stride, pad, OH, OW);
+                       stride, pad, OH, OW, ldi, ldo);
   NNCV_HIP_CHECK(hipGetLastError());
 }
 

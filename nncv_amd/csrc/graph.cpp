@@ -228,6 +228,89 @@ Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, lon
     nodes_[i + 1].skip = nodes_[i + 2].skip = nodes_[i + 3].skip = true;
     i += 3;
   }
+
+  // x + act(conv(.)): the ADD rides in the convolution's epilogue
+  static const bool no_add = getenv("NNCV_HIP_NO_ADD_FUSION") != nullptr;
+  for (int i = 0; !no_add && i + 1 < n; ++i) {
+    const GraphOp &cv = ops[i], &ad = ops[i + 1];
+    if (cv.kind != NNCV_HIP_OP_CONV || cv.in[1] >= 0 || ad.kind != NNCV_HIP_OP_ADD || ad.act != kActNone) continue;
+    if (readers[cv.out] != 1 || logical_[cv.out] != channels_[cv.out]) continue;
+    const int other = ad.in[0] == cv.out ? ad.in[1] : (ad.in[1] == cv.out ? ad.in[0] : -1);
+    if (other < 0 || other == cv.out) continue;
+    nodes_[i].add_res = other;
+    nodes_[i].add_out = ad.out;
+    nodes_[i + 1].skip = true;
+  }
+
+  // concatenation views
+  view_of_.assign(n_tensors_, -1);
+  view_c0_.assign(n_tensors_, 0);
+  static const bool no_views = getenv("NNCV_HIP_NO_CONCAT_VIEWS") != nullptr;
+  if (!no_views) {
+    std::vector<int> producer(n_tensors_, -1), cat_uses(n_tensors_, 0);
+    for (int i = 0; i < n; ++i) {
+      producer[nodes_[i].add_out >= 0 ? nodes_[i].add_out : ops[i].out] = i;
+      if (ops[i].kind == NNCV_HIP_OP_CONCAT)
+        for (int k = 0; k < 4; ++k)
+          if (ops[i].in[k] >= 0) ++cat_uses[ops[i].in[k]];
+    }
+    // may operator i read tensor t at a pitch / write its result at a pitch?
+    auto reads_pitched = [&](int i, int t) {
+      const GraphOp& o = ops[i];
+      if (nodes_[i].skip)  // merged into its predecessor: the residual of a conv + ADD pair shares the result's pitch
+        return i > 0 && nodes_[i - 1].add_out >= 0 && nodes_[i - 1].add_res != t;
+      switch (o.kind) {
+        case NNCV_HIP_OP_CONV: return o.in[1] != t;  // not as the residual
+        case NNCV_HIP_OP_MAXPOOL:
+        case NNCV_HIP_OP_UPSAMPLE2X:
+        case NNCV_HIP_OP_ADD:
+        case NNCV_HIP_OP_ACT:
+        case NNCV_HIP_OP_CONCAT:
+        case NNCV_HIP_OP_YOLO_DETECT: return true;
+        default: return false;
+      }
+    };
+    auto writes_pitched = [&](int i) {
+      const GraphOp& o = ops[i];
+      if (nodes_[i].se_head || nodes_[i].skip) return false;
+      switch (o.kind) {
+        case NNCV_HIP_OP_CONV: return o.in[1] < 0 && nodes_[i].add_res < 0;  // residual and result share one pitch
+        case NNCV_HIP_OP_MAXPOOL:
+        case NNCV_HIP_OP_UPSAMPLE2X:
+        case NNCV_HIP_OP_ADD:
+        case NNCV_HIP_OP_ACT:
+        case NNCV_HIP_OP_CONCAT: return true;
+        default: return false;
+      }
+    };
+    for (int i = 0; i < n; ++i) {
+      if (ops[i].kind != NNCV_HIP_OP_CONCAT) continue;
+      int c0 = 0;
+      for (int k = 0; k < 4; ++k) {
+        const int t = ops[i].in[k];
+        if (t < 0) continue;
+        bool ok = t != 0 && cat_uses[t] == 1 && producer[t] >= 0 && writes_pitched(producer[t]) && logical_[t] == channels_[t];
+        for (int j = 0; ok && j < n; ++j)
+          for (int q = 0; q < 4; ++q)
+            if (ops[j].in[q] == t && !reads_pitched(j, t)) ok = false;
+        if (ok) {
+          view_of_[t] = ops[i].out;
+          view_c0_[t] = c0;
+        }
+        c0 += channels_[t];
+      }
+    }
+  }
+}
+
+void Graph::root_of(int t, int* root, int* c0) const {
+  int off = 0;
+  while (view_of_[t] >= 0) {
+    off += view_c0_[t];
+    t = view_of_[t];
+  }
+  *root = t;
+  *c0 = off;
 }
 
 const Graph::Plan& Graph::plan_of(int N, int H, int W) const {
@@ -293,9 +376,26 @@ const Graph::Plan& Graph::plan_of(int N, int H, int W) const {
     if (nodes_[i].op.kind == NNCV_HIP_OP_YOLO_DETECT) life[t].bytes = 256;  // written straight to the caller's buffer
   }
   life[nodes_[n - 1].op.out].last_op = n + 1;
+  // a tensor that lives inside a concatenated one has no memory of its own; the concatenated
+  // tensor is live from its first such input to the last reader of any of them
+  for (int t = 1; t < n_tensors_; ++t) {
+    if (view_of_[t] < 0) continue;
+    int root, c0;
+    root_of(t, &root, &c0);
+    life[root].first_op = std::min(life[root].first_op, life[t].first_op);
+    life[root].last_op = std::max(life[root].last_op, life[t].last_op);
+  }
+  for (int t = 1; t < n_tensors_; ++t)
+    if (view_of_[t] >= 0) life[t] = TensorLife{life[t].first_op, life[t].first_op, 0, 0};
+  for (int i = 0; i < n; ++i)  // the output of a convolution that was merged with its ADD is never stored
+    if (nodes_[i].add_out >= 0) life[nodes_[i].op.out] = TensorLife{i + 1, i + 1, 0, 0};
   p.total = plan_offsets(life, 256);
   p.offset.resize(n_tensors_);
-  for (int t = 0; t < n_tensors_; ++t) p.offset[t] = life[t].offset;
+  for (int t = 0; t < n_tensors_; ++t) {
+    int root, c0;
+    root_of(t, &root, &c0);
+    p.offset[t] = life[root].offset + (size_t)c0 * es;
+  }
   if (plans_.size() >= 8) plans_.erase(plans_.begin());
   plans_.push_back(std::move(p));
   return plans_.back();
@@ -315,6 +415,13 @@ void Graph::forward(const void* src, int N, int H, int W, float* out, void* ws, 
   const Plan& p = plan_of(N, H, W);
   char* base = static_cast<char*>(ws);
   auto at = [&](int t) -> void* { return base + p.offset[t]; };
+  // elements between consecutive pixels of tensor t: its own channel count, or that of the
+  // concatenated tensor it lives in
+  auto pitch = [&](int t) {
+    int root, c0;
+    root_of(t, &root, &c0);
+    return channels_[root];
+  };
   launch_relayout(src, dt_, strides_of(kNCHW, c_in_, H, W), at(0), dt_, strides_of(kNHWC, channels_[0], H, W), N, c_in_,
                   channels_[0], H, W, false, s);
   for (size_t i = 0; i < nodes_.size(); ++i) {
@@ -334,13 +441,20 @@ void Graph::forward(const void* src, int N, int H, int W, float* out, void* ws, 
     switch (op.kind) {
       case NNCV_HIP_OP_CONV: {
         IgemmArgs g{};
-        g.in = at(op.in[0]); g.wt = nd.wt.get(); g.wt_frag = nd.wfrag.get(); g.out = at(op.out);
+        const int dst = nd.add_out >= 0 ? nd.add_out : op.out;
+        g.in = at(op.in[0]); g.wt = nd.wt.get(); g.wt_frag = nd.wfrag.get(); g.out = at(dst);
         g.scale = nd.scale.as<float>(); g.shift = nd.shift.as<float>();
-        g.residual = op.in[1] >= 0 ? at(op.in[1]) : nullptr;
+        g.residual = nd.add_res >= 0 ? at(nd.add_res) : (op.in[1] >= 0 ? at(op.in[1]) : nullptr);
         // padding filters (zero rows, zero scale/shift) are computed like any other: o.C >= op.F
         g.N = N; g.H = a.H; g.W = a.W; g.C = a.C; g.F = o.C; g.R = g.S = op.K; g.OH = o.H; g.OW = o.W;
         g.stride_h = g.stride_w = op.stride; g.pad_h = g.pad_w = op.pad;
-        g.relu = op.act; g.ldo = o.C; g.batch = 1;
+        g.relu = nd.add_res >= 0 ? (op.act | kActResidualAfter) : op.act;
+        g.ldo = pitch(dst); g.batch = 1;
+        if (pitch(op.in[0]) != a.C) {  // the input is a slice of a wider tensor
+          g.pix_stride = pitch(op.in[0]);
+          const unsigned long long span = (unsigned long long)N * a.H * a.W * g.pix_stride * dtype_size(dt_);
+          g.in_bytes = span < 0xffffffffull ? (unsigned)span : 0xffffffffu;
+        }
         g.alg_flops = 2.0 * N * o.H * o.W * op.F * (double)op.K * op.K * logical_[op.in[0]];
         launch_igemm(g, dt_, dt_, s);
         break;
@@ -355,7 +469,8 @@ void Graph::forward(const void* src, int N, int H, int W, float* out, void* ws, 
         break;
       }
       case NNCV_HIP_OP_MAXPOOL:
-        launch_maxpool_nhwc(at(op.in[0]), at(op.out), dt_, N, a.H, a.W, a.C, op.K, op.stride, op.pad, s);
+        launch_maxpool_nhwc(at(op.in[0]), at(op.out), dt_, N, a.H, a.W, a.C, op.K, op.stride, op.pad, s, pitch(op.in[0]),
+                            pitch(op.out));
         break;
       case NNCV_HIP_OP_GAVGPOOL:
         launch_global_avgpool_nhwc(at(op.in[0]), at(op.out), dt_, N, a.H * a.W, a.C, s);
@@ -364,30 +479,35 @@ void Graph::forward(const void* src, int N, int H, int W, float* out, void* ws, 
         launch_scale_channels(at(op.in[0]), at(op.in[1]), at(op.out), dt_, N, a.H * a.W, a.C, s);
         break;
       case NNCV_HIP_OP_ADD:
-        launch_eltwise(at(op.in[0]), at(op.in[1]), at(op.out), dt_, (long long)N * a.H * a.W * a.C, op.act, s);
+        launch_eltwise_pitched(at(op.in[0]), pitch(op.in[0]), at(op.in[1]), pitch(op.in[1]), at(op.out), pitch(op.out), dt_,
+                               (long long)N * a.H * a.W, a.C, op.act, s);
         break;
       case NNCV_HIP_OP_ACT:
-        launch_eltwise(at(op.in[0]), nullptr, at(op.out), dt_, (long long)N * a.H * a.W * a.C, op.act, s);
+        launch_eltwise_pitched(at(op.in[0]), pitch(op.in[0]), nullptr, pitch(op.in[0]), at(op.out), pitch(op.out), dt_,
+                               (long long)N * a.H * a.W, a.C, op.act, s);
         break;
       case NNCV_HIP_OP_CONCAT: {
         int c0 = 0;
         for (int k = 0; k < 4; ++k) {
           if (op.in[k] < 0) continue;
           const int Ck = p.dims[op.in[k]].C;
-          launch_concat_slice(at(op.in[k]), at(op.out), dt_, (long long)N * o.H * o.W, Ck, o.C, c0, s);
+          // inputs that live in this tensor already are in place; the others are copied into their slice
+          if (view_of_[op.in[k]] != op.out)
+            launch_concat_slice(at(op.in[k]), static_cast<char*>(at(op.out)) + (size_t)c0 * dtype_size(dt_), dt_,
+                                (long long)N * o.H * o.W, Ck, pitch(op.out), 0, s, pitch(op.in[k]));
           c0 += Ck;
         }
         break;
       }
       case NNCV_HIP_OP_UPSAMPLE2X:
-        launch_upsample2x(at(op.in[0]), at(op.out), dt_, N, a.H, a.W, a.C, a.C, 0, s);
+        launch_upsample2x(at(op.in[0]), at(op.out), dt_, N, a.H, a.W, a.C, pitch(op.out), 0, s, pitch(op.in[0]));
         break;
       case NNCV_HIP_OP_YOLO_DETECT: {
         long long box0 = 0;
         for (int k = 0; k < 3 && op.in[k] >= 0; ++k) {
           const Dims h = p.dims[op.in[k]];
           DetectArgs d{};
-          d.head = at(op.in[k]); d.out = out; d.N = N; d.H = h.H; d.W = h.W; d.A = op.K; d.F = op.F; d.ldc = h.C;
+          d.head = at(op.in[k]); d.out = out; d.N = N; d.H = h.H; d.W = h.W; d.A = op.K; d.F = op.F; d.ldc = pitch(op.in[k]);
           d.box0 = box0; d.boxes_total = o.C; d.stride = detect_stride_[k];
           for (int q = 0; q < op.K * 2; ++q) d.anchor_wh[q] = detect_anchor_wh_[k * op.K * 2 + q];
           launch_yolo_detect(d, dt_, s);

@@ -40,6 +40,10 @@ class Graph {
     // tensor" whose three intermediate tensors have no other reader: the four operators run as one
     // squeeze-excitation launch and the next three nodes are skipped.
     bool se_head = false, skip = false;
+    // Set on a CONV whose only reader is the ADD that follows it (x + act(conv), a YOLOv5
+    // Bottleneck): the convolution adds `add_res` after its activation and writes the ADD's
+    // output tensor `add_out`; the ADD node is skipped.
+    int add_res = -1, add_out = -1;
   };
   struct Dims { int C, H, W; };
   struct Plan {
@@ -54,6 +58,11 @@ class Graph {
   std::vector<Node> nodes_;
   std::vector<int> channels_;  // per tensor, as stored (padded to a whole 16-byte vector)
   std::vector<int> logical_;   // per tensor, as the network defines it
+  // Concatenation without copies: a tensor that is an input of one CONCAT, and whose producer and
+  // readers can all address rows at a pitch, lives inside the concatenated tensor (`view_of_` =
+  // that tensor, `view_c0_` = its channel offset there).  Chains are resolved by root_of().
+  std::vector<int> view_of_, view_c0_;
+  void root_of(int t, int* root, int* c0) const;
   std::vector<float> detect_anchor_wh_, detect_stride_;  // YOLO_DETECT: host copies of anchors * stride, strides
   std::vector<int> last_use_;  // per tensor: index of the last operator that reads it
   mutable std::vector<Plan> plans_;

@@ -192,17 +192,27 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(const IgemmArgs a) {
         if (a.scale) y *= *reinterpret_cast<const floatx4*>(a.scale + f0);
         if (a.shift) y += *reinterpret_cast<const floatx4*>(a.shift + f0);
         const long long o = (long long)gp * a.ldo + f0;
+        const bool res_after = a.relu & kActResidualAfter;
+        float r4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         if (res) {
           const V4 rv = *reinterpret_cast<const V4*>(res + o);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) y[e] += (float)rv[e];
+          for (int e = 0; e < 4; ++e) r4[e] = (float)rv[e];
+        }
+        if (res && !res_after) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) y[e] += r4[e];
         }
         if (a.relu == kActRelu) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) y[e] = relu_ugt(y[e]);
         } else if (a.relu) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) y[e] = act_apply(y[e], a.relu);
+          for (int e = 0; e < 4; ++e) y[e] = act_apply(y[e], a.relu & 0xff);
+        }
+        if (res && res_after) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) y[e] += r4[e];
         }
         V4 ov;
 #pragma unroll

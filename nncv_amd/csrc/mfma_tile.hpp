@@ -164,7 +164,8 @@ __device__ __forceinline__ void tile_reduce_store(const floatx16 (&acc)[2][2], u
     for (int q = 0; q < FPL / 4; ++q)
 #pragma unroll
       for (int e = 0; e < 4; ++e) y[4 * q + e] = v[it][q][e] * ss.sc[4 * q + e] + ss.sh[4 * q + e];
-    if (res) {
+    const bool res_after = ACT && (relu & kActResidualAfter);  // y = act(conv) + residual instead of act(conv + residual)
+    if (res && !res_after) {
 #pragma unroll
       for (int e = 0; e < FPL; ++e) y[e] += (float)rv[it][e];
     }
@@ -173,7 +174,11 @@ __device__ __forceinline__ void tile_reduce_store(const floatx16 (&acc)[2][2], u
       for (int e = 0; e < FPL; ++e) y[e] = relu_ugt(y[e]);
     } else if (ACT && relu) {
 #pragma unroll
-      for (int e = 0; e < FPL; ++e) y[e] = act_apply(y[e], relu);
+      for (int e = 0; e < FPL; ++e) y[e] = act_apply(y[e], relu & 0xff);
+    }
+    if (res && res_after) {
+#pragma unroll
+      for (int e = 0; e < FPL; ++e) y[e] += (float)rv[it][e];
     }
     VO ov;
 #pragma unroll

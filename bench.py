@@ -50,14 +50,16 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--batch", type=int, default=32)
+    ap.add_argument("--batch", type=int, default=0, help="0 = the workload's default (32; yolov5s 16)")
     ap.add_argument("--algo", default="auto", choices=["auto", "winograd", "igemm"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-batch1", action="store_true", help="skip the batch-1 measurement (for per-kernel profiles)")
     ap.add_argument("--profile-steps", type=int, default=5)
-    ap.add_argument("--workload", default="resnet18", choices=["resnet18", "mobilenetv3"],
-                    help="resnet18 = the headline configuration; mobilenetv3 = the network of tests/Nets/MobileNetV3.mlir "
-                         "through the operator-list executor (same step definition, its own JSON line)")
+    ap.add_argument("--workload", default="resnet18", choices=["resnet18", "mobilenetv3", "yolov5s"],
+                    help="resnet18 = the headline configuration; mobilenetv3 / yolov5s = the networks of tests/Nets/MobileNetV3.mlir "
+                         "and Yolov5s.mlir through the operator-list executor (same step definition, their own JSON line; "
+                         "default batch 32 at 224x224 and 16 at 640x640)")
+    ap.add_argument("--image", type=int, default=0, help="image side for the graph workloads (0 = 224 / 640)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a known-size kernel to scale HBM counters by)")
     args = ap.parse_args()
@@ -74,8 +76,10 @@ def main():
         sys.stderr.write("bench.py: no GPU visible\n")
         sys.exit(1)
     L = abi.lib()  # raises if the HIP library is missing: there is no fallback path
-    if args.workload == "mobilenetv3":
-        return bench_mobilenetv3(args, L)
+    if args.batch <= 0:
+        args.batch = 16 if args.workload == "yolov5s" else 32
+    if args.workload != "resnet18":
+        return bench_graph(args, L)
     algo = {"auto": abi.ALGO_AUTO, "winograd": abi.ALGO_WINOGRAD, "igemm": abi.ALGO_IGEMM}[args.algo]
 
     N, H = args.batch, 224
@@ -200,24 +204,35 @@ def main():
     print(json.dumps(out))
 
 
-def bench_mobilenetv3(args, L):
-    """MobileNetV3-small forward (fp16 storage / fp32 accumulate, [batch,3,224,224] resident in HBM) through
-    nncv_hip_graph_forward; same timing protocol as the headline workload."""
+def bench_graph(args, L):
+    """MobileNetV3-small ([batch,3,224,224] -> [batch,1000]) or YOLOv5s ([batch,3,640,640] -> [batch,25200,85]) forward, fp16
+    storage / fp32 accumulate, input resident in HBM, through nncv_hip_graph_forward; same timing protocol as the
+    headline workload."""
     import numpy as np
     import torch
-    from nncv_amd import abi, mobilenetv3_spec as mspec, synth
+    from nncv_amd import abi, synth
+    import oracle
 
-    N, H = args.batch, 224
-    blob32 = synth.mobilenetv3_params()
-    ops, n_elems = abi.mobilenetv3_small_ops()
+    yolo = args.workload == "yolov5s"
+    N, H = args.batch, args.image or (640 if yolo else 224)
+    if yolo:
+        from nncv_amd import yolov5s_spec as mspec
+        blob32, ops = synth.yolov5s_params(), mspec.graph_ops()
+        name, fixture = "YOLOv5s", "tests/Nets/Yolov5s.mlir"
+    else:
+        from nncv_amd import mobilenetv3_spec as mspec
+        blob32, ops = synth.mobilenetv3_params(), abi.mobilenetv3_small_ops()[0]
+        name, fixture = "MobileNetV3-small", "tests/Nets/MobileNetV3.mlir"
     g = abi.graph_create(ops, 3, blob32.astype(np.float16))
-    x = synth.cfg4_input(N).astype(np.float16)
+    oc, oh, ow = abi.graph_output_shape(g, H, H)
+    per_image = oc * oh * ow
+    x = synth.uniform(4000, (N, 3, H, H), 0.0, 1.0).astype(np.float16)
     xd = torch.from_numpy(x).cuda()
-    logits = torch.empty((N, 1000), dtype=torch.float32, device="cuda")
+    result = torch.empty((N, per_image), dtype=torch.float32, device="cuda")
     stream = torch.cuda.current_stream().cuda_stream
 
     def step(xt, out, n):
-        abi.check(L.nncv_hip_graph_forward(g, xt.data_ptr(), n, H, H, out.data_ptr(), n * 1000, stream))
+        abi.check(L.nncv_hip_graph_forward(g, xt.data_ptr(), n, H, H, out.data_ptr(), n * per_image, stream))
 
     def timed(xt, out, n, warmup, steps):
         for _ in range(warmup):
@@ -229,13 +244,13 @@ def bench_mobilenetv3(args, L):
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps
 
-    sec = timed(xd, logits, N, args.warmup, args.steps)
-    x1, l1 = xd[:1].contiguous(), torch.empty((1, 1000), dtype=torch.float32, device="cuda")
-    sec1 = None if args.no_batch1 else timed(x1, l1, 1, args.warmup, max(args.steps, 50))
+    sec = timed(xd, result, N, args.warmup, args.steps)
+    x1, r1 = xd[:1].contiguous(), torch.empty((1, per_image), dtype=torch.float32, device="cuda")
+    sec1 = None if args.no_batch1 else timed(x1, r1, 1, args.warmup, max(args.steps, 50))
     abi.profile_enable(True)
     abi.profile_report()
     for _ in range(args.profile_steps):
-        step(xd, logits, N)
+        step(xd, result, N)
     torch.cuda.synchronize()
     prof = abi.profile_report()
     abi.profile_enable(False)
@@ -244,44 +259,57 @@ def bench_mobilenetv3(args, L):
     for tag, v in sorted(prof.items(), key=lambda kv: -kv[1]["ms"]):
         kernels[tag] = {"launches_per_step": v["launches"] / args.profile_steps, "ms_per_step": round(v["ms"] / args.profile_steps, 5),
                         "share": round(v["ms"] / total_ms, 4), "avg_launch_us": round(v["ms"] / v["launches"] * 1e3, 3),
+                        "tflops": round(v["flops"] / (v["ms"] * 1e-3) / 1e12, 3) if v["flops"] else None,
                         "gbs": round(v["bytes"] / (v["ms"] * 1e-3) / 1e9, 2)}
-    # every kernel of this network moves a few MB per launch: the bound is HBM / launch latency, so the
-    # dominant tag is priced in algorithmic bytes (one HIP event pair per launch, ~4 us of event latency included)
+    # Dominant tag, one HIP event pair per launch (~4 us of event latency included).  MobileNetV3's launches move a
+    # few MB each: priced in algorithmic bytes against HBM.  YOLOv5s' dominant tag is an MFMA convolution instance.
     dom = max(prof, key=lambda t: prof[t]["ms"])
     d = prof[dom]
-    achieved = d["bytes"] / (d["ms"] * 1e-3) / 1e9
-    roofline = {"kernel": dom, "bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 5), "traffic": None, "avg_launch_us": round(d["ms"] / d["launches"] * 1e3, 3),
-                "launches": d["launches"], "timing": "one HIP event pair per launch"}
+    if yolo and d["flops"] > 0:
+        achieved = d["flops"] / (d["ms"] * 1e-3) / 1e12
+        roofline = {"kernel": dom, "bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 5)}
+    else:
+        achieved = d["bytes"] / (d["ms"] * 1e-3) / 1e9
+        roofline = {"kernel": dom, "bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(achieved / HBM_PEAK_GBS, 5)}
+    roofline.update({"traffic": None, "avg_launch_us": round(d["ms"] / d["launches"] * 1e3, 3), "launches": d["launches"],
+                     "timing": "one HIP event pair per launch, all launches of the tag in %d passes" % args.profile_steps})
     flops_step = mspec.flops_per_image(H) * N
     out = {
-        "metric": "mobilenetv3_small_fp16_bs%d_images_per_s" % N, "value": round(N / sec, 2), "unit": "images/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec * 1e3, 4),
+        "metric": "%s_fp16_bs%d_images_per_s" % ("yolov5s" if yolo else "mobilenetv3_small", N), "value": round(N / sec, 2),
+        "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 (fp32 accumulate)", "data": "synthetic",
-        "config": {"workload": "MobileNetV3-small forward (the network of tests/Nets/MobileNetV3.mlir), fp16, input [%d,3,224,224], "
-                               "seeded U[0,1] input, random-init weights from a model.bin-order blob" % N,
+        "config": {"workload": "%s forward (the network of %s), fp16, input [%d,3,%d,%d], seeded U[0,1] input, random-init weights "
+                               "from a model.bin-order blob" % (name, fixture, N, H, H),
                    "batch": N, "image": H, "input_resident_in_hbm": True},
         "tflops_effective": round(flops_step / sec / 1e12, 3),
         "batch1": None if sec1 is None else {"images_per_s": round(1.0 / sec1, 2), "ms_per_image": round(sec1 * 1e3, 4)},
         "roofline": roofline, "kernels": kernels, "device": L.nncv_hip_device_arch().decode(),
     }
     if not args.no_cpu_baseline:
-        import oracle
         hb = synth.round_fp16(blob32)
-        T = {name: hb[o:o + mspec.numel(shape)].reshape(shape) for name, (o, shape) in mspec.offsets().items()}
         xf = x.astype(np.float32)
-        nb = min(8, N)
-        oracle.mobilenetv3_forward(xf[:1], T)
+        nb = min(2 if yolo else 8, N)
+        if yolo:
+            run = lambda xs: oracle.run_graph(ops, xs, hb, 3, conv=oracle.hwp_conv2d)
+            what = "operator-list evaluator of oracle/ with the OpenMP x AVX2 convolution (oracle/hostwparallel.cpp), numpy for the rest"
+            cores = min(len(os.sched_getaffinity(0)), int(os.environ.get("OMP_NUM_THREADS", 1 << 10)))
+        else:
+            T = {n_: hb[o:o + mspec.numel(shape)].reshape(shape) for n_, (o, shape) in mspec.offsets().items()}
+            run = lambda xs: oracle.mobilenetv3_forward(xs, T)
+            what = "scalar C / numpy restatement of the fixture's operators (oracle/)"
+            cores = 1
+        run(xf[:1])
         done, t0 = 0, time.perf_counter()
         while True:
-            oracle.mobilenetv3_forward(xf[:nb], T)
+            run(xf[:nb])
             done += nb
             dt = time.perf_counter() - t0
             if dt > 10.0 or done >= 4096:
                 break
-        out["cpu_baseline"] = {"value": round(done / dt, 3), "unit": "images/s", "cores": 1, "kind": "port",
-                               "sample": "%d images (batches of %d) in %.1f s; fp32 scalar C / numpy restatement of the fixture's "
-                                         "operators (oracle/)" % (done, nb, dt)}
+        out["cpu_baseline"] = {"value": round(done / dt, 3), "unit": "images/s", "cores": cores, "kind": "port",
+                               "sample": "%d images (batches of %d) in %.1f s; fp32, %s" % (done, nb, dt, what)}
     L.nncv_hip_graph_destroy(g)
     print(json.dumps(out))
 

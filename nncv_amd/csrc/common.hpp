@@ -172,6 +172,9 @@ void launch_argmax_rows(const float* x, int* idx, int N, int F, hipStream_t s);
 // generic strided copy/cast between layouts: dst[n,c,h,w] (+)= (c < Csrc ? src[n,c,h,w] : 0) for c < Cdst
 void launch_relayout(const void* src, int src_dt, Strides4 ss, void* dst, int dst_dt, Strides4 ds, int N,
                      int Csrc, int Cdst, int H, int W, bool accumulate, hipStream_t s);
+// image [N,C,H,W] with C <= one 16-byte vector -> NHWC [N,H,W,vector], zero padded channels
+bool image_to_nhwc_applicable(int dt, int C);
+void launch_image_to_nhwc(const void* src, void* dst, int dt, int N, int C, int H, int W, hipStream_t s);
 // stem input: NCHW [N,3,H,W] -> zero-haloed pixel-pair image [N][H+6][(W+8)/2][8]
 void launch_stem_pack(const void* src, int src_dt, void* dst, int dst_dt, int N, int H, int W, hipStream_t s);
 // weights FCRS -> [F][R][S][Cp] (Cp >= C, zero filled), cast to dst_dt

@@ -545,39 +545,39 @@ void launch_maxpool_nhwc(const void* in, void* out, int dt, int N, int H, int W,
 // ---------------------------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void yolo_detect_kernel(const DetectArgs a) {
-  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  const long long per_img = (long long)a.A * a.H * a.W * a.F;
-  if (idx >= per_img * a.N) return;
-  const int n = (int)(idx / per_img);
-  long long r = idx - n * per_img;
-  const int k = (int)(r % a.F);
-  r /= a.F;
-  const int x = (int)(r % a.W);
-  r /= a.W;
-  const int y = (int)(r % a.H);
-  const int an = (int)(r / a.H);
+  // blockIdx.y = (image, anchor); blockIdx.x walks the H*W*F values of that anchor, F fastest
+  const int n = blockIdx.y / a.A, an = blockIdx.y - n * a.A;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  const int HWF = a.H * a.W * a.F;
+  if (i >= HWF) return;
+  const int pix = i / a.F, k = i - pix * a.F;
   const T* head = static_cast<const T*>(a.head);
-  const float v = (float)head[(((long long)n * a.H + y) * a.W + x) * a.ldc + an * a.F + k];
+  const float v = (float)head[((long long)n * a.H * a.W + pix) * a.ldc + an * a.F + k];
   const float sg = 1.0f / (expf(-v) + 1.0f);
   float o = sg;
-  if (k < 2) {
-    const float g = (float)(k == 0 ? x : y) - 0.5f;
-    o = (sg * 2.0f + g) * a.stride;
-  } else if (k < 4) {
-    const float t = sg * 2.0f;
-    o = (t * t) * a.anchor_wh[an * 2 + (k - 2)];
+  if (k < 4) {
+    const int y = pix / a.W, x = pix - y * a.W;
+    if (k < 2) {
+      const float g = (float)(k == 0 ? x : y) - 0.5f;
+      o = (sg * 2.0f + g) * a.stride;
+    } else {
+      const float t = sg * 2.0f;
+      o = (t * t) * a.anchor_wh[an * 2 + (k - 2)];
+    }
   }
-  a.out[((long long)n * a.boxes_total + a.box0 + ((long long)an * a.H + y) * a.W + x) * a.F + k] = o;
+  a.out[((long long)n * a.boxes_total + a.box0 + (long long)an * a.H * a.W) * a.F + i] = o;
 }
 
 void launch_yolo_detect(const DetectArgs& a, int dt, hipStream_t s) {
   NNCV_REQUIRE(a.A >= 1 && a.A <= 4 && a.F >= 5 && a.A * a.F <= a.ldc && a.N >= 1 && a.H >= 1 && a.W >= 1, "yolo_detect: bad shape");
+  NNCV_REQUIRE((long long)a.H * a.W * a.F < (1ll << 31) && (long long)a.N * a.A <= 65535, "yolo_detect: level too large");
   const long long work = (long long)a.N * a.A * a.H * a.W * a.F;
   ProfScope prof("yolo_detect", 0.0, (double)work * (dtype_size(dt) + 4.0), s);
+  dim3 grid((unsigned)(((long long)a.H * a.W * a.F + 255) / 256), (unsigned)(a.N * a.A));
   if (dt == kF16)
-    hipLaunchKernelGGL((yolo_detect_kernel<half_t>), dim3(grid_for(work)), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((yolo_detect_kernel<half_t>), grid, dim3(256), 0, s, a);
   else
-    hipLaunchKernelGGL((yolo_detect_kernel<float>), dim3(grid_for(work)), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((yolo_detect_kernel<float>), grid, dim3(256), 0, s, a);
   NNCV_HIP_CHECK(hipGetLastError());
 }
 

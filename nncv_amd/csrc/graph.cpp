@@ -422,8 +422,11 @@ void Graph::forward(const void* src, int N, int H, int W, float* out, void* ws, 
     root_of(t, &root, &c0);
     return channels_[root];
   };
-  launch_relayout(src, dt_, strides_of(kNCHW, c_in_, H, W), at(0), dt_, strides_of(kNHWC, channels_[0], H, W), N, c_in_,
-                  channels_[0], H, W, false, s);
+  if (image_to_nhwc_applicable(dt_, c_in_))
+    launch_image_to_nhwc(src, at(0), dt_, N, c_in_, H, W, s);
+  else
+    launch_relayout(src, dt_, strides_of(kNCHW, c_in_, H, W), at(0), dt_, strides_of(kNHWC, channels_[0], H, W), N, c_in_,
+                    channels_[0], H, W, false, s);
   for (size_t i = 0; i < nodes_.size(); ++i) {
     const Node& nd = nodes_[i];
     const GraphOp& op = nd.op;

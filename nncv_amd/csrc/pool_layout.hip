@@ -361,6 +361,41 @@ void launch_relayout(const void* src, int src_dt, Strides4 ss, void* dst, int ds
 }
 
 // ---------------------------------------------------------------------------------------------
+// Network input of the graph executor: NCHW with a few channels (an image: 3) -> NHWC padded to
+// one 16-byte vector per pixel.  One thread per pixel: the C plane reads are coalesced across the
+// wave (consecutive pixels), the write is one whole vector per lane.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void image_to_nhwc_kernel(const T* __restrict__ src, T* __restrict__ dst, int C, long long HW,
+                                                            long long total) {
+  constexpr int VN = Vec16<T>::n;
+  typedef typename Vec16<T>::type V;
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const long long n = idx / HW, p = idx - n * HW;
+  V v;
+#pragma unroll
+  for (int c = 0; c < VN; ++c) v[c] = c < C ? src[(n * C + c) * HW + p] : (T)0.0f;
+  *reinterpret_cast<V*>(dst + idx * VN) = v;
+}
+
+bool image_to_nhwc_applicable(int dt, int C) { return C >= 1 && C <= (dt == kF16 ? 8 : 4); }
+
+void launch_image_to_nhwc(const void* src, void* dst, int dt, int N, int C, int H, int W, hipStream_t s) {
+  NNCV_REQUIRE(image_to_nhwc_applicable(dt, C), "image_to_nhwc: too many channels for one vector");
+  const long long HW = (long long)H * W, total = HW * N;
+  if (total == 0) return;
+  const long long grid = (total + 255) / 256;
+  NNCV_REQUIRE(grid < (1ll << 31), "image_to_nhwc: grid too large");
+  ProfScope prof("image_to_nhwc", 0.0, (double)dtype_size(dt) * total * (C + (dt == kF16 ? 8 : 4)), s);
+  if (dt == kF16)
+    hipLaunchKernelGGL((image_to_nhwc_kernel<half_t>), dim3((unsigned)grid), dim3(256), 0, s, (const half_t*)src, (half_t*)dst, C, HW, total);
+  else
+    hipLaunchKernelGGL((image_to_nhwc_kernel<float>), dim3((unsigned)grid), dim3(256), 0, s, (const float*)src, (float*)dst, C, HW, total);
+  NNCV_HIP_CHECK(hipGetLastError());
+}
+
+// ---------------------------------------------------------------------------------------------
 // Stem input packing.  The 7x7 stride-2 pad-3 convolution over 3 channels
 // (tests/Nets/Res18.mlir:118-124) is run by the implicit-GEMM kernel as a 7x4 stride-(2,1)
 // convolution over "pixel pairs": the NCHW image becomes [N][H+6][Wp][8] where element

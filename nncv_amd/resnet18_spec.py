@@ -78,3 +78,41 @@ def flops_per_image(h):
         oh = (hin + 2 * p - r) // s + 1
         total += 2 * oh * oh * f * c * r * r
     return total + 2 * 512 * 1000
+
+
+def graph_ops():
+    """The same network as an operator list for the generic executor (nncv_hip_graph_*): what the
+    hard-wired ResNet18 object computes, without its fused stem / shortcut / head kernels."""
+    from . import abi
+    off = offsets()
+    ops = []
+    nxt = [1]
+
+    def new_id():
+        nxt[0] += 1
+        return nxt[0] - 1
+
+    def conv_bn(x, conv, bn, k, stride, pad, act, residual=-1):
+        o = abi.graph_op(abi.OP_CONV, [x, residual], new_id(), F=off[conv + ".weight"][1][0], K=k, stride=stride, pad=pad, act=act,
+                         eps=1e-5, w=off[conv + ".weight"][0],
+                         bn=tuple(off[bn + s][0] for s in (".weight", ".bias", ".running_mean", ".running_var")))
+        ops.append(o)
+        return o.out
+
+    x = conv_bn(0, "conv1", "bn1", 7, 2, 3, abi.ACT_RELU)
+    ops.append(abi.graph_op(abi.OP_MAXPOOL, [x], new_id(), K=3, stride=2, pad=1))
+    x = ops[-1].out
+    cin = 64
+    for li, f in enumerate(WIDTHS, start=1):
+        for blk in range(2):
+            p = "layer%d.%d" % (li, blk)
+            stride = 2 if (li > 1 and blk == 0) else 1
+            idn = x
+            y = conv_bn(x, p + ".conv1", p + ".bn1", 3, stride, 1, abi.ACT_RELU)
+            if stride != 1 or cin != f:
+                idn = conv_bn(x, p + ".downsample.0", p + ".downsample.1", 1, stride, 0, abi.ACT_NONE)
+            x = conv_bn(y, p + ".conv2", p + ".bn2", 3, 1, 1, abi.ACT_RELU, residual=idn)
+            cin = f
+    ops.append(abi.graph_op(abi.OP_GAVGPOOL, [x], new_id(), stride=0))
+    ops.append(abi.graph_op(abi.OP_CONV, [ops[-1].out], new_id(), F=1000, K=1, w=off["fc.weight"][0], bias=off["fc.bias"][0]))
+    return ops

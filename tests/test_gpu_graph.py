@@ -325,3 +325,25 @@ def test_squeeze_excitation_block(dt, C, SQ, H, W, N):
     else:
         assert rel_l2(got, want) < 2e-3
     g.close()
+
+
+@pytest.mark.parametrize("dt", [abi.F32, abi.F16])
+def test_resnet18_as_an_operator_list(dt):
+    """tests/Nets/Res18.mlir through the generic executor: same logits as the oracle and as the hard-wired model."""
+    from nncv_amd import resnet18_spec
+    from gpu_util import Model
+    blob = synth.resnet18_params()
+    x = synth.uniform(7700, (2, 3, 96, 64), 0.0, 1.0)
+    if dt == abi.F16:
+        blob, x = r16(blob), r16(x)
+    g = Graph(resnet18_spec.graph_ops(), 3, blob, dt)
+    xd = dev(x, dt)
+    got = host(g(xd)).reshape(2, 1000)
+    want = oracle.resnet18_forward(x, blob)
+    hard = host(Model(blob, dt)(xd))
+    if dt == abi.F32:
+        assert max_rel(got, want) < FP32_MAX_REL and max_rel(hard, want) < FP32_MAX_REL
+    else:
+        assert rel_l2(got, want) < FP16_REL_L2 and rel_l2(got, hard) < FP16_REL_L2
+    assert np.array_equal(got.argmax(1), want.argmax(1))
+    g.close()

@@ -65,3 +65,14 @@ def test_resnet18_oracle_non_square_batch_independent():
     both = oracle.resnet18_forward(x, blob)
     one = oracle.resnet18_forward(x[1:2], blob)
     assert np.array_equal(both[1:2], one)
+
+
+def test_operator_list_evaluator_reproduces_the_network_oracle():
+    """oracle.run_graph over resnet18_spec.graph_ops() (the checker of the generic executor) against the
+    C restatement of the whole network, which the tests above pin: two independently written walks of
+    tests/Nets/Res18.mlir must agree."""
+    blob = synth.resnet18_params()
+    x = synth.uniform(3009, (2, 3, 72, 56), 0.0, 1.0)
+    got = oracle.run_graph(spec.graph_ops(), x, blob, 3).reshape(2, 1000)
+    want = oracle.resnet18_forward(x, blob)
+    assert np.abs(got - want).max() <= 1e-6 * np.abs(want).max()

@@ -174,7 +174,12 @@ void launch_relayout(const void* src, int src_dt, Strides4 ss, void* dst, int ds
                      int Csrc, int Cdst, int H, int W, bool accumulate, hipStream_t s);
 // image [N,C,H,W] with C <= one 16-byte vector -> NHWC [N,H,W,vector], zero padded channels
 bool image_to_nhwc_applicable(int dt, int C);
-void launch_image_to_nhwc(const void* src, void* dst, int dt, int N, int C, int H, int W, hipStream_t s);
+// (Cp: channels per pixel of dst, 0 = one vector; 4 with fp16 = the pixel-pair form)
+void launch_image_to_nhwc(const void* src, void* dst, int dt, int N, int C, int H, int W, hipStream_t s, int Cp = 0);
+// fp16 filters [F,C<=4,K,K] of a stride-2 convolution re-laid for an image stored as pixel pairs:
+// dst [Fp][K][S2][8], S2 = ceil((K + pad%2) / 2); the convolution then runs with S = S2, stride 1 and
+// padding (pad + 1) / 2 along x over W/2 pairs of 8 channels
+void launch_weight_pairs(const void* w, int w_dt, void* dst, int F, int Fp, int C, int K, int pad, hipStream_t s);
 // stem input: NCHW [N,3,H,W] -> zero-haloed pixel-pair image [N][H+6][(W+8)/2][8]
 void launch_stem_pack(const void* src, int src_dt, void* dst, int dst_dt, int N, int H, int W, hipStream_t s);
 // weights FCRS -> [F][R][S][Cp] (Cp >= C, zero filled), cast to dst_dt

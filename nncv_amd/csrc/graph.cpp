@@ -229,6 +229,19 @@ Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, lon
     i += 3;
   }
 
+  // an image convolution (fp16, <= 4 channels, stride 2) that is the only reader of the input
+  static const bool no_pairs = getenv("NNCV_HIP_NO_PAIR_STEM") != nullptr;
+  if (!no_pairs && dt == kF16 && c_in_ <= 4 && readers[0] == 1)
+    for (int i = 0; i < n; ++i)
+      if (ops[i].kind == NNCV_HIP_OP_CONV && ops[i].in[0] == 0 && ops[i].stride == 2 && ops[i].in[1] < 0) {
+        const GraphOp& o = ops[i];
+        const int Fp = channels_[o.out], S2 = (o.K + (o.pad & 1) + 1) / 2;
+        nodes_[i].wt_pairs.reset((size_t)Fp * o.K * S2 * 8 * es);
+        launch_weight_pairs(param(o.w, (long long)o.F * c_in_ * o.K * o.K, "pair stem w"), dt, nodes_[i].wt_pairs.get(), o.F, Fp, c_in_,
+                            o.K, o.pad, s);
+        pair_stem_ = i;
+      }
+
   // x + act(conv(.)): the ADD rides in the convolution's epilogue
   static const bool no_add = getenv("NNCV_HIP_NO_ADD_FUSION") != nullptr;
   for (int i = 0; !no_add && i + 1 < n; ++i) {
@@ -422,7 +435,10 @@ void Graph::forward(const void* src, int N, int H, int W, float* out, void* ws, 
     root_of(t, &root, &c0);
     return channels_[root];
   };
-  if (image_to_nhwc_applicable(dt_, c_in_))
+  const bool pairs = pair_stem_ >= 0 && W % 2 == 0;
+  if (pairs)
+    launch_image_to_nhwc(src, at(0), dt_, N, c_in_, H, W, s, 4);
+  else if (image_to_nhwc_applicable(dt_, c_in_))
     launch_image_to_nhwc(src, at(0), dt_, N, c_in_, H, W, s);
   else
     launch_relayout(src, dt_, strides_of(kNCHW, c_in_, H, W), at(0), dt_, strides_of(kNHWC, channels_[0], H, W), N, c_in_,
@@ -453,6 +469,11 @@ void Graph::forward(const void* src, int N, int H, int W, float* out, void* ws, 
         g.stride_h = g.stride_w = op.stride; g.pad_h = g.pad_w = op.pad;
         g.relu = nd.add_res >= 0 ? (op.act | kActResidualAfter) : op.act;
         g.ldo = pitch(dst); g.batch = 1;
+        if (pairs && (int)i == pair_stem_) {  // the image as [N][H][W/2][2 pixels x 4 channels]
+          g.wt = nd.wt_pairs.get();
+          g.W = a.W / 2; g.C = 8; g.S = (op.K + (op.pad & 1) + 1) / 2;
+          g.stride_w = 1; g.pad_w = (op.pad + 1) / 2;
+        }
         if (pitch(op.in[0]) != a.C) {  // the input is a slice of a wider tensor
           g.pix_stride = pitch(op.in[0]);
           const unsigned long long span = (unsigned long long)N * a.H * a.W * g.pix_stride * dtype_size(dt_);

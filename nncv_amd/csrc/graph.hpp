@@ -44,6 +44,7 @@ class Graph {
     // Bottleneck): the convolution adds `add_res` after its activation and writes the ADD's
     // output tensor `add_out`; the ADD node is skipped.
     int add_res = -1, add_out = -1;
+    DeviceBuffer wt_pairs;  // see pair_stem_
   };
   struct Dims { int C, H, W; };
   struct Plan {
@@ -62,6 +63,10 @@ class Graph {
   // readers can all address rows at a pitch, lives inside the concatenated tensor (`view_of_` =
   // that tensor, `view_c0_` = its channel offset there).  Chains are resolved by root_of().
   std::vector<int> view_of_, view_c0_;
+  // Index of the one convolution that reads the network input, when it is an fp16 stride-2
+  // convolution over <= 4 channels: for even W the input is then stored as pixel pairs (4 channels
+  // per pixel) and that convolution walks pairs (launch_weight_pairs); -1 otherwise.
+  int pair_stem_ = -1;
   void root_of(int t, int* root, int* c0) const;
   std::vector<float> detect_anchor_wh_, detect_stride_;  // YOLO_DETECT: host copies of anchors * stride, strides
   std::vector<int> last_use_;  // per tensor: index of the last operator that reads it

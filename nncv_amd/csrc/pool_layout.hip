@@ -365,33 +365,74 @@ void launch_relayout(const void* src, int src_dt, Strides4 ss, void* dst, int ds
 // one 16-byte vector per pixel.  One thread per pixel: the C plane reads are coalesced across the
 // wave (consecutive pixels), the write is one whole vector per lane.
 // ---------------------------------------------------------------------------------------------
-template <typename T>
+template <typename T, int CP>
 __global__ __launch_bounds__(256) void image_to_nhwc_kernel(const T* __restrict__ src, T* __restrict__ dst, int C, long long HW,
                                                             long long total) {
-  constexpr int VN = Vec16<T>::n;
-  typedef typename Vec16<T>::type V;
+  typedef T V __attribute__((ext_vector_type(CP)));
   const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const long long n = idx / HW, p = idx - n * HW;
   V v;
 #pragma unroll
-  for (int c = 0; c < VN; ++c) v[c] = c < C ? src[(n * C + c) * HW + p] : (T)0.0f;
-  *reinterpret_cast<V*>(dst + idx * VN) = v;
+  for (int c = 0; c < CP; ++c) v[c] = c < C ? src[(n * C + c) * HW + p] : (T)0.0f;
+  *reinterpret_cast<V*>(dst + idx * CP) = v;
 }
 
 bool image_to_nhwc_applicable(int dt, int C) { return C >= 1 && C <= (dt == kF16 ? 8 : 4); }
 
-void launch_image_to_nhwc(const void* src, void* dst, int dt, int N, int C, int H, int W, hipStream_t s) {
-  NNCV_REQUIRE(image_to_nhwc_applicable(dt, C), "image_to_nhwc: too many channels for one vector");
+// Cp: channels per pixel in dst; one 16-byte vector (8 halves / 4 floats), or for fp16 half a
+// vector (4), which makes two horizontally adjacent pixels one vector (the pixel-pair form).
+void launch_image_to_nhwc(const void* src, void* dst, int dt, int N, int C, int H, int W, hipStream_t s, int Cp) {
+  const int vn = dt == kF16 ? 8 : 4;
+  if (Cp == 0) Cp = vn;
+  NNCV_REQUIRE(image_to_nhwc_applicable(dt, C) && C <= Cp && (Cp == vn || (dt == kF16 && Cp == 4)),
+               "image_to_nhwc: channel count not covered");
   const long long HW = (long long)H * W, total = HW * N;
   if (total == 0) return;
   const long long grid = (total + 255) / 256;
   NNCV_REQUIRE(grid < (1ll << 31), "image_to_nhwc: grid too large");
-  ProfScope prof("image_to_nhwc", 0.0, (double)dtype_size(dt) * total * (C + (dt == kF16 ? 8 : 4)), s);
-  if (dt == kF16)
-    hipLaunchKernelGGL((image_to_nhwc_kernel<half_t>), dim3((unsigned)grid), dim3(256), 0, s, (const half_t*)src, (half_t*)dst, C, HW, total);
+  ProfScope prof("image_to_nhwc", 0.0, (double)dtype_size(dt) * total * (C + Cp), s);
+  if (dt == kF16 && Cp == 8)
+    hipLaunchKernelGGL((image_to_nhwc_kernel<half_t, 8>), dim3((unsigned)grid), dim3(256), 0, s, (const half_t*)src, (half_t*)dst, C, HW, total);
+  else if (dt == kF16)
+    hipLaunchKernelGGL((image_to_nhwc_kernel<half_t, 4>), dim3((unsigned)grid), dim3(256), 0, s, (const half_t*)src, (half_t*)dst, C, HW, total);
   else
-    hipLaunchKernelGGL((image_to_nhwc_kernel<float>), dim3((unsigned)grid), dim3(256), 0, s, (const float*)src, (float*)dst, C, HW, total);
+    hipLaunchKernelGGL((image_to_nhwc_kernel<float, 4>), dim3((unsigned)grid), dim3(256), 0, s, (const float*)src, (float*)dst, C, HW, total);
+  NNCV_HIP_CHECK(hipGetLastError());
+}
+
+// Filters of a stride-2 convolution over an image stored as pixel pairs ([N][H][W/2][2 pixels x 4
+// channels], fp16): with ix = 2*ox - pad + s, the pair holding column ix is ox - pad2 + s2, so the
+// horizontal walk becomes stride 1 over S2 pairs and the K axis shrinks from K*K*8 (3 channels
+// padded to a whole vector) to K*S2*8.
+//   pad even: pad2 = pad/2,     S2 = ceil(K/2),     element (s2, p) is filter column 2*s2 + p
+//   pad odd : pad2 = (pad+1)/2, S2 = ceil((K+1)/2), element (s2, p) is filter column 2*s2 + p - 1
+// (zero outside 0..K-1 and for channels >= C).  dst: [Fp][K][S2][8], rows >= F zero.
+template <typename Ts>
+__global__ void weight_pairs_kernel(const Ts* __restrict__ w, half_t* __restrict__ dst, int F, int C, int K, int S2, int shift,
+                                    int total) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int e = i & 7, c = e & 3, pp = e >> 2;
+  int r = i >> 3;
+  const int s2 = r % S2; r /= S2;
+  const int kr = r % K;
+  const int f = r / K;
+  const int sc = 2 * s2 + pp - shift;
+  float v = 0.0f;
+  if (f < F && c < C && sc >= 0 && sc < K) v = (float)w[((f * C + c) * K + kr) * K + sc];
+  dst[i] = (half_t)v;
+}
+
+void launch_weight_pairs(const void* w, int w_dt, void* dst, int F, int Fp, int C, int K, int pad, hipStream_t s) {
+  NNCV_REQUIRE(C >= 1 && C <= 4 && K >= 1 && Fp >= F, "weight_pairs: shape not covered");
+  const int shift = pad & 1, S2 = (K + shift + 1) / 2;
+  const int total = Fp * K * S2 * 8;
+  const unsigned grid = (unsigned)((total + 255) / 256);
+  if (w_dt == kF16)
+    hipLaunchKernelGGL((weight_pairs_kernel<half_t>), dim3(grid), dim3(256), 0, s, (const half_t*)w, (half_t*)dst, F, C, K, S2, shift, total);
+  else
+    hipLaunchKernelGGL((weight_pairs_kernel<float>), dim3(grid), dim3(256), 0, s, (const float*)w, (half_t*)dst, F, C, K, S2, shift, total);
   NNCV_HIP_CHECK(hipGetLastError());
 }
 

@@ -177,7 +177,7 @@ def test_mobilenetv3_fp32(blob, shape):
     g.close()
 
 
-@pytest.mark.parametrize("shape", [(2, 3, 64, 64), (32, 3, 224, 224)])
+@pytest.mark.parametrize("shape", [(2, 3, 64, 64), (32, 3, 224, 224), (3, 3, 100, 77)])  # odd width: no pixel pairs
 def test_mobilenetv3_fp16(blob, shape):
     b16 = r16(blob)
     ops, n = abi.mobilenetv3_small_ops()

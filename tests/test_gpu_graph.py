@@ -209,6 +209,14 @@ def test_mobilenetv3_through_reference_abi(blob):
     assert got.shape == (1, 1000)
     assert max_rel(got, want) < FP32_MAX_REL
     assert np.array_equal(got.argmax(1), want.argmax(1))
+    # the half-precision symbol takes the same route (all three memrefs hold IEEE half bits)
+    b16 = blob.astype(np.float16)
+    x16 = x.astype(np.float16)
+    got16 = abi.forward(x16, b16)
+    want16 = oracle.mobilenetv3_forward(x16.astype(np.float32), tensors_of(b16.astype(np.float32)))
+    assert got16.dtype == np.float16 and got16.shape == (1, 1000)
+    assert rel_l2(got16.astype(np.float32), want16) < FP16_REL_L2
+    assert np.array_equal(got16.argmax(1), want16.argmax(1))
 
 
 # ---------------------------------------------------------------------------------------------

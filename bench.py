@@ -64,8 +64,8 @@ def main():
                     help="also run one 256 MiB device-to-device copy (a known-size kernel to scale HBM counters by)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        sys.stderr.write("bench.py: this build measures ONE GPU only (the path shards over the batch with no "
-                         "communication; see DESIGN.md). Run with --gpus 1.\n")
+        sys.stderr.write("bench.py: this build measures ONE GPU only (inference shards over the batch with no "
+                         "communication between GPUs, so a second GPU adds nothing to measure). Run with --gpus 1.\n")
         sys.exit(2)
 
     import numpy as np

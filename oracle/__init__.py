@@ -3,6 +3,26 @@
 TEST INFRASTRUCTURE ONLY.  May be imported by tests/, by __graft_entry__.smoke() and by the
 cpu_baseline leg of bench.py — never by nncv_amd/ (the product fails loudly without its HIP
 library instead of falling back to this).
+
+Besides the C functions (pinning status in the header of nncv_oracle.c) this module restates in
+numpy the operators of the reference's other network fixtures; what pins each:
+  depthwise_conv2d_nchw_chw, batchnorm_eps, hardswish, hardsigmoid, silu, sigmoid, maxpool_nchw,
+  upsample2x_nearest   torch CPU library routines in float64 (conv2d groups=C, batch_norm,
+                       hardswish, hardsigmoid, silu, max_pool2d, interpolate), closed forms at the knees
+                       and special values, a deliberately transposed filter that must fail
+                       (tests/test_oracle_mobilenetv3.py)
+  mobilenetv3_forward  a float64 torch composition of torchvision's mobilenet_v3_small.forward, block
+                       by block; the tensor table against the fixture's 52 convolution shapes, its 210
+                       constants and the published parameter count (same file)
+  yolo_detect          closed forms on non-square grids (cell centres / anchors at sigmoid 0.5, the
+                       extremes, one-hot channel placement) (tests/test_oracle_yolov5s.py)
+  run_graph            reproduces the C ResNet-18 oracle over resnet18_spec.graph_ops()
+                       (tests/test_oracle_resnet18.py), mobilenetv3_forward, and a float64 torch
+                       composition of YOLOv5s whose 60 convolution shapes and 13 concatenations are
+                       checked, in order, against tests/Nets/Yolov5s.mlir
+  preprocess_u8, top1_scan, hwp_*   tests/test_oracle_ops.py
+Parity unpinned, as for the C part: the exact fp32 summation order of the reference's compiled
+object (it cannot be built here); the restatements keep the fixtures' operation order.
 """
 import ctypes
 import os

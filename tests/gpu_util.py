@@ -94,7 +94,10 @@ class Conv:
             self.h = None
 
     def __del__(self):
-        self.close()
+        try:
+            self.close()
+        except Exception:  # interpreter shutdown: the modules this needs may be gone already
+            pass
 
 
 class Model:
@@ -130,7 +133,10 @@ class Model:
             self.h = None
 
     def __del__(self):
-        self.close()
+        try:
+            self.close()
+        except Exception:  # interpreter shutdown: the modules this needs may be gone already
+            pass
 
 
 class Graph:
@@ -154,4 +160,7 @@ class Graph:
             self.h = None
 
     def __del__(self):
-        self.close()
+        try:
+            self.close()
+        except Exception:  # interpreter shutdown: the modules this needs may be gone already
+            pass

@@ -146,3 +146,20 @@ def test_fp16_fused_stem_propagates_nan(blob):
     assert np.array_equal(np.isnan(tap), np.isnan(want_tap))
     ok = ~np.isnan(want_tap)
     assert rel_l2(tap[ok], want_tap[ok]) < 2e-3
+
+
+@pytest.mark.parametrize("shape", [(1, 3, 32, 32), (3, 3, 33, 47), (2, 3, 225, 223), (1, 3, 330, 70), (33, 3, 64, 64)])
+def test_unusual_sizes_both_types(blob, shape):
+    """Smallest image the network accepts, odd and very oblong images, a batch that is not a power of two:
+    the tile planners, the fused stem (even widths only) and its fallback all see shapes they were not tuned for."""
+    x = synth.uniform(3011, shape, 0.0, 1.0)
+    print("sizes", shape, flush=True)
+    m32 = Model(blob, abi.F32)
+    got, want = host(m32(dev(x))), oracle.resnet18_forward(x, blob)
+    assert max_rel(got, want) < FP32_MAX_REL and (got.argmax(1) == want.argmax(1)).all()
+    m32.close()
+    b16, x16 = synth.round_fp16(blob), synth.round_fp16(x)
+    m16 = Model(b16, abi.F16)
+    got16, want16 = host(m16(dev(x16, abi.F16))), oracle.resnet18_forward(x16, b16)
+    assert rel_l2(got16, want16) < FP16_REL_L2 and (got16.argmax(1) == want16.argmax(1)).all()
+    m16.close()

@@ -141,3 +141,30 @@ def test_producer_from_state_dict_and_dump(tmp_path):
     del bad["fc.weight"]
     with pytest.raises(KeyError):
         modelbin.resnet18_blob_from_state_dict(bad)
+
+
+@pytest.mark.parametrize("arch", ["mobilenetv3_small", "yolov5s"])
+def test_producer_for_the_other_networks(tmp_path, arch):
+    """The same producer over the MobileNetV3-small and YOLOv5s tables: round trip through a safetensors
+    state_dict, tensor count and element count of the file, strides filled in for YOLOv5s."""
+    from safetensors.numpy import save_file
+    spec = modelbin.spec_of(arch)
+    blob = synth.mobilenetv3_params() if arch == "mobilenetv3_small" else synth.yolov5s_params()
+    sd, off = {}, 0
+    for name, shape in spec.tensor_table():
+        k = spec.numel(shape)
+        sd[name] = blob[off:off + k].reshape(shape).copy()
+        off += k
+    if arch == "yolov5s":
+        del sd["model.24.stride"]  # ultralytics keeps it as an attribute
+    src, out = str(tmp_path / "m.safetensors"), str(tmp_path / "m.bin")
+    save_file(sd, src)
+    assert modelbin.main(["from-state-dict", src, out, "--arch", arch]) == 0
+    index, data = modelbin.read(out)
+    assert len(index) == spec.NUM_TENSORS and data.size == spec.NUM_ELEMENTS
+    assert [n for n, _, _ in index] == [n for n, _ in spec.tensor_table()]
+    assert np.array_equal(data, blob)
+    with pytest.raises(ValueError):
+        modelbin.blob_from_state_dict(sd, "resnet18" if False else "bogus")
+    with pytest.raises(KeyError):
+        modelbin.blob_from_state_dict(sd, "resnet18")

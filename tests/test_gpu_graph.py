@@ -355,3 +355,43 @@ def test_resnet18_as_an_operator_list(dt):
         assert rel_l2(got, want) < FP16_REL_L2 and rel_l2(got, hard) < FP16_REL_L2
     assert np.array_equal(got.argmax(1), want.argmax(1))
     g.close()
+
+
+@pytest.mark.parametrize("dt", [abi.F32, abi.F16])
+def test_nested_concatenation_views(dt):
+    """Concatenations whose inputs are themselves concatenations, max-pools, adds and activations: tensors living in
+    slices of slices, read at a pitch by 3x3 and 1x1 convolutions, against the dense evaluator."""
+    sizes, ops = [], []
+
+    def take(n):
+        off = sum(sizes)
+        sizes.append(n)
+        return off
+
+    def conv(i, o, cin, F, k, act=abi.ACT_RELU):
+        ops.append(abi.graph_op(abi.OP_CONV, [i], o, F=F, K=k, stride=1, pad=(k - 1) // 2, act=act, w=take(F * cin * k * k), bias=take(F)))
+
+    C = 16
+    conv(0, 1, 3, C, 3)                                                   # a
+    conv(0, 2, 3, 2 * C, 1, abi.ACT_HARDSWISH)                            # b
+    ops.append(abi.graph_op(abi.OP_CONCAT, [1, 2], 3, stride=0))          # c1 = [a, b]            (3C)
+    ops.append(abi.graph_op(abi.OP_MAXPOOL, [1], 4, K=3, stride=1, pad=1))  # e = pool(a): reads a inside c1 inside c2
+    ops.append(abi.graph_op(abi.OP_ACT, [2], 5, act=abi.ACT_SILU, stride=0))  # f = silu(b)
+    ops.append(abi.graph_op(abi.OP_ADD, [4, 1], 6, act=abi.ACT_NONE, stride=0))  # g = e + a
+    ops.append(abi.graph_op(abi.OP_CONCAT, [3, 6, 5], 7, stride=0))       # c2 = [c1, g, f]        (3C + C + 2C)
+    conv(3, 8, 3 * C, C, 3)                                               # 3x3 over the slice c1 of c2
+    conv(7, 9, 6 * C, 2 * C, 1, abi.ACT_NONE)                             # 1x1 over all of c2
+    ops.append(abi.graph_op(abi.OP_CONCAT, [8, 9], 10, stride=0))         # output [C + 2C]
+    blob = synth.normal(7800, (sum(sizes),), std=0.2)
+    x = synth.normal(7801, (2, 3, 11, 14))
+    if dt == abi.F16:
+        blob, x = r16(blob), r16(x)
+    g = Graph(ops, 3, blob, dt)
+    assert abi.graph_output_shape(g.h, 11, 14) == (3 * C, 11, 14)
+    got = host(g(dev(x, dt)))
+    want = oracle.run_graph(ops, x, blob, 3)
+    if dt == abi.F32:
+        assert max_rel(got, want) < FP32_MAX_REL
+    else:
+        assert rel_l2(got, want) < FP16_REL_L2
+    g.close()

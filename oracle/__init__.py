@@ -447,8 +447,17 @@ def hwp_lib():
             raise RuntimeError("%s is missing: run `make -C oracle`" % p)
         L = ctypes.CDLL(p)
         L.hwp_conv2d_nchw_fchw.argtypes = [_f32p, _f32p, _f32p] + [ctypes.c_int] * 9
+        L.hwp_set_num_threads.argtypes = [ctypes.c_int]
+        L.hwp_set_num_threads.restype = None
         _HWP = L
     return _HWP
+
+
+def hwp_threads(n=None):
+    """Threads the OpenMP x AVX2 restatement uses; n sets it for the calls that follow."""
+    if n is not None:
+        hwp_lib().hwp_set_num_threads(int(n))
+    return int(hwp_lib().hwp_num_threads())
 
 
 def hwp_conv2d(x, w, stride=1, pad=0):

@@ -15,6 +15,8 @@
 #include <vector>
 
 extern "C" int hwp_num_threads() { return omp_get_max_threads(); }
+// number of OpenMP threads of the following calls (the reference's `-num-threads`, default 4: main.cpp:231)
+extern "C" void hwp_set_num_threads(int n) { if (n > 0) omp_set_num_threads(n); }
 
 // y[N][F][OH][OW] = conv(x[N][C][H][W] with a zero halo of `pad`, w[F][C][R][S]), stride `stride`.
 extern "C" int hwp_conv2d_nchw_fchw(const float* x, const float* w, float* y, int N, int C, int H, int W, int F, int R, int S,

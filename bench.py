@@ -86,9 +86,14 @@ def main():
     blob32 = synth.resnet18_params()
     blob = blob32.astype(np.float16)
     x = synth.cfg4_input(N).astype(np.float16)
+    torch.zeros(1, device="cuda")  # HIP context up before the clock starts
+    torch.cuda.synchronize()
+    t_create = time.perf_counter()
     model = L.nncv_hip_resnet18_create(blob.ctypes.data, blob.size, abi.F16, algo)
     if not model:
         raise RuntimeError(L.nncv_hip_last_error().decode())
+    # one-time cost of a model: upload of the 23 MB blob, BN fold, filter re-lay (synchronous)
+    t_create = time.perf_counter() - t_create
     xd = torch.from_numpy(x).cuda()
     logits = torch.empty((N, 1000), dtype=torch.float32, device="cuda")
     stream = torch.cuda.current_stream().cuda_stream
@@ -188,6 +193,7 @@ def main():
         "frac_of_fp16_mfma_peak": round(flops_step / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 5),
         "conv3x3s1_gflop_per_step": round(conv3x3_flops / 1e9, 2),
         "batch1": None if sec1 is None else {"images_per_s": round(1.0 / sec1, 2), "ms_per_image": round(sec1 * 1e3, 4)},
+        "model_create_ms": round(t_create * 1e3, 2),
         "roofline": roofline,
         "kernels": kernels,
         "device": L.nncv_hip_device_arch().decode(),

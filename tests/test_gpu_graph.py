@@ -395,3 +395,28 @@ def test_nested_concatenation_views(dt):
     else:
         assert rel_l2(got, want) < FP16_REL_L2
     g.close()
+
+
+@pytest.mark.parametrize("dt", [abi.F32, abi.F16])
+def test_random_operator_lists(dt):
+    """40 seeded random graphs per element type against the evaluator (tests/graph_gen.py)."""
+    from graph_gen import random_case
+    f16 = dt == abi.F16
+    done = 0
+    for seed in range(5000, 5040):
+        case = random_case(seed, f16)
+        if case is None:
+            continue
+        ops, cin, blob, x = case
+        print("seed", seed, "kinds", [int(o.kind) for o in ops], "input", x.shape, flush=True)
+        g = Graph(ops, cin, blob, dt)
+        got = host(g(dev(x, dt)))
+        want = oracle.run_graph(ops, x, blob, cin)
+        g.close()
+        assert got.shape == want.shape and np.array_equal(np.isnan(got), np.isnan(want)), seed
+        fin = np.isfinite(want) & np.isfinite(got)
+        if fin.any():
+            err = rel_l2(got[fin], want[fin]) if f16 else max_rel(got[fin], want[fin])
+            assert err < (FP16_REL_L2 if f16 else FP32_MAX_REL), (seed, err)
+        done += 1
+    assert done >= 30

@@ -184,3 +184,23 @@ def test_mobilenetv3_oracle_batch_independent():
     full = oracle.mobilenetv3_forward(x, T)
     one = oracle.mobilenetv3_forward(x[1:2], T)
     assert np.array_equal(full[1:2], one)
+
+
+def test_random_graph_generator_is_deterministic_and_evaluable():
+    """The seeded generator behind the executor's random-graph GPU test: same seed, same graph; every graph it
+    emits is well formed for the evaluator."""
+    import sys
+    import os
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    from graph_gen import random_case
+    kinds = set()
+    for seed in range(5000, 5012):
+        a, b = random_case(seed, False), random_case(seed, False)
+        if a is None:
+            assert b is None
+            continue
+        assert [bytes(o) for o in a[0]] == [bytes(o) for o in b[0]] and np.array_equal(a[3], b[3])
+        y = oracle.run_graph(a[0], a[3], a[2], a[1])
+        assert y.shape[0] == a[3].shape[0]
+        kinds.update(int(o.kind) for o in a[0])
+    assert len(kinds) >= 6

@@ -120,3 +120,52 @@ def test_conv_time_helper_reports_a_plausible_duration():
     abi.check(abi.lib().nncv_hip_conv_time(layer.h, xd.data_ptr(), 2, 14, 14, None, out.data_ptr(), 20, None, ctypes.byref(avg)))
     assert np.array_equal(out.cpu().numpy(), want)
     assert 1.0 < avg.value < 1000.0
+
+
+@pytest.mark.parametrize("dt", [abi.F32, abi.F16])
+def test_random_layers(dt):
+    """50 seeded random layers per element type: channel counts from one vector to 256, filters not multiples of the
+    tiles, 1x1..7x7 windows, stride 1 / 2, with and without padding, BatchNorm, residual and any fused activation,
+    odd and oblong images -- whichever kernel the dispatcher picks must agree with the oracle."""
+    f16 = dt == abi.F16
+    vn = 8 if f16 else 4
+    done = 0
+    for seed in range(9000, 9050):
+        rng = np.random.default_rng(seed)
+        C = vn * int(rng.choice([1, 2, 3, 4, 8, 8, 16, 16, 32]))
+        F = 4 * int(rng.choice([1, 2, 3, 8, 16, 16, 18, 32, 50]))
+        if f16:
+            F = (F + 7) // 8 * 8
+        R = int(rng.choice([1, 3, 3, 3, 5, 7]))
+        stride = int(rng.choice([1, 1, 2]))
+        pad = int(rng.choice([0, (R - 1) // 2, (R - 1) // 2]))
+        H, W, N = int(rng.integers(R, 40)), int(rng.integers(R, 70)), int(rng.integers(1, 6))
+        OH, OW = (H + 2 * pad - R) // stride + 1, (W + 2 * pad - R) // stride + 1
+        act = int(rng.choice([abi.ACT_NONE, abi.ACT_RELU, abi.ACT_RELU, abi.ACT_HARDSWISH, abi.ACT_SILU]))
+        use_bn, use_res = rng.random() < 0.7, rng.random() < 0.4
+        wino = R == 3 and stride == 1 and act <= abi.ACT_RELU and rng.random() < 0.25
+        x = synth.normal(seed, (N, C, H, W))
+        w = synth.normal(seed + 1, (F, C, R, R), std=float(np.sqrt(2.0 / (C * R * R))))
+        bn = bn_params(seed + 2, F) if use_bn else None
+        res = synth.normal(seed + 6, (N, F, OH, OW)) if use_res else None
+        if f16:
+            x, w = synth.round_fp16(x), synth.round_fp16(w)
+            bn = tuple(synth.round_fp16(b) for b in bn) if bn else None
+            res = synth.round_fp16(res) if res is not None else None
+        print("seed", seed, (N, C, F, H, W, R, stride, pad), "act", act, "bn", use_bn, "res", use_res, "winograd", wino, flush=True)
+        y = oracle.conv2d_nchw_fchw(oracle.pad_nchw(x, pad) if pad else x, w, stride)
+        if bn:
+            y = oracle.batchnorm(y, *bn)
+        if res is not None:
+            y = (y + res).astype(np.float32)
+        want = oracle.ACTIVATIONS[act](y)
+        conv = Conv(dt, w, stride, pad, bn=bn, relu=act, algo=abi.ALGO_WINOGRAD if wino else abi.ALGO_IGEMM)
+        rd = dev(nhwc(res), dt) if res is not None else None
+        got = nchw(host(conv(dev(nhwc(x), dt), abi.NHWC, residual=rd)))
+        conv.close()
+        if f16:
+            assert rel_l2(got, want) < (3e-2 if wino else FP16_REL_L2), seed  # F(4,3) in half costs about 10x the rounding error
+        else:
+            assert max_rel(got, want) < FP32_MAX_REL, seed
+        done += 1
+    assert done == 50

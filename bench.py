@@ -48,8 +48,9 @@ DOMINANT_TRAFFIC = {  # profiles/resnet18_fp16_bs32_hbm_counters.txt, launches w
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    # defaults long enough for the clocks to settle: 50 steps after 10 (15 ms of work) read 7 % low
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--batch", type=int, default=0, help="0 = the workload's default (32; yolov5s 16)")
     ap.add_argument("--algo", default="auto", choices=["auto", "winograd", "igemm"])
     ap.add_argument("--no-cpu-baseline", action="store_true")

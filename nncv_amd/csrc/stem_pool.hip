@@ -5,7 +5,8 @@
 // The 112x112x64 convolution output (51 MB at batch 32, four times the pooled tensor) never
 // reaches memory.  A workgroup owns a 7x8 tile of pooled pixels, i.e. a 15x17 tile of convolution
 // pixels (255 of the 256 MFMA pixel slots of four 64x64 wave tiles) and a 35x40 tile of the image:
-//   1. the image tile is packed into LDS as rows of pixel PAIRS, [row][pair][2 px][c0 c1 c2 0],
+//   1. the image tile is packed into LDS as rows of pixel PAIRS, [row][pair][2 px][c0 c1 c2 0]
+//      (one 16-byte write per pair),
 //      so that one filter row (8 px x 4 ch = 32 halves) is 64 contiguous bytes starting at the
 //      pair of the output pixel (stride 2 = one pair per output pixel): every MFMA operand is one
 //      aligned 16-byte LDS read at a constant offset, with no im2col anywhere;
@@ -35,7 +36,6 @@ constexpr int kInBytes = kITH * kInPitch;
 constexpr int kConvPitch = 144;        // 64 halves + 16 pad
 constexpr int kConvBytes = 256 * kConvPitch;
 constexpr int kTabBytes = 2 * 64 * 4;  // scale, shift
-constexpr int kLoads = (kITH * kPairs * 3 + 255) / 256;  // 4-byte loads per thread and tile
 constexpr unsigned kOOBs = 0x7fff0000u;
 
 typedef unsigned short ushort2v __attribute__((ext_vector_type(2)));
@@ -64,18 +64,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int lrow = lane & 31, lchunk = lane >> 5;
   const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(a.in, a.in_bytes);
 
-  // ---- loader: element e = i*256 + tid of the [3][35][20] dwords of an image tile.  Only the LDS
-  //      offset of each element is kept; row, pair and channel are decoded from it per tile
-  //      (the registers are needed for the filters) ----
-  int l_off[kLoads];
+  // ---- loader: element e = i*256 + tid of the [35][20] pixel pairs of an image tile.  A thread
+  //      fetches the pair's three channel dwords (two adjacent pixels of one channel each; lanes
+  //      walk the pairs of a row, so every channel plane is read in contiguous runs) and deposits
+  //      the packed pair [c0 c1 c2 0 | c0 c1 c2 0] as ONE 16-byte LDS write: consecutive lanes hit
+  //      consecutive 16-byte bank groups, where per-channel 2-byte deposits collided ----
+  constexpr int kElems = (kITH * kPairs + 255) / 256;  // pairs per thread and tile
+  int l_off[kElems];
 #pragma unroll
-  for (int i = 0; i < kLoads; ++i) {
+  for (int i = 0; i < kElems; ++i) {
     const int e = i * 256 + tid;
-    const int c = e / (kITH * kPairs), rem = e - c * (kITH * kPairs);
-    const int row = rem / kPairs, pr = rem - row * kPairs;
-    l_off[i] = e < 3 * kITH * kPairs ? row * kInPitch + pr * 16 + c * 2 : -1;
+    const int row = e / kPairs, pr = e - row * kPairs;
+    l_off[i] = e < kITH * kPairs ? row * kInPitch + pr * 16 : -1;
   }
-  unsigned pix[kLoads];
+  unsigned pix[kElems][3];
   auto tile_origin = [&](int t, int& n, int& py0, int& px0) {
     n = t / (a.tiles_x * a.tiles_y);
     const int r = t - n * (a.tiles_x * a.tiles_y);
@@ -89,20 +91,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int iy0 = 4 * py0 - 5, ix0 = 4 * px0 - 6;  // conv row 2*py0-1 -> image row 2*(2*py0-1)-3; column one further left (pairs)
     const int base = (n * 3 * a.H + iy0) * a.W + ix0;
 #pragma unroll
-    for (int i = 0; i < kLoads; ++i) {
-      const int row = l_off[i] / kInPitch, in_row = l_off[i] - row * kInPitch;
-      const int col = (in_row >> 4) * 2, c = (in_row & 15) >> 1;
+    for (int i = 0; i < kElems; ++i) {
+      const int row = l_off[i] / kInPitch, col = ((l_off[i] - row * kInPitch) >> 4) * 2;
       const bool ok = (l_off[i] >= 0) & ((unsigned)(iy0 + row) < (unsigned)a.H) & ((unsigned)(ix0 + col) < (unsigned)a.W);
-      const int g_rel = (c * a.H + row) * a.W + col;
-      pix[i] = __builtin_amdgcn_raw_buffer_load_b32(rs_in, ok ? (unsigned)(base + g_rel) * 2u : kOOBs, 0, 0);
+#pragma unroll
+      for (int c = 0; c < 3; ++c) {
+        const int g_rel = (c * a.H + row) * a.W + col;
+        pix[i][c] = __builtin_amdgcn_raw_buffer_load_b32(rs_in, ok ? (unsigned)(base + g_rel) * 2u : kOOBs, 0, 0);
+      }
     }
   };
   auto deposit = [&]() {
 #pragma unroll
-    for (int i = 0; i < kLoads; ++i)
+    for (int i = 0; i < kElems; ++i)
       if (l_off[i] >= 0) {
-        *reinterpret_cast<unsigned short*>(in_t + l_off[i]) = (unsigned short)(pix[i] & 0xffffu);
-        *reinterpret_cast<unsigned short*>(in_t + l_off[i] + 8) = (unsigned short)(pix[i] >> 16);
+        u32x4 v;
+        v[0] = (pix[i][0] & 0xffffu) | (pix[i][1] << 16);
+        v[1] = pix[i][2] & 0xffffu;
+        v[2] = (pix[i][0] >> 16) | (pix[i][1] & 0xffff0000u);
+        v[3] = pix[i][2] >> 16;
+        *reinterpret_cast<u32x4*>(in_t + l_off[i]) = v;
       }
   };
 

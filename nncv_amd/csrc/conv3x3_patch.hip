@@ -39,7 +39,7 @@ constexpr int kXcdsP = 8;
 template <int WS> struct PatchCap;     // patch capacity in pixels for 64*WS slots
 template <> struct PatchCap<4> { static constexpr int pix = 384; };
 template <> struct PatchCap<2> { static constexpr int pix = 256; };
-template <> struct PatchCap<1> { static constexpr int pix = 128; };
+template <> struct PatchCap<1> { static constexpr int pix = 192; };
 }  // namespace
 
 struct PatchArgs {
@@ -331,7 +331,8 @@ static bool plan_patch(int N, int H, int W, int F, int slabs, int* WS, int* TN, 
     if (!plan_tile(N, H, W, 64 * ws, cap, cover, &tn, &th, &lg)) continue;
     const long long tiles = (long long)((N + tn - 1) / tn) * ((H + th - 1) / th);
     const double used = (double)N * H * W / ((double)tiles * 64 * ws);
-    const double fill = tiles * fb >= 256 ? 1.0 : (double)(tiles * fb) / 256.0;
+    // "every CU busy" saturates at 7/8 of them: past that a narrower tile only adds halo re-reads
+    const double fill = tiles * fb >= 224 ? 1.0 : (double)(tiles * fb) / 224.0;
     const double score = used * fill;
     if (score > best * 1.05) {
       best = score; *WS = ws; *TN = tn; *TH = th; *rw_log = lg;

@@ -122,6 +122,7 @@ struct IgemmArgs {
   // all F filters.  aux_f0 = 0: none; otherwise a multiple of 128.  Fast kernel only.
   int aux_f0, aux_tap, aux_relu, aux_ldo;
   void* aux_out;
+  const void* aux_wt_frag;  // the auxiliary 1x1 filters alone, fragment-major (launch_weight_frag1x1), or null
 };
 // in_dt: element type of in/wt (kF32 | kF16); out_dt: element type of out/residual.
 // Dispatches to the fast kernel (igemm_fast.hip) when C is a multiple of one K step and the
@@ -187,6 +188,8 @@ void launch_weight_frsc(const void* w, int w_dt, void* dst, int dst_dt, int F, i
                         hipStream_t s);
 // 3x3 weights FCHW -> fragment-major order of conv3x3_patch.hip, F padded to a multiple of 64
 void launch_weight_frag3x3(const void* w, int w_dt, void* dst, int dst_dt, int F, int C, hipStream_t s);
+// 1x1 weights [F][C] in the same order with one tap per slab (IgemmArgs::aux_wt_frag)
+void launch_weight_frag1x1(const void* w, int w_dt, void* dst, int dst_dt, int F, int C, hipStream_t s);
 // stem weights [64,3,7,7] -> [64][7][4][8] over (pixel-pair, channel4); pair sp / pixel p holds
 // filter column 2*sp + p - col_shift (zero outside 0..6)
 void launch_stem_weight(const void* w, int w_dt, void* dst, int dst_dt, int F, int col_shift, hipStream_t s);

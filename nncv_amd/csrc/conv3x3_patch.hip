@@ -53,26 +53,135 @@ struct PatchArgs {
   int TN, TH;            // tile: TN images x TH rows x W columns
   int tiles_y;           // ceil(H / TH)
   int tiles;             // ceil(N / TN) * tiles_y
-  int rw_log;            // patch loader: 2^rw_log >= W + 2 pixels per loader row
+  int rw_log;            // patch loader: 2^rw_log >= patch columns per loader row
+  int OH, OW;            // output size (stride 2; stride 1: H, W)
   int xcd_by_filter;     // XCD <- filter block instead of XCD <- tile range
   unsigned in_bytes, wf_bytes;
-  float inv_ph, inv_thw, inv_w;  // 1/(TH+2), 1/(TH*W), 1/W
+  float inv_ph, inv_thw, inv_w;  // 1/(patch rows per image), 1/(TH*OW), 1/OW
+  // Stride 2 only: filter blocks >= aux_fb0 (in units of the workgroup's 32*NI filters) belong to a
+  // 1x1 stride-2 convolution over the same input (the shortcut of a down-sampling block), with its
+  // own output tensor [N][OH][OW][aux_F], scale/shift and ReLU flag.  aux_F = 0: none.
+  const void* aux_wf;    // fragment-major, one tap per slab (launch_weight_frag1x1)
+  void* aux_out;
+  const float* aux_scale;
+  const float* aux_shift;
+  int aux_F, aux_relu, aux_fb0;
+  unsigned aux_wf_bytes;
 };
 
-template <int WS, int WK>
+template <int WS, int WK, int ST = 1>
 struct PatchCfg {
   static constexpr int NW = WS * WK, NT = 64 * NW;
-  static constexpr int cover = WS == 4 ? 384 : WS == 2 ? 256 : 192;  // padded patch pixels the loader can walk
+  // padded patch pixels the loader can walk.  A stride-2 tile reads four input pixels per output
+  // pixel: its patch is about four times the size for the same number of slots.
+  static constexpr int cover = ST == 2 ? (WS == 2 ? 576 : 288) : WS == 4 ? 384 : WS == 2 ? 256 : 192;
   static constexpr int passes = cover / (NT / 8);  // loader passes per thread: NT/8 pixels each
   static constexpr int nset = WK == 4 ? 9 : 3;  // weight register sets = taps in flight; divides 9
-  static constexpr int cap = PatchCap<WS>::pix;
+  static constexpr int cap = ST == 2 ? (WS == 2 ? 522 : 288) : PatchCap<WS>::pix;
+  // instances whose tap loop keeps no patch prefetch registers alive: single-slab layers only
+  static constexpr bool reload = ST == 2 ? WS == 1 : WS != 4;
   static constexpr int patch_bytes = cap * kPitch;
   static constexpr int load_bytes = patch_bytes + NT * 16;  // + one dump slot per thread
   static constexpr int tile_bytes = WS * WK * kTileBytes;  // one copy per K group
   static constexpr int smem = load_bytes > tile_bytes ? load_bytes : tile_bytes;
 };
 
+// The auxiliary 1x1 stride-2 filter blocks of a stride-2 launch.  Their pixels are the centre taps
+// of the tile's slots, so the "patch" is just those 64*WS pixels, one LDS cell per slot, and the
+// walk is one tap per slab.  A ninth of the work of a 3x3 block: these workgroups have the highest
+// block indices and fill the tail of the launch.
 template <typename T, typename OutT, int WS, int WK, int NI>
+__device__ __forceinline__ void patch_aux_1x1(const PatchArgs& a, unsigned char* smem, int n0, int y0, int fb, int tid) {
+  constexpr int NT = 64 * WS * WK, ES = sizeof(T), KPG = 4 / WK;
+  constexpr int AP = 64 * WS / (NT / 8);  // loader passes: NT/8 pixels each
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ws = wave % WS, wk = wave / WS;
+  const int lrow = lane & 31, lchunk = lane >> 5;
+  const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(a.in, a.in_bytes);
+  const __amdgpu_buffer_rsrc_t rs_wf = make_rsrc(a.aux_wf, a.aux_wf_bytes);
+  const int nslab = a.C * ES / 128;
+  const int nslots = a.TN * a.TH * a.OW;
+  auto decode = [&](int sl, int* n, int* oy, int* ox) {
+    int nl = 0, rem = sl;
+    if (a.TN > 1) nl = fast_div(sl, a.TH * a.OW, a.inv_thw, &rem);
+    const int ty = fast_div(rem, a.OW, a.inv_w, ox);
+    *n = n0 + nl;
+    *oy = y0 + ty;
+    return (sl < nslots) & (*n < a.N) & (*oy < a.OH);
+  };
+  const int p8 = tid >> 3, pc = (tid & 7) * 16;
+  const unsigned ces = (unsigned)(a.C * ES);
+  unsigned aoff[AP];
+#pragma unroll
+  for (int i = 0; i < AP; ++i) {
+    int n, oy, ox;
+    const bool ok = decode(i * (NT / 8) + p8, &n, &oy, &ox);
+    aoff[i] = ok ? __umul24((unsigned)((n * a.H + 2 * oy) * a.W + 2 * ox), ces) + pc : kOOBp;
+  }
+  u32x4 aregs[AP];
+  auto aload = [&](int slab) {
+#pragma unroll
+    for (int i = 0; i < AP; ++i) aregs[i] = __builtin_amdgcn_raw_buffer_load_b128(rs_in, aoff[i] + slab * 128, 0, 0);
+  };
+  auto astore = [&]() {
+#pragma unroll
+    for (int i = 0; i < AP; ++i) *reinterpret_cast<u32x4*>(smem + (i * (NT / 8) + p8) * kPitch + pc) = aregs[i];
+  };
+  aload(0);
+  const int wbase = NI == 2 ? (fb * nslab * 8 + wk * KPG * 2) * 1024 : ((fb >> 1) * nslab * 8 + wk * KPG * 2 + (fb & 1)) * 1024;
+  const unsigned wlane = lane * 16;
+  EpiScale<OutT> ess;
+  ess.load(lane, fb * (32 * NI), a.aux_F, a.aux_scale, a.aux_shift);
+  int cell[2], obase[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int sl = ws * 64 + j * 32 + lrow;
+    int n, oy, ox;
+    const bool ok = decode(sl, &n, &oy, &ox);
+    cell[j] = sl * kPitch + (lchunk + 2 * wk * KPG) * 16;
+    obase[j] = ok ? ((n * a.OH + oy) * a.OW + ox) * a.aux_F : -1;
+  }
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+  astore();
+  __syncthreads();
+  for (int slab = 0; slab < nslab; ++slab) {
+    const bool more = slab + 1 < nslab;
+    if (more) aload(slab + 1);
+    u32x4 w[KPG][NI];
+#pragma unroll
+    for (int k = 0; k < KPG; ++k)
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+        w[k][i] = __builtin_amdgcn_raw_buffer_load_b128(rs_wf, wlane, wbase + slab * 8192 + (k * 2 + i) * 1024, 0);
+#pragma unroll
+    for (int k = 0; k < KPG; ++k) {
+      u32x4 p[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) p[j] = *reinterpret_cast<const u32x4*>(smem + cell[j] + k * 32);
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) Mma<T>::run(w[k][i], p[j], acc[i][j]);
+    }
+    if (more) {
+      __syncthreads();  // every wave is done with this slab's pixels
+      astore();
+      __syncthreads();
+    }
+  }
+  __syncthreads();  // LDS becomes the output tiles
+  tile_reduce_store<OutT, WK, NI, false>(acc, smem + ws * WK * kTileBytes, wk, lane, obase, fb * (32 * NI), a.aux_F, ess,
+                                         static_cast<const OutT*>(nullptr), static_cast<OutT*>(a.aux_out), a.aux_relu);
+}
+
+template <typename T, typename OutT, int WS, int WK, int NI, int ST>
 __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv3x3_patch_kernel(
     // the values the patch addressing needs first, as plain leading arguments: those are preloaded
     // into SGPRs at wave launch, the struct behind them is fetched by a scalar load as usual
@@ -81,7 +190,8 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   PatchArgs a = a_rest;
   a.in = in_p; a.tiles = tiles_p; a.tiles_y = tiles_y_p; a.TN = tn_p; a.TH = th_p; a.N = n_p; a.H = h_p; a.W = w_p; a.C = c_p;
   a.rw_log = rw_log_p; a.xcd_by_filter = xcd_by_filter_p; a.in_bytes = in_bytes_p;
-  typedef PatchCfg<WS, WK> Cfg;
+  typedef PatchCfg<WS, WK, ST> Cfg;
+  static_assert(ST == 1 || ST == 2, "stride 1 or 2");
   constexpr int NT = Cfg::NT, kPasses = Cfg::passes, NSET = Cfg::nset;
   constexpr int kDepth = WK == 1 ? 3 : 4;  // pixel-operand ring: LDS reads run kDepth-1 steps ahead of their MFMAs
   constexpr int ES = sizeof(T);
@@ -109,7 +219,18 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   if (tile >= a.tiles) return;
   const int f0blk = fblk * (32 * NI);
   const int n0 = (tile / a.tiles_y) * a.TN, y0 = (tile % a.tiles_y) * a.TH;
-  const int PH = a.TH + 2, PW = a.W + 2;
+  if constexpr (ST == 2) {
+    if (fblk >= a.aux_fb0) {  // uniform for the workgroup
+      patch_aux_1x1<T, OutT, WS, WK, NI>(a, smem, n0, y0, fblk - a.aux_fb0, threadIdx.x);
+      return;
+    }
+  }
+  // Stride 2: output row ty / column tx of the tile reads patch rows 2ty..2ty+2 and columns
+  // 2tx..2tx+2.  The patch keeps the even and the odd columns of a row apart (PWh pixels each), so
+  // that the slots of consecutive output pixels stay consecutive in LDS for every tap.
+  const int OH = ST == 1 ? a.H : a.OH, OW = ST == 1 ? a.W : a.OW;
+  const int PH = ST == 1 ? a.TH + 2 : 2 * a.TH + 1, PW = ST == 1 ? a.W + 2 : 2 * OW + 1;
+  const int PWh = OW + 1;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in an SGPR
@@ -119,7 +240,7 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   const __amdgpu_buffer_rsrc_t rs_wf = make_rsrc(a.wf, a.wf_bytes);
   // The widest tile keeps no patch prefetch registers alive in the tap loop: the host only picks it
   // for single-slab layers, and its loop never reloads the patch.
-  constexpr bool kReload = WS != 4;
+  constexpr bool kReload = Cfg::reload;
   const int nslab = a.C * ES / 128;
   const int niter = nslab * 9;  // one iteration = one tap of one slab
 
@@ -131,12 +252,12 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   const unsigned ces = (unsigned)(a.C * ES);
   unsigned pvoff[kPasses];
   if (a.TN == 1) {  // one image per tile: patch row r is image row y0 - 1 + r
-    const int rowbase = (n0 * a.H + y0 - 1) * a.W - 1;
+    const int rowbase = (n0 * a.H + ST * y0 - 1) * a.W - 1;
 #pragma unroll
     for (int i = 0; i < kPasses; ++i) {
       const int q = i * (NT / 8) + p8;
       const int r = q >> a.rw_log, px = q & rwm;
-      const bool ok = (r < prows) & ((unsigned)(y0 - 1 + r) < (unsigned)a.H) & ((unsigned)(px - 1) < (unsigned)a.W);
+      const bool ok = (r < prows) & ((unsigned)(ST * y0 - 1 + r) < (unsigned)a.H) & ((unsigned)(px - 1) < (unsigned)a.W);
       const unsigned off = __umul24((unsigned)(rowbase + (int)__umul24(r, a.W) + px), ces) + pc;
       pvoff[i] = ok ? off : kOOBp;
     }
@@ -147,7 +268,7 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
       const int r = q >> a.rw_log, px = q & rwm;
       int py;
       const int n = n0 + fast_div(r, PH, a.inv_ph, &py);
-      const int iy = y0 + py - 1;
+      const int iy = ST * y0 + py - 1;
       const bool ok = (r < prows) & (n < a.N) & ((unsigned)iy < (unsigned)a.H) & ((unsigned)(px - 1) < (unsigned)a.W);
       const unsigned off = __umul24((unsigned)((n * a.H + iy) * a.W + px - 1), ces) + pc;
       pvoff[i] = ok ? off : kOOBp;
@@ -165,7 +286,8 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
     for (int i = 0; i < kPasses; ++i) {
       const int q = i * (NT / 8) + p8;
       const int r = q >> a.rw_log, px = q & rwm;
-      const int dst = (int)__umul24(__umul24(r, PW) + px, kPitch) + pc;
+      const int cell = ST == 1 ? __umul24(r, PW) + px : __umul24(2 * r + (px & 1), PWh) + (px >> 1);
+      const int dst = (int)__umul24(cell, kPitch) + pc;
       *reinterpret_cast<u32x4*>(patch + (((px < PW) & (r < prows)) ? dst : dump)) = pregs[i];
     }
   };
@@ -194,19 +316,20 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   ess.load(lane, f0blk, a.F, a.scale, a.shift);
 
   // ---- this lane's two pixel slots ----
-  const int nslots = a.TN * a.TH * a.W;
+  const int nslots = a.TN * a.TH * OW;
   int sbase[2];  // byte offset of the slot's tap-(0,0) pixel in the patch
   int obase[2];  // element offset of the slot's output pixel row, or -1
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int sl = ws * 64 + j * 32 + lrow;
     int nl = 0, rem = sl, tx;
-    if (a.TN > 1) nl = fast_div(sl, a.TH * a.W, a.inv_thw, &rem);
-    const int ty = fast_div(rem, a.W, a.inv_w, &tx);
-    const bool ok = (sl < nslots) & ((n0 + nl) < a.N) & ((y0 + ty) < a.H);
+    if (a.TN > 1) nl = fast_div(sl, a.TH * OW, a.inv_thw, &rem);
+    const int ty = fast_div(rem, OW, a.inv_w, &tx);
+    const bool ok = (sl < nslots) & ((n0 + nl) < a.N) & ((y0 + ty) < OH);
     // slots beyond the tile read pixel 0 of the patch; their results are never stored
-    sbase[j] = (ok ? (int)__umul24(__umul24(__umul24(nl, PH) + ty, PW) + tx, kPitch) : 0) + (lchunk + 2 * wk * KPG) * 16;
-    obase[j] = ok ? (((n0 + nl) * a.H + y0 + ty) * a.W + tx) * a.F : -1;
+    const int cell = ST == 1 ? __umul24(__umul24(nl, PH) + ty, PW) + tx : __umul24(__umul24(nl, PH) + 2 * ty, 2 * PWh) + tx;
+    sbase[j] = (ok ? (int)__umul24(cell, kPitch) : 0) + (lchunk + 2 * wk * KPG) * 16;
+    obase[j] = ok ? (((n0 + nl) * OH + y0 + ty) * OW + tx) * a.F : -1;
   }
 
   floatx16 acc[2][2];  // [filter half][pixel half]; with NI = 1 only acc[0] is used
@@ -228,14 +351,18 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
 #pragma unroll
   for (int r = 0; r < 3; ++r)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) rowbase[r][j] = sbase[j] + r * PW * kPitch;
+    for (int j = 0; j < 2; ++j) rowbase[r][j] = sbase[j] + r * (ST == 1 ? PW : 2 * PWh) * kPitch;
+  const int odd_col = PWh * kPitch;  // stride 2: from an even column to the odd one right of it
   u32x4 ring[kDepth][2];
   auto ldp = [&](auto step_c) {
     constexpr int st = decltype(step_c)::value;
     constexpr int t = st / KPG, k = st % KPG;
 #pragma unroll
     for (int j = 0; j < 2; ++j)
-      ring[st % kDepth][j] = *reinterpret_cast<const u32x4*>(patch + rowbase[t / 3][j] + (t % 3) * kPitch + k * 32);
+      if constexpr (ST == 1)
+        ring[st % kDepth][j] = *reinterpret_cast<const u32x4*>(patch + rowbase[t / 3][j] + (t % 3) * kPitch + k * 32);
+      else  // filter columns 0, 1, 2 = even column, the odd one after it, the next even one
+        ring[st % kDepth][j] = *reinterpret_cast<const u32x4*>(patch + rowbase[t / 3][j] + (t % 3 == 1 ? odd_col : 0) + (t % 3 == 2 ? kPitch : 0) + k * 32);
   };
   auto prime = [&](auto self, auto d_c) -> void {  // the first kDepth-1 steps of a fresh patch
     constexpr int d = decltype(d_c)::value;
@@ -285,15 +412,18 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
                               static_cast<const OutT*>(a.residual), static_cast<OutT*>(a.out), a.relu);
 }
 
-// Tile choice for 64*ws slots: TN images x TH rows x W columns, patch of at most `cap` pixels,
-// which the loader walks as rows of 2^rw_log pixels, `cover` padded pixels at most.
-static bool plan_tile(int N, int H, int W, int slots, int cap, int cover, int* TN, int* TH, int* rw_log) {
-  const int PW = W + 2;
+// Tile choice for 64*ws slots: TN images x TH output rows x W output columns, patch of at most
+// `cap` pixels, which the loader walks as rows of 2^rw_log pixels, `cover` padded pixels at most.
+// H, W: output size (= input size at stride 1).
+static bool plan_tile(int st, int N, int H, int W, int slots, int cap, int cover, int* TN, int* TH, int* rw_log) {
+  const int PW = st == 1 ? W + 2 : 2 * W + 1;       // patch columns the loader walks
+  const int cells = st == 1 ? W + 2 : 2 * (W + 1);  // LDS cells per patch row
+  auto prow = [&](int th) { return st == 1 ? th + 2 : 2 * th + 1; };
   int lg = 0;
   while ((1 << lg) < PW) ++lg;
   if ((1 << lg) > 64 || W > slots) return false;
   const int max_rows = cover >> lg;  // patch rows the loader can cover
-  auto fits = [&](int tn, int th) { return tn * th * W <= slots && tn * (th + 2) * PW <= cap && tn * (th + 2) <= max_rows; };
+  auto fits = [&](int tn, int th) { return tn * th * W <= slots && tn * prow(th) * cells <= cap && tn * prow(th) <= max_rows; };
   int thmax = 0;
   for (int th = 1; th <= H; ++th)
     if (fits(1, th)) thmax = th;
@@ -313,7 +443,7 @@ static bool plan_tile(int N, int H, int W, int slots, int cap, int cover, int* T
 }
 
 // Picks the wave arrangement: the largest pixel tile that still gives (about) every CU a workgroup.
-static bool plan_patch(int N, int H, int W, int F, int slabs, int* WS, int* TN, int* TH, int* rw_log) {
+static bool plan_patch(int st, int N, int H, int W, int F, int slabs, int* WS, int* TN, int* TH, int* rw_log) {
   static const int force = [] {
     const char* e = getenv("NNCV_HIP_PATCH_WS");
     return e ? atoi(e) : 0;
@@ -324,11 +454,18 @@ static bool plan_patch(int N, int H, int W, int F, int slabs, int* WS, int* TN, 
   double best = 0.0;
   for (int ws : {4, 2, 1}) {
     if (force && ws != force) continue;
-    if (ws == 4 && slabs != 1) continue;  // the WS=4 instance handles one slab
-    const int cap = ws == 4 ? PatchCap<4>::pix : ws == 2 ? PatchCap<2>::pix : PatchCap<1>::pix;
+    int cap, cover;
+    if (st == 1) {
+      if (ws == 4 && slabs != 1) continue;  // the WS=4 instance handles one slab
+      cap = ws == 4 ? PatchCfg<4, 1>::cap : ws == 2 ? PatchCfg<2, 2>::cap : PatchCfg<1, 4>::cap;
+      cover = ws == 4 ? PatchCfg<4, 1>::cover : ws == 2 ? PatchCfg<2, 2>::cover : PatchCfg<1, 4>::cover;
+    } else {
+      if (ws == 4 || (ws == 2 && slabs != 1)) continue;  // stride 2: the WS=2 instance handles one slab
+      cap = ws == 2 ? PatchCfg<2, 2, 2>::cap : PatchCfg<1, 4, 2>::cap;
+      cover = ws == 2 ? PatchCfg<2, 2, 2>::cover : PatchCfg<1, 4, 2>::cover;
+    }
     int tn, th, lg;
-    const int cover = ws == 4 ? PatchCfg<4, 1>::cover : ws == 2 ? PatchCfg<2, 2>::cover : PatchCfg<1, 4>::cover;
-    if (!plan_tile(N, H, W, 64 * ws, cap, cover, &tn, &th, &lg)) continue;
+    if (!plan_tile(st, N, H, W, 64 * ws, cap, cover, &tn, &th, &lg)) continue;
     const long long tiles = (long long)((N + tn - 1) / tn) * ((H + th - 1) / th);
     const double used = (double)N * H * W / ((double)tiles * 64 * ws);
     // "every CU busy" saturates at 7/8 of them: past that a narrower tile only adds halo re-reads
@@ -345,54 +482,82 @@ bool conv3x3_patch_applicable(const IgemmArgs& a, int in_dt) {
   static const bool off = getenv("NNCV_HIP_NO_PATCH") != nullptr;
   const int slab = in_dt == kF16 ? 64 : 32;
   int ws, tn, th, lg;
-  return !off && a.aux_f0 == 0 && a.relu <= kActRelu && a.wt_frag && a.R == 3 && a.S == 3 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 1 && a.pad_w == 1 &&
-         a.batch == 1 && a.pix_stride == 0 && a.C % slab == 0 && a.F % 8 == 0 && a.ldo == a.F &&
-         (long long)a.N * a.H * a.W * a.F < (1ll << 31) && (long long)a.N * a.H * a.W < (1 << 24) && a.in_bytes < kOOBp &&
-         (long long)((a.F + 63) / 64) * 64 * 9 * a.C * (long long)dtype_size(in_dt) < (1ll << 31) &&
-         plan_patch(a.N, a.H, a.W, a.F, a.C / slab, &ws, &tn, &th, &lg);
+  static const bool off2 = getenv("NNCV_HIP_NO_PATCH_S2") != nullptr;
+  const int st = a.stride_h;
+  // auxiliary filters: the centre tap of a stride-2 launch, given fragment-major
+  const int fmain = a.aux_f0 ? a.aux_f0 : a.F, faux = a.F - fmain;
+  const bool aux_ok = a.aux_f0 == 0 || (st == 2 && a.aux_tap == 4 && a.aux_wt_frag && a.aux_out && a.aux_relu <= kActRelu && a.aux_f0 % 64 == 0 &&
+                                        faux % 8 == 0 && a.aux_ldo == faux);
+  return !off && aux_ok && a.relu <= kActRelu && a.wt_frag && a.R == 3 && a.S == 3 && (st == 1 || (st == 2 && !off2)) && a.stride_w == st &&
+         a.pad_h == 1 && a.pad_w == 1 && a.OH == (a.H - 1) / st + 1 && a.OW == (a.W - 1) / st + 1 &&
+         a.batch == 1 && a.pix_stride == 0 && a.C % slab == 0 && fmain % 8 == 0 && a.ldo == fmain &&
+         (long long)a.N * a.OH * a.OW * std::max(fmain, faux) < (1ll << 31) && (long long)a.N * a.H * a.W < (1 << 24) && a.in_bytes < kOOBp &&
+         (long long)((std::max(fmain, faux) + 63) / 64) * 64 * 9 * a.C * (long long)dtype_size(in_dt) < (1ll << 31) &&
+         plan_patch(st, a.N, a.OH, a.OW, fmain, a.C / slab, &ws, &tn, &th, &lg);
 }
 
-template <typename T, typename OutT, int WS, int WK, int NI>
+template <typename T, typename OutT, int WS, int WK, int NI, int ST = 1>
 static void launch_patch_cfg(const PatchArgs& a, double flops, double bytes, const char* tag, hipStream_t s) {
-  typedef PatchCfg<WS, WK> Cfg;
-  auto kern = conv3x3_patch_kernel<T, OutT, WS, WK, NI>;
+  typedef PatchCfg<WS, WK, ST> Cfg;
+  auto kern = conv3x3_patch_kernel<T, OutT, WS, WK, NI, ST>;
   static const bool attr = [&] {
     NNCV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::smem));
     return true;
   }();
   (void)attr;
   ProfScope prof(tag, flops, bytes, s);
-  dim3 grid((a.tiles + kXcdsP - 1) / kXcdsP * kXcdsP, (a.F + 32 * NI - 1) / (32 * NI));
-  hipLaunchKernelGGL(kern, grid, dim3(Cfg::NT), Cfg::smem, s, a.in, a.tiles, a.tiles_y, a.TN, a.TH, a.N, a.H, a.W, a.C, a.rw_log,
-                     a.xcd_by_filter, a.in_bytes, a);
+  const int fblocks = (a.F + 32 * NI - 1) / (32 * NI) + (a.aux_F + 32 * NI - 1) / (32 * NI);
+  PatchArgs b = a;
+  b.aux_fb0 = (a.F + 32 * NI - 1) / (32 * NI);
+  if (b.xcd_by_filter && fblocks % kXcdsP != 0) b.xcd_by_filter = 0;
+  dim3 grid((a.tiles + kXcdsP - 1) / kXcdsP * kXcdsP, fblocks);
+  hipLaunchKernelGGL(kern, grid, dim3(Cfg::NT), Cfg::smem, s, b.in, b.tiles, b.tiles_y, b.TN, b.TH, b.N, b.H, b.W, b.C, b.rw_log,
+                     b.xcd_by_filter, b.in_bytes, b);
 }
 
 void launch_conv3x3_patch(const IgemmArgs& g, int in_dt, int out_dt, hipStream_t s) {
   PatchArgs a{};
   a.in = g.in; a.wf = g.wt_frag; a.out = g.out; a.scale = g.scale; a.shift = g.shift; a.residual = g.residual;
-  a.N = g.N; a.H = g.H; a.W = g.W; a.C = g.C; a.F = g.F; a.relu = g.relu;
+  a.N = g.N; a.H = g.H; a.W = g.W; a.C = g.C; a.F = g.aux_f0 ? g.aux_f0 : g.F; a.relu = g.relu;
+  if (g.aux_f0) {
+    a.aux_F = g.F - g.aux_f0; a.aux_wf = g.aux_wt_frag; a.aux_out = g.aux_out; a.aux_relu = g.aux_relu;
+    a.aux_scale = g.scale ? g.scale + g.aux_f0 : nullptr; a.aux_shift = g.shift ? g.shift + g.aux_f0 : nullptr;
+    a.aux_wf_bytes = (unsigned)((size_t)((a.aux_F + 63) / 64) * 64 * g.C * dtype_size(in_dt));
+  }
   int ws = 0;
-  NNCV_REQUIRE(plan_patch(a.N, a.H, a.W, a.F, a.C * (int)dtype_size(in_dt) / 128, &ws, &a.TN, &a.TH, &a.rw_log),
+  const int st = g.stride_h;
+  a.OH = g.OH; a.OW = g.OW;
+  NNCV_REQUIRE(plan_patch(st, a.N, a.OH, a.OW, a.F, a.C * (int)dtype_size(in_dt) / 128, &ws, &a.TN, &a.TH, &a.rw_log),
                "conv3x3_patch: no tile fits");
-  a.tiles_y = (a.H + a.TH - 1) / a.TH;
+  a.tiles_y = (a.OH + a.TH - 1) / a.TH;
   a.tiles = ((a.N + a.TN - 1) / a.TN) * a.tiles_y;
   a.in_bytes = g.in_bytes;
   a.wf_bytes = (unsigned)((size_t)((a.F + 63) / 64) * 64 * 9 * a.C * dtype_size(in_dt));
   a.xcd_by_filter = ((a.F + 63) / 64) % kXcdsP == 0 && a.wf_bytes > (2u << 20);
-  a.inv_ph = 1.0f / (a.TH + 2);
-  a.inv_thw = 1.0f / (a.TH * a.W);
-  a.inv_w = 1.0f / a.W;
-  const double P = (double)a.N * a.H * a.W;
-  const double flops = 2.0 * P * a.F * 9.0 * a.C;
+  a.inv_ph = 1.0f / (st == 1 ? a.TH + 2 : 2 * a.TH + 1);
+  a.inv_thw = 1.0f / (a.TH * a.OW);
+  a.inv_w = 1.0f / a.OW;
+  const double P = (double)a.N * a.OH * a.OW;
+  const double flops = 2.0 * P * a.C * (9.0 * a.F + a.aux_F);
   const double es = dtype_size(in_dt), os = dtype_size(out_dt);
-  const double bytes = es * (P * a.C + 9.0 * a.C * a.F) + os * P * a.F * (a.residual ? 2 : 1);
+  const double bytes = es * ((double)a.N * a.H * a.W * a.C + a.C * (9.0 * a.F + a.aux_F)) + os * P * (a.F * (a.residual ? 2 : 1) + a.aux_F);
   const bool h = in_dt == kF16 && out_dt == kF16, f = in_dt == kF32 && out_dt == kF32;
   NNCV_REQUIRE(h || f, "conv3x3_patch: unsupported dtype combination");
   // Few workgroups (small batch on the deep layers: each streams its filter block's weights through
   // one CU's 64 B/clk vector-memory path): split the 64-filter blocks in two and use twice the CUs.
-  const bool halves = ws == 1 && (long long)a.tiles * ((a.F + 63) / 64) < 128 && a.F % 64 == 0;
+  const bool halves = ws == 1 && (long long)a.tiles * ((a.F + 63) / 64 + (a.aux_F + 63) / 64) < 128 && a.F % 64 == 0;
   if (halves) a.xcd_by_filter = (a.F / 32) % kXcdsP == 0 && a.wf_bytes > (2u << 20);
-  if (h) {
+  if (st == 2) {
+    if (h) {
+      if (ws == 2) launch_patch_cfg<half_t, half_t, 2, 2, 2, 2>(a, flops, bytes, "conv3x3s2_patch<f16,2,2>", s);
+      else if (halves) launch_patch_cfg<half_t, half_t, 1, 4, 1, 2>(a, flops, bytes, "conv3x3s2_patch<f16,1,4,half>", s);
+      else launch_patch_cfg<half_t, half_t, 1, 4, 2, 2>(a, flops, bytes, "conv3x3s2_patch<f16,1,4>", s);
+    } else {
+      if (ws == 2) launch_patch_cfg<float, float, 2, 2, 2, 2>(a, flops, bytes, "conv3x3s2_patch<f32,2,2>", s);
+      else if (halves) launch_patch_cfg<float, float, 1, 4, 1, 2>(a, flops, bytes, "conv3x3s2_patch<f32,1,4,half>", s);
+      else launch_patch_cfg<float, float, 1, 4, 2, 2>(a, flops, bytes, "conv3x3s2_patch<f32,1,4>", s);
+    }
+  } else if (h) {
     if (ws == 4) launch_patch_cfg<half_t, half_t, 4, 1, 2>(a, flops, bytes, "conv3x3_patch<f16,4,1>", s);
     else if (ws == 2) launch_patch_cfg<half_t, half_t, 2, 2, 2>(a, flops, bytes, "conv3x3_patch<f16,2,2>", s);
     else if (halves) launch_patch_cfg<half_t, half_t, 1, 4, 1>(a, flops, bytes, "conv3x3_patch<f16,1,4,half>", s);

@@ -119,7 +119,7 @@ Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, lon
         nd.wt.reset((size_t)Cstored * op.K * op.K * C * es);
         NNCV_HIP_CHECK(hipMemsetAsync(nd.wt.get(), 0, nd.wt.bytes(), s));
         launch_weight_frsc(w, dt, nd.wt.get(), dt, op.F, Cl, op.K, op.K, C, s);
-        if (op.K == 3 && op.stride == 1 && op.pad == 1 && Cl == C && Cstored == op.F && C % (128 / (int)es) == 0) {
+        if (op.K == 3 && (op.stride == 1 || op.stride == 2) && op.pad == 1 && Cl == C && Cstored == op.F && C % (128 / (int)es) == 0) {
           nd.wfrag.reset((size_t)((op.F + 63) / 64) * 64 * 9 * C * es);
           launch_weight_frag3x3(w, dt, nd.wfrag.get(), dt, op.F, C, s);
         }

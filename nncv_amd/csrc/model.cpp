@@ -49,7 +49,7 @@ ConvLayer::ConvLayer(const Desc& d, const void* w, const void* gamma, const void
     wt_.reset((size_t)Fp * d.R * d.S * Cp * es);
     NNCV_HIP_CHECK(hipMemsetAsync(wt_.get(), 0, wt_.bytes(), s));
     launch_weight_frsc(w, d.dt, wt_.get(), d.dt, d.F, d.C, d.R, d.S, Cp, s);
-    if (d.R == 3 && d.S == 3 && d.stride == 1 && d.pad == 1 && d.C % (128 / (int)es) == 0) {
+    if (d.R == 3 && d.S == 3 && (d.stride == 1 || d.stride == 2) && d.pad == 1 && d.C % (128 / (int)es) == 0) {
       wfrag_.reset((size_t)((d.F + 63) / 64) * 64 * 9 * d.C * es);
       launch_weight_frag3x3(w, d.dt, wfrag_.get(), d.dt, d.F, d.C, s);
     }
@@ -141,6 +141,10 @@ bool ConvLayer::fuse_shortcut(const ConvLayer& ds, hipStream_t s) {
   NNCV_HIP_CHECK(hipMemcpyAsync(shift_cat_.get(), shift_.get(), (size_t)d_.F * 4, hipMemcpyDeviceToDevice, s));
   NNCV_HIP_CHECK(hipMemcpyAsync(scale_cat_.as<float>() + d_.F, ds.scale_.get(), (size_t)q.F * 4, hipMemcpyDeviceToDevice, s));
   NNCV_HIP_CHECK(hipMemcpyAsync(shift_cat_.as<float>() + d_.F, ds.shift_.get(), (size_t)q.F * 4, hipMemcpyDeviceToDevice, s));
+  if (wfrag_.get() && d_.C % (128 / (int)es) == 0) {
+    aux_wfrag_.reset((size_t)((q.F + 63) / 64) * 64 * d_.C * es);
+    launch_weight_frag1x1(ds.wt_.get(), d_.dt, aux_wfrag_.get(), d_.dt, q.F, d_.C, s);  // [F][1][1][C] rows
+  }
   aux_F_ = q.F;
   aux_relu_ = q.relu;
   aux_flops_per_pixel_ = 2.0 * q.F * q.C;
@@ -152,7 +156,7 @@ void ConvLayer::forward_with_shortcut(const void* in, int N, int H, int W, void*
   const int OH = out_h(H), OW = out_w(W);
   NNCV_REQUIRE(N > 0 && OH > 0 && OW > 0, "conv: empty tensor");
   IgemmArgs a{};
-  a.in = in; a.wt = wt_cat_.get(); a.out = out;
+  a.in = in; a.wt = wt_cat_.get(); a.wt_frag = wfrag_.get(); a.aux_wt_frag = aux_wfrag_.get(); a.out = out;
   a.scale = scale_cat_.as<float>(); a.shift = shift_cat_.as<float>();
   a.N = N; a.H = H; a.W = W; a.C = d_.C; a.F = d_.F + aux_F_; a.R = 3; a.S = 3; a.OH = OH; a.OW = OW;
   a.stride_h = a.stride_w = d_.stride; a.pad_h = a.pad_w = 1;

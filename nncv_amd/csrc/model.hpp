@@ -57,6 +57,7 @@ class ConvLayer {
   int algo_;
   DeviceBuffer wt_, wfrag_, U_, scale_, shift_, wt_shift_;
   DeviceBuffer wt_cat_, scale_cat_, shift_cat_;  // this layer's filters followed by the fused shortcut's
+  DeviceBuffer aux_wfrag_;  // the fused shortcut's filters alone, fragment-major (stride-2 patch kernel)
   int aux_F_ = 0;
   int aux_relu_ = 0;
   double aux_flops_per_pixel_ = 0.0;

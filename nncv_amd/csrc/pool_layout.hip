@@ -515,40 +515,49 @@ void launch_weight_frsc(const void* w, int w_dt, void* dst, int dst_dt, int F, i
 // contiguous kilobyte, lane L holding filter fb*64 + i*32 + L%32, channels
 // sl*SLAB + (L/32 + 2*kk)*CE .. +CE-1 (CE = elements per 16 bytes, SLAB = 8*CE):
 //   offset(fb, sl, tap, kk, i, L) = (((((fb*nslab + sl)*9 + tap)*4 + kk)*2 + i)*64 + L) * 16 bytes.
-// Filters beyond F are zero.
-template <typename Ts, typename Td>
+// Filters beyond F are zero.  TAPS = 1 is the same order for 1x1 filters (the shortcut convolution
+// that rides on a stride-2 3x3 one).
+template <typename Ts, typename Td, int TAPS>
 __global__ void weight_frag3x3_kernel(const Ts* __restrict__ w, Td* __restrict__ dst, int F, int C, int Fp) {
   constexpr int CE = 16 / (int)sizeof(Td);
   const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;  // one 16-byte chunk each
   const int nslab = C / (8 * CE);
-  const long long total = (long long)(Fp / 64) * nslab * 9 * 4 * 2 * 64;
+  const long long total = (long long)(Fp / 64) * nslab * TAPS * 4 * 2 * 64;
   if (idx >= total) return;
   const int L = (int)(idx & 63);
   long long r = idx >> 6;
   const int i = (int)(r & 1); r >>= 1;
   const int kk = (int)(r & 3); r >>= 2;
-  const int tap = (int)(r % 9); r /= 9;
+  const int tap = (int)(r % TAPS); r /= TAPS;
   const int sl = (int)(r % nslab);
   const int fb = (int)(r / nslab);
   const int f = fb * 64 + i * 32 + (L & 31);
   const int c0 = sl * 8 * CE + ((L >> 5) + 2 * kk) * CE;
   Td* d = dst + idx * CE;
 #pragma unroll
-  for (int e = 0; e < CE; ++e) d[e] = f < F ? (Td)(float)w[((long long)f * C + c0 + e) * 9 + tap] : (Td)0.0f;
+  for (int e = 0; e < CE; ++e) d[e] = f < F ? (Td)(float)w[((long long)f * C + c0 + e) * TAPS + tap] : (Td)0.0f;
+}
+
+template <int TAPS>
+static void launch_weight_frag(const void* w, int w_dt, void* dst, int dst_dt, int F, int C, hipStream_t s) {
+  const int ce = dst_dt == kF16 ? 8 : 4;
+  NNCV_REQUIRE(C % (8 * ce) == 0, "weight_frag: C must be a multiple of the 128-byte slab");
+  const int Fp = (F + 63) / 64 * 64;
+  const long long total = (long long)(Fp / 64) * (C / (8 * ce)) * TAPS * 4 * 2 * 64;
+  const unsigned grid = (unsigned)((total + 255) / 256);
+#define LAUNCH(TS, TD) hipLaunchKernelGGL((weight_frag3x3_kernel<TS, TD, TAPS>), dim3(grid), dim3(256), 0, s, (const TS*)w, (TD*)dst, F, C, Fp)
+  if (w_dt == kF32 && dst_dt == kF32) LAUNCH(float, float);
+  else if (w_dt == kF16 && dst_dt == kF16) LAUNCH(half_t, half_t);
+  else fail("weight_frag: unsupported dtype combination");
+#undef LAUNCH
+  NNCV_HIP_CHECK(hipGetLastError());
 }
 
 void launch_weight_frag3x3(const void* w, int w_dt, void* dst, int dst_dt, int F, int C, hipStream_t s) {
-  const int ce = dst_dt == kF16 ? 8 : 4;
-  NNCV_REQUIRE(C % (8 * ce) == 0, "weight_frag3x3: C must be a multiple of the 128-byte slab");
-  const int Fp = (F + 63) / 64 * 64;
-  const long long total = (long long)(Fp / 64) * (C / (8 * ce)) * 9 * 4 * 2 * 64;
-  const unsigned grid = (unsigned)((total + 255) / 256);
-#define LAUNCH(TS, TD) hipLaunchKernelGGL((weight_frag3x3_kernel<TS, TD>), dim3(grid), dim3(256), 0, s, (const TS*)w, (TD*)dst, F, C, Fp)
-  if (w_dt == kF32 && dst_dt == kF32) LAUNCH(float, float);
-  else if (w_dt == kF16 && dst_dt == kF16) LAUNCH(half_t, half_t);
-  else fail("weight_frag3x3: unsupported dtype combination");
-#undef LAUNCH
-  NNCV_HIP_CHECK(hipGetLastError());
+  launch_weight_frag<9>(w, w_dt, dst, dst_dt, F, C, s);
+}
+void launch_weight_frag1x1(const void* w, int w_dt, void* dst, int dst_dt, int F, int C, hipStream_t s) {
+  launch_weight_frag<1>(w, w_dt, dst, dst_dt, F, C, s);
 }
 
 template <typename Ts, typename Td>

@@ -40,6 +40,14 @@ CASES = [  # N, C, F, H, W, R, stride, pad
     (2, 64, 72, 30, 62, 3, 1, 1),     # widest row the patch loader takes, F not a multiple of 64
     (1, 64, 64, 20, 64, 3, 1, 1),     # too wide for the patch kernel: falls back to implicit GEMM
     (2, 64, 64, 23, 17, 3, 1, 1),     # ragged: H not a multiple of the row tile
+    # stride 2 through the LDS-patch kernel (even / odd columns of the patch kept apart)
+    (4, 64, 128, 56, 56, 3, 2, 1),    # 2x2 waves, TH=4, one slab
+    (3, 128, 256, 28, 28, 3, 2, 1),   # 1x4 waves, TH=4, two slabs, last row tile short
+    (5, 256, 64, 14, 14, 3, 2, 1),    # whole image per tile, four slabs
+    (9, 64, 72, 7, 7, 3, 2, 1),       # several images per tile, F not a multiple of 64
+    (2, 64, 64, 23, 17, 3, 2, 1),     # odd sizes: the last input row / column is read by the last output only
+    (2, 128, 64, 30, 62, 3, 2, 1),    # widest row the loader takes at stride 2
+    (1, 64, 64, 9, 63, 3, 2, 1),      # one column too wide: implicit GEMM
 ]
 
 

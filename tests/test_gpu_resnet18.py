@@ -77,6 +77,32 @@ def test_fp16_small_batch(blob):
             assert (got.argmax(1) == want.argmax(1)).all()
 
 
+def test_fp16_layers_take_the_kernels_they_are_measured_on(blob):
+    """The launch tags of one fp16 forward pass at 224x224: every 3x3 layer goes through the LDS-patch kernel, the three
+    stride-2 ones through its stride-2 form with the 1x1 shortcut riding along (no separate shortcut launch), so a silent
+    fall-back to the implicit-GEMM kernels shows up here and not only in the timings."""
+    hb = synth.round_fp16(blob)
+    x = synth.round_fp16(synth.uniform(4003, (4, 3, 224, 224), 0.0, 1.0))
+    m = Model(hb, abi.F16, abi.ALGO_IGEMM)
+    xd = dev(x, abi.F16)
+    m(xd)
+    torch.cuda.synchronize()
+    abi.profile_enable(True)
+    try:
+        abi.profile_report()
+        got = host(m(xd))
+        rep = abi.profile_report()
+    finally:
+        abi.profile_enable(False)
+    print({k: v["launches"] for k, v in rep.items()}, flush=True)
+    count = lambda prefix: sum(v["launches"] for k, v in rep.items() if k.startswith(prefix))
+    assert count("conv3x3_patch") == 13
+    assert count("conv3x3s2_patch") == 3
+    assert count("igemm") == 0
+    assert sum(v["launches"] for v in rep.values()) == 18  # + stem/pool and pool/FC
+    assert rel_l2(got, oracle.resnet18_forward(x, hb)) < FP16_REL_L2
+
+
 def test_graph_replay_matches_eager_every_time(blob):
     """The device entry point captures the forward into a HIP graph on the second call with the
     same buffers and replays it afterwards: every replay must equal the eager result, also when the

@@ -123,6 +123,13 @@ struct IgemmArgs {
   int aux_f0, aux_tap, aux_relu, aux_ldo;
   void* aux_out;
   const void* aux_wt_frag;  // the auxiliary 1x1 filters alone, fragment-major (launch_weight_frag1x1), or null
+  // Optional scratch for splitting K over workgroups (conv3x3_patch.hip, small fp32 launches only):
+  // splitk_ws holds fp32 partial tiles for the duration of the launch; splitk_counters are
+  // splitk_counters_n ints that are zero before the launch and zero again after it.  Null: no split.
+  void* splitk_ws;
+  size_t splitk_ws_bytes;
+  int* splitk_counters;
+  int splitk_counters_n;
 };
 // in_dt: element type of in/wt (kF32 | kF16); out_dt: element type of out/residual.
 // Dispatches to the fast kernel (igemm_fast.hip) when C is a multiple of one K step and the

@@ -67,7 +67,145 @@ struct PatchArgs {
   const float* aux_shift;
   int aux_F, aux_relu, aux_fb0;
   unsigned aux_wf_bytes;
+  // K split over workgroups (the SK instances): grid.z = ksplit workgroups share an output tile, each
+  // walks `spk` channel slabs; their fp32 partial tiles meet in `partial` and the last one to
+  // arrive (ticket from `counters`) sums them in slab order and runs the epilogue.
+  float* partial;  // [tiles * filter blocks][ksplit][64][64]
+  int* counters;   // [tiles * filter blocks], zero between launches
+  int ksplit, spk;
 };
+
+// tile_reduce_store (mfma_tile.hpp) for one of `ksplit` workgroups that hold partial sums of the same
+// output tile.  Every workgroup reduces its K groups through LDS as usual, writes the fp32 result to
+// its slot of `partial`, and takes a ticket; the workgroup that draws the last ticket adds the ksplit
+// tiles in index order (so the sum does not depend on which one was last), applies the epilogue and
+// stores.  It also returns the counter to zero for the next launch.  No workgroup ever waits.
+constexpr int kMaxSplit = 16;  // workgroups per output tile at most
+
+template <typename OutT, int NG, int NI>
+__device__ __forceinline__ void tile_reduce_store_splitk(const floatx16 (&acc)[2][2], unsigned char* tile, int g, int lane, int tid,
+                                                         const int (&rowoff)[2], int f0, int F, const EpiScale<OutT>& ss,
+                                                         const OutT* res, OutT* out, int relu, float* partial, int* counter, int z,
+                                                         int ksplit) {
+  const int lrow = lane & 31, lchunk = lane >> 5;
+  constexpr int FPL = EpiScale<OutT>::FPL, LPR = EpiScale<OutT>::LPR;
+  constexpr int RPI = 64 / LPR, NIT = 64 / NG / RPI;
+  static_assert(NIT >= 1, "too many K groups for this output type");
+  typedef OutT VO __attribute__((ext_vector_type(FPL)));
+  const int fc = (lane % LPR) * FPL;
+  const bool lane_on = fc < 32 * NI;
+  const bool fok = f0 + fc < F && lane_on;
+  int o[NIT];
+  VO rv[NIT];
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int row = g * (64 / NG) + it * RPI + lane / LPR;
+    const int o0 = __shfl(rowoff[0], row & 31), o1 = __shfl(rowoff[1], row & 31);
+    o[it] = (row & 32) ? o1 : o0;
+    if (!fok) o[it] = -1;
+  }
+  if (res) {
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const long long off = o[it] >= 0 ? (long long)o[it] + f0 + fc : 0;
+      rv[it] = *reinterpret_cast<const VO*>(res + off);
+    }
+  }
+  unsigned char* mine = tile + g * kTileBytes;
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        floatx4* p = reinterpret_cast<floatx4*>(mine + (j * 32 + lrow) * kTilePitch + (i * 32 + 8 * q + 4 * lchunk) * 4);
+        *p = floatx4{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+      }
+  __syncthreads();
+  floatx4 v[NIT][FPL / 4];
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int row = g * (64 / NG) + it * RPI + lane / LPR;
+#pragma unroll
+    for (int q = 0; q < FPL / 4; ++q) {
+      floatx4 sum = *reinterpret_cast<const floatx4*>(tile + row * kTilePitch + fc * 4 + q * 16);
+#pragma unroll
+      for (int k = 1; k < NG; ++k) sum += *reinterpret_cast<const floatx4*>(tile + k * kTileBytes + row * kTilePitch + fc * 4 + q * 16);
+      v[it][q] = sum;
+    }
+  }
+  // This workgroup's partial tile -> global memory, then the ticket.  The tile is written and later
+  // read with device-scope relaxed atomics (8 bytes each): those are performed where all XCDs see
+  // them, so no cache write-back / invalidate fence is needed (a device-scope fence writes the whole
+  // L2 back and costs tens of microseconds here); waiting for the stores to be acknowledged orders
+  // them before the ticket.
+  typedef unsigned long long u64;
+  typedef u64 u64x2 __attribute__((ext_vector_type(2)));
+  if (lane_on) {
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int row = g * (64 / NG) + it * RPI + lane / LPR;
+#pragma unroll
+      for (int q = 0; q < FPL / 4; ++q) {
+        u64* p = reinterpret_cast<u64*>(partial + ((size_t)z * 64 + row) * 64 + fc + 4 * q);
+        const u64x2 bits = __builtin_bit_cast(u64x2, v[it][q]);
+        __hip_atomic_store(p, bits[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(p + 1, bits[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_waitcnt(0);  // every store of this wave has been acknowledged
+  __syncthreads();                // ... and of every wave (all are done reading the LDS tiles, too)
+  int* flag = reinterpret_cast<int*>(tile);
+  if (tid == 0) *flag = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  if (*flag != ksplit - 1) return;  // uniform for the workgroup
+  if (tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  // all kMaxSplit loads of a row segment are requested before the first addition (a chain of
+  // dependent round trips to memory would cost more than the split saves); slots past ksplit read
+  // tile 0 and are not added
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int row = g * (64 / NG) + it * RPI + lane / LPR;
+#pragma unroll
+    for (int q = 0; q < FPL / 4; ++q) {
+      u64x2 bits[kMaxSplit];
+#pragma unroll
+      for (int zz = 0; zz < kMaxSplit; ++zz) {
+        u64* p = reinterpret_cast<u64*>(partial + ((size_t)(zz < ksplit ? zz : 0) * 64 + row) * 64 + (lane_on ? fc : 0) + 4 * q);
+        bits[zz][0] = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        bits[zz][1] = __hip_atomic_load(p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      floatx4 sum = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int zz = 0; zz < kMaxSplit; ++zz)
+        if (zz < ksplit) sum += __builtin_bit_cast(floatx4, bits[zz]);
+      v[it][q] = sum;
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    float y[FPL];
+#pragma unroll
+    for (int q = 0; q < FPL / 4; ++q)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) y[4 * q + e] = v[it][q][e] * ss.sc[4 * q + e] + ss.sh[4 * q + e];
+    if (res) {
+#pragma unroll
+      for (int e = 0; e < FPL; ++e) y[e] += (float)rv[it][e];
+    }
+    if (relu == kActRelu) {
+#pragma unroll
+      for (int e = 0; e < FPL; ++e) y[e] = relu_ugt(y[e]);
+    }
+    VO ov;
+#pragma unroll
+    for (int e = 0; e < FPL; ++e) ov[e] = (OutT)y[e];
+    if (o[it] >= 0) *reinterpret_cast<VO*>(out + (long long)o[it] + f0 + fc) = ov;
+  }
+}
 
 template <int WS, int WK, int ST = 1>
 struct PatchCfg {
@@ -181,7 +319,7 @@ __device__ __forceinline__ void patch_aux_1x1(const PatchArgs& a, unsigned char*
                                          static_cast<const OutT*>(nullptr), static_cast<OutT*>(a.aux_out), a.aux_relu);
 }
 
-template <typename T, typename OutT, int WS, int WK, int NI, int ST>
+template <typename T, typename OutT, int WS, int WK, int NI, int ST, bool SK>
 __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv3x3_patch_kernel(
     // the values the patch addressing needs first, as plain leading arguments: those are preloaded
     // into SGPRs at wave launch, the struct behind them is fetched by a scalar load as usual
@@ -221,6 +359,7 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   const int n0 = (tile / a.tiles_y) * a.TN, y0 = (tile % a.tiles_y) * a.TH;
   if constexpr (ST == 2) {
     if (fblk >= a.aux_fb0) {  // uniform for the workgroup
+      if (SK && blockIdx.z != 0) return;  // the auxiliary blocks do not split K
       patch_aux_1x1<T, OutT, WS, WK, NI>(a, smem, n0, y0, fblk - a.aux_fb0, threadIdx.x);
       return;
     }
@@ -241,7 +380,9 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   // The widest tile keeps no patch prefetch registers alive in the tap loop: the host only picks it
   // for single-slab layers, and its loop never reloads the patch.
   constexpr bool kReload = Cfg::reload;
-  const int nslab = a.C * ES / 128;
+  const int nslab_all = a.C * ES / 128;
+  const int slab0 = SK ? (int)blockIdx.z * a.spk : 0;  // this workgroup's first slab and how many it walks
+  const int nslab = SK ? min(a.spk, nslab_all - slab0) : nslab_all;
   const int niter = nslab * 9;  // one iteration = one tap of one slab
 
   // ---- patch loader: 8 threads per pixel, NT/8 pixels per pass; the patch is walked as rows of
@@ -277,7 +418,7 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   u32x4 pregs[kPasses];
   auto pload = [&](int slab) {
 #pragma unroll
-    for (int i = 0; i < kPasses; ++i) pregs[i] = __builtin_amdgcn_raw_buffer_load_b128(rs_in, pvoff[i] + slab * 128, 0, 0);
+    for (int i = 0; i < kPasses; ++i) pregs[i] = __builtin_amdgcn_raw_buffer_load_b128(rs_in, pvoff[i] + (slab0 + slab) * 128, 0, 0);
   };
   // Lanes whose pass lies outside the patch store to a private dump slot behind it: no divergence.
   const int dump = Cfg::patch_bytes + tid * 16;
@@ -297,7 +438,9 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   // ---- weights: iteration `it`, sub-step k of this K group, filter half i of 64-filter block fb is
   //      the kilobyte at (fb*niter*8 + it*8 + k*2 + i)*1024; NSET register sets hold iterations
   //      it .. it+NSET-1.  An NI = 1 workgroup owns one half of a 64-filter block. ----
-  const int wbase = NI == 2 ? (fblk * niter * 8 + wk * KPG * 2) * 1024 : ((fblk >> 1) * niter * 8 + wk * KPG * 2 + (fblk & 1)) * 1024;
+  const int niter_all = nslab_all * 9;
+  const int wbase = (NI == 2 ? (fblk * niter_all * 8 + wk * KPG * 2) * 1024 : ((fblk >> 1) * niter_all * 8 + wk * KPG * 2 + (fblk & 1)) * 1024) +
+                    slab0 * 9 * 8192;
   const unsigned wlane = lane * 16;
   auto wfrag = [](int k, int i) { return (k * 2 + i) * 1024; };  // byte offset of fragment (k, i) inside an iteration
   auto wload = [&](u32x4(&r)[NF], int it) {
@@ -408,8 +551,15 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   }
   __syncthreads();  // every wave is done with the patch: LDS becomes the output tiles
 
-  tile_reduce_store<OutT, WK, NI, false>(acc, smem + ws * WK * kTileBytes, wk, lane, obase, f0blk, a.F, ess,
-                              static_cast<const OutT*>(a.residual), static_cast<OutT*>(a.out), a.relu);
+  if constexpr (SK) {
+    const int wg = tile * gridDim.y + fblk;
+    tile_reduce_store_splitk<OutT, WK, NI>(acc, smem + ws * WK * kTileBytes, wk, lane, tid, obase, f0blk, a.F, ess,
+                                           static_cast<const OutT*>(a.residual), static_cast<OutT*>(a.out), a.relu,
+                                           a.partial + (size_t)wg * a.ksplit * 4096, a.counters + wg, blockIdx.z, a.ksplit);
+  } else {
+    tile_reduce_store<OutT, WK, NI, false>(acc, smem + ws * WK * kTileBytes, wk, lane, obase, f0blk, a.F, ess,
+                                           static_cast<const OutT*>(a.residual), static_cast<OutT*>(a.out), a.relu);
+  }
 }
 
 // Tile choice for 64*ws slots: TN images x TH output rows x W output columns, patch of at most
@@ -496,10 +646,10 @@ bool conv3x3_patch_applicable(const IgemmArgs& a, int in_dt) {
          plan_patch(st, a.N, a.OH, a.OW, fmain, a.C / slab, &ws, &tn, &th, &lg);
 }
 
-template <typename T, typename OutT, int WS, int WK, int NI, int ST = 1>
+template <typename T, typename OutT, int WS, int WK, int NI, int ST = 1, bool SK = false>
 static void launch_patch_cfg(const PatchArgs& a, double flops, double bytes, const char* tag, hipStream_t s) {
   typedef PatchCfg<WS, WK, ST> Cfg;
-  auto kern = conv3x3_patch_kernel<T, OutT, WS, WK, NI, ST>;
+  auto kern = conv3x3_patch_kernel<T, OutT, WS, WK, NI, ST, SK>;
   static const bool attr = [&] {
     NNCV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::smem));
     return true;
@@ -510,7 +660,7 @@ static void launch_patch_cfg(const PatchArgs& a, double flops, double bytes, con
   PatchArgs b = a;
   b.aux_fb0 = (a.F + 32 * NI - 1) / (32 * NI);
   if (b.xcd_by_filter && fblocks % kXcdsP != 0) b.xcd_by_filter = 0;
-  dim3 grid((a.tiles + kXcdsP - 1) / kXcdsP * kXcdsP, fblocks);
+  dim3 grid((a.tiles + kXcdsP - 1) / kXcdsP * kXcdsP, fblocks, SK ? a.ksplit : 1);
   hipLaunchKernelGGL(kern, grid, dim3(Cfg::NT), Cfg::smem, s, b.in, b.tiles, b.tiles_y, b.TN, b.TH, b.N, b.H, b.W, b.C, b.rw_log,
                      b.xcd_by_filter, b.in_bytes, b);
 }
@@ -547,6 +697,29 @@ void launch_conv3x3_patch(const IgemmArgs& g, int in_dt, int out_dt, hipStream_t
   // one CU's 64 B/clk vector-memory path): split the 64-filter blocks in two and use twice the CUs.
   const bool halves = ws == 1 && (long long)a.tiles * ((a.F + 63) / 64 + (a.aux_F + 63) / 64) < 128 && a.F % 64 == 0;
   if (halves) a.xcd_by_filter = (a.F / 32) % kXcdsP == 0 && a.wf_bytes > (2u << 20);
+  // fp32, still few workgroups, several slabs: split K over up to 256 / workgroups workgroups.  An
+  // fp32 wave needs 64 cycles of the matrix pipe per 32x32x2 product, so a deep layer at batch 1
+  // (16 workgroups = 64 of the chip's 1024 SIMDs) is bound by those few waves' matrix time, and
+  // spreading K over more SIMDs pays for the reduction through memory (about 5 us).  In fp16 the
+  // same launches are four times shorter and the reduction costs more than it saves (measured:
+  // layer4 at batch 1 6.5 -> 10 us), so the split is fp32 only.
+  static const int sk_env = [] {
+    const char* e = getenv("NNCV_HIP_SPLITK");
+    return e ? atoi(e) : -1;
+  }();
+  a.ksplit = 1;
+  if (halves && in_dt == kF32 && sk_env != 0 && g.splitk_ws && g.splitk_counters) {
+    const int nslab = a.C * (int)dtype_size(in_dt) / 128;
+    const long long wgs = (long long)a.tiles * (a.F / 32 + (a.aux_F + 31) / 32);
+    const int want = (int)std::min<long long>(std::min(nslab, kMaxSplit), sk_env > 0 ? sk_env : 256 / wgs);
+    if (want >= 2 && wgs <= g.splitk_counters_n) {
+      a.spk = (nslab + want - 1) / want;
+      a.ksplit = (nslab + a.spk - 1) / a.spk;
+      if ((size_t)wgs * a.ksplit * 4096 * sizeof(float) > g.splitk_ws_bytes) a.ksplit = 1;
+    }
+    a.partial = static_cast<float*>(g.splitk_ws);
+    a.counters = g.splitk_counters;
+  }
   if (st == 2) {
     if (h) {
       if (ws == 2) launch_patch_cfg<half_t, half_t, 2, 2, 2, 2>(a, flops, bytes, "conv3x3s2_patch<f16,2,2>", s);
@@ -554,6 +727,7 @@ void launch_conv3x3_patch(const IgemmArgs& g, int in_dt, int out_dt, hipStream_t
       else launch_patch_cfg<half_t, half_t, 1, 4, 2, 2>(a, flops, bytes, "conv3x3s2_patch<f16,1,4>", s);
     } else {
       if (ws == 2) launch_patch_cfg<float, float, 2, 2, 2, 2>(a, flops, bytes, "conv3x3s2_patch<f32,2,2>", s);
+      else if (a.ksplit > 1) launch_patch_cfg<float, float, 1, 4, 1, 2, true>(a, flops, bytes, "conv3x3s2_patch<f32,1,4,half,splitk>", s);
       else if (halves) launch_patch_cfg<float, float, 1, 4, 1, 2>(a, flops, bytes, "conv3x3s2_patch<f32,1,4,half>", s);
       else launch_patch_cfg<float, float, 1, 4, 2, 2>(a, flops, bytes, "conv3x3s2_patch<f32,1,4>", s);
     }
@@ -565,6 +739,7 @@ void launch_conv3x3_patch(const IgemmArgs& g, int in_dt, int out_dt, hipStream_t
   } else {
     if (ws == 4) launch_patch_cfg<float, float, 4, 1, 2>(a, flops, bytes, "conv3x3_patch<f32,4,1>", s);
     else if (ws == 2) launch_patch_cfg<float, float, 2, 2, 2>(a, flops, bytes, "conv3x3_patch<f32,2,2>", s);
+    else if (a.ksplit > 1) launch_patch_cfg<float, float, 1, 4, 1, 1, true>(a, flops, bytes, "conv3x3_patch<f32,1,4,half,splitk>", s);
     else if (halves) launch_patch_cfg<float, float, 1, 4, 1>(a, flops, bytes, "conv3x3_patch<f32,1,4,half>", s);
     else launch_patch_cfg<float, float, 1, 4, 2>(a, flops, bytes, "conv3x3_patch<f32,1,4>", s);
   }

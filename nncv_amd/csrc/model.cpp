@@ -16,6 +16,10 @@ static int env_algo3x3() {
 
 static int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
+// scratch of the patch kernel's K split: at most 256 workgroups' 64x64 fp32 partial tiles
+constexpr size_t kSplitKWsBytes = 256 * 4096 * sizeof(float);
+constexpr int kSplitKCounters = 256;
+
 ConvLayer::ConvLayer(const Desc& d, const void* w, const void* gamma, const void* beta, const void* mean, const void* var,
                      hipStream_t s)
     : d_(d) {
@@ -52,6 +56,10 @@ ConvLayer::ConvLayer(const Desc& d, const void* w, const void* gamma, const void
     if (d.R == 3 && d.S == 3 && (d.stride == 1 || d.stride == 2) && d.pad == 1 && d.C % (128 / (int)es) == 0) {
       wfrag_.reset((size_t)((d.F + 63) / 64) * 64 * 9 * d.C * es);
       launch_weight_frag3x3(w, d.dt, wfrag_.get(), d.dt, d.F, d.C, s);
+      if (d.dt == kF32) {
+        splitk_counters_.reset(kSplitKCounters * sizeof(int));
+        NNCV_HIP_CHECK(hipMemsetAsync(splitk_counters_.get(), 0, splitk_counters_.bytes(), s));
+      }
     }
   }
   if (gamma) {
@@ -78,6 +86,7 @@ size_t ConvLayer::workspace_bytes(int N, int H, int W, bool strided) const {
   // strided (operator-level) form of the igemm path stages NHWC copies of input and output
   if (strided && !d_.stem && algo_ == kAlgoIgemm)
     b += align256((size_t)N * H * W * round_up(d_.C, ce) * es) + 2 * align256((size_t)N * OH * OW * round_up(d_.F, 4) * es);
+  if (!strided && splitk_counters_.get()) b += kSplitKWsBytes;
   return b;
 }
 
@@ -111,6 +120,10 @@ void ConvLayer::forward(const void* in, int N, int H, int W, const void* residua
   a.N = N; a.H = H; a.W = W; a.C = d_.C; a.F = d_.F; a.R = d_.R; a.S = d_.S; a.OH = OH; a.OW = OW;
   a.stride_h = a.stride_w = d_.stride; a.pad_h = a.pad_w = d_.pad;
   a.relu = d_.relu; a.ldo = d_.F; a.batch = 1;
+  if (ws && splitk_counters_.get()) {
+    a.splitk_ws = ws; a.splitk_ws_bytes = kSplitKWsBytes;
+    a.splitk_counters = splitk_counters_.as<int>(); a.splitk_counters_n = kSplitKCounters;
+  }
   launch_igemm(a, d_.dt, d_.dt, s);
 }
 
@@ -151,7 +164,8 @@ bool ConvLayer::fuse_shortcut(const ConvLayer& ds, hipStream_t s) {
   return true;
 }
 
-void ConvLayer::forward_with_shortcut(const void* in, int N, int H, int W, void* out, void* shortcut_out, hipStream_t s) const {
+void ConvLayer::forward_with_shortcut(const void* in, int N, int H, int W, void* out, void* shortcut_out, void* ws,
+                                      hipStream_t s) const {
   NNCV_REQUIRE(aux_F_ > 0, "conv: no fused shortcut");
   const int OH = out_h(H), OW = out_w(W);
   NNCV_REQUIRE(N > 0 && OH > 0 && OW > 0, "conv: empty tensor");
@@ -163,6 +177,10 @@ void ConvLayer::forward_with_shortcut(const void* in, int N, int H, int W, void*
   a.relu = d_.relu; a.ldo = d_.F; a.batch = 1;
   a.aux_f0 = d_.F; a.aux_tap = 4; a.aux_relu = aux_relu_; a.aux_ldo = aux_F_; a.aux_out = shortcut_out;
   a.alg_flops = (2.0 * d_.F * 9.0 * d_.C + aux_flops_per_pixel_) * N * OH * OW;
+  if (ws && splitk_counters_.get()) {
+    a.splitk_ws = ws; a.splitk_ws_bytes = kSplitKWsBytes;
+    a.splitk_counters = splitk_counters_.as<int>(); a.splitk_counters_n = kSplitKCounters;
+  }
   launch_igemm(a, d_.dt, d_.dt, s);
 }
 
@@ -347,7 +365,7 @@ void ResNet18::forward(const void* src, int N, int H, int W, void* logits, void*
     const int oh = b.c1->out_h(h), ow = b.c1->out_w(w);
     const void* shortcut = x;
     if (b.ds && b.c1->has_shortcut()) {
-      b.c1->forward_with_shortcut(x, N, h, w, y1, idn, s);
+      b.c1->forward_with_shortcut(x, N, h, w, y1, idn, cws, s);
       shortcut = idn;
     } else {
       b.c1->forward(x, N, h, w, nullptr, y1, cws, s);

@@ -50,7 +50,7 @@ class ConvLayer {
   bool fuse_shortcut(const ConvLayer& ds, hipStream_t s);
   bool has_shortcut() const { return aux_F_ > 0; }
   // forward() of this layer into `out` and of the fused shortcut into `shortcut_out`
-  void forward_with_shortcut(const void* in, int N, int H, int W, void* out, void* shortcut_out, hipStream_t s) const;
+  void forward_with_shortcut(const void* in, int N, int H, int W, void* out, void* shortcut_out, void* ws, hipStream_t s) const;
 
  private:
   Desc d_;
@@ -58,6 +58,7 @@ class ConvLayer {
   DeviceBuffer wt_, wfrag_, U_, scale_, shift_, wt_shift_;
   DeviceBuffer wt_cat_, scale_cat_, shift_cat_;  // this layer's filters followed by the fused shortcut's
   DeviceBuffer aux_wfrag_;  // the fused shortcut's filters alone, fragment-major (stride-2 patch kernel)
+  DeviceBuffer splitk_counters_;  // tickets of the patch kernel's K split (fp32); zero between launches
   int aux_F_ = 0;
   int aux_relu_ = 0;
   double aux_flops_per_pixel_ = 0.0;

@@ -177,3 +177,38 @@ def test_random_layers(dt):
             assert max_rel(got, want) < FP32_MAX_REL, seed
         done += 1
     assert done == 50
+
+
+def test_fp32_k_split_over_workgroups_is_exact_and_repeatable():
+    """A deep fp32 3x3 layer at batch 1 has too few workgroups for the chip, so the patch kernel splits its K walk over
+    several per output tile; the last one to arrive adds the partial tiles in slab order.  Whichever arrives last, the bits
+    must be the same on every launch (the tickets return to zero each time), and they must match the oracle."""
+    N, C, F, H = 1, 512, 512, 7
+    x = synth.normal(7100, (N, C, H, H))
+    w = synth.normal(7101, (F, C, 3, 3), std=float(np.sqrt(2.0 / (C * 9))))
+    bn = bn_params(7102, F)
+    res = synth.normal(7106, (N, F, H, H))
+    want = oracle_layer(x, w, 1, 1, bn, res, relu=True)
+    layer = Conv(abi.F32, w, 1, 1, bn=bn, relu=True, algo=abi.ALGO_IGEMM)
+    xd, rd = dev(nhwc(x), abi.F32), dev(nhwc(res), abi.F32)
+    abi.profile_enable(True)
+    try:
+        abi.profile_report()
+        first = host(layer(xd, abi.NHWC, residual=rd))
+        tags = list(abi.profile_report())
+    finally:
+        abi.profile_enable(False)
+    print("tags", tags, flush=True)
+    assert any("splitk" in t for t in tags)
+    assert max_rel(nchw(first), want) < FP32_MAX_REL
+    for _ in range(20):
+        again = host(layer(xd, abi.NHWC, residual=rd))
+        assert np.array_equal(first.view(np.uint32), again.view(np.uint32))
+    # a stride-2 layer with several slabs takes the same path
+    w2 = synth.normal(7111, (F, 256, 3, 3), std=float(np.sqrt(2.0 / (256 * 9))))
+    x2 = synth.normal(7110, (2, 256, 14, 14))
+    l2 = Conv(abi.F32, w2, 2, 1, bn=bn, relu=False, algo=abi.ALGO_IGEMM)
+    got2 = nchw(host(l2(dev(nhwc(x2), abi.F32), abi.NHWC)))
+    assert max_rel(got2, oracle_layer(x2, w2, 2, 1, bn, None, relu=False)) < FP32_MAX_REL
+    layer.close()
+    l2.close()

@@ -2,8 +2,9 @@
 //
 // The implicit-GEMM kernels gather every input pixel once per filter tap, i.e. nine times, from
 // L2, and need a workgroup barrier per K step.  Here a workgroup owns an output tile of TN images
-// x TH rows x the full width W (at most 64*WS pixel "slots") and 64 filters, and per 128-byte
-// channel slab (64 halves / 32 floats):
+// x TH rows x TW columns (at most 64*WS pixel "slots"; TW is the full width unless a row is wider
+// than the 64 pixels the loader walks, in which case rows are cut into column tiles) and 64
+// filters, and per 128-byte channel slab (64 halves / 32 floats):
 //   * loads the (TH+2) x (W+2) haloed input patch ONCE into LDS (zero halo straight from the
 //     buffer-load range check; the reference materialises it with tensor.pad,
 //     tests/Nets/Res18.mlir:152-155),
@@ -50,14 +51,15 @@ struct PatchArgs {
   const float* shift;    // [F] or null
   const void* residual;  // like out, or null
   int N, H, W, C, F, relu;
-  int TN, TH;            // tile: TN images x TH rows x W columns
-  int tiles_y;           // ceil(H / TH)
+  int TN, TH;            // tile: TN images x TH output rows x TW output columns
+  int tiles_y;           // tiles per group of TN images: ceil(OH / TH) row bands x NTX column tiles
   int tiles;             // ceil(N / TN) * tiles_y
+  int txw;               // TW | NTX << 16.  NTX = 1 (TW = the full output width) unless a row is too wide for the loader
   int rw_log;            // patch loader: 2^rw_log >= patch columns per loader row
   int OH, OW;            // output size (stride 2; stride 1: H, W)
   int xcd_by_filter;     // XCD <- filter block instead of XCD <- tile range
   unsigned in_bytes, wf_bytes;
-  float inv_ph, inv_thw, inv_w;  // 1/(patch rows per image), 1/(TH*OW), 1/OW
+  float inv_ph, inv_thw, inv_w;  // 1/(patch rows per image), 1/(TH*TW), 1/TW
   // Stride 2 only: filter blocks >= aux_fb0 (in units of the workgroup's 32*NI filters) belong to a
   // 1x1 stride-2 convolution over the same input (the shortcut of a down-sampling block), with its
   // own output tensor [N][OH][OW][aux_F], scale/shift and ReLU flag.  aux_F = 0: none.
@@ -229,7 +231,7 @@ struct PatchCfg {
 // walk is one tap per slab.  A ninth of the work of a 3x3 block: these workgroups have the highest
 // block indices and fill the tail of the launch.
 template <typename T, typename OutT, int WS, int WK, int NI>
-__device__ __forceinline__ void patch_aux_1x1(const PatchArgs& a, unsigned char* smem, int n0, int y0, int fb, int tid) {
+__device__ __forceinline__ void patch_aux_1x1(const PatchArgs& a, unsigned char* smem, int n0, int y0, int x0, int fb, int tid) {
   constexpr int NT = 64 * WS * WK, ES = sizeof(T), KPG = 4 / WK;
   constexpr int AP = 64 * WS / (NT / 8);  // loader passes: NT/8 pixels each
   const int lane = tid & 63;
@@ -239,14 +241,16 @@ __device__ __forceinline__ void patch_aux_1x1(const PatchArgs& a, unsigned char*
   const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(a.in, a.in_bytes);
   const __amdgpu_buffer_rsrc_t rs_wf = make_rsrc(a.aux_wf, a.aux_wf_bytes);
   const int nslab = a.C * ES / 128;
-  const int nslots = a.TN * a.TH * a.OW;
+  const int TW = a.txw & 0xffff;
+  const int nslots = a.TN * a.TH * TW;
   auto decode = [&](int sl, int* n, int* oy, int* ox) {
-    int nl = 0, rem = sl;
-    if (a.TN > 1) nl = fast_div(sl, a.TH * a.OW, a.inv_thw, &rem);
-    const int ty = fast_div(rem, a.OW, a.inv_w, ox);
+    int nl = 0, rem = sl, tx;
+    if (a.TN > 1) nl = fast_div(sl, a.TH * TW, a.inv_thw, &rem);
+    const int ty = fast_div(rem, TW, a.inv_w, &tx);
     *n = n0 + nl;
     *oy = y0 + ty;
-    return (sl < nslots) & (*n < a.N) & (*oy < a.OH);
+    *ox = x0 + tx;
+    return (sl < nslots) & (*n < a.N) & (*oy < a.OH) & (*ox < a.OW);
   };
   const int p8 = tid >> 3, pc = (tid & 7) * 16;
   const unsigned ces = (unsigned)(a.C * ES);
@@ -324,8 +328,9 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
     // the values the patch addressing needs first, as plain leading arguments: those are preloaded
     // into SGPRs at wave launch, the struct behind them is fetched by a scalar load as usual
     const void* in_p, int tiles_p, int tiles_y_p, int tn_p, int th_p, int n_p, int h_p, int w_p, int c_p, int rw_log_p,
-    int xcd_by_filter_p, unsigned in_bytes_p, const PatchArgs a_rest) {
+    int xcd_by_filter_p, unsigned in_bytes_p, int txw_p, const PatchArgs a_rest) {
   PatchArgs a = a_rest;
+  a.txw = txw_p;
   a.in = in_p; a.tiles = tiles_p; a.tiles_y = tiles_y_p; a.TN = tn_p; a.TH = th_p; a.N = n_p; a.H = h_p; a.W = w_p; a.C = c_p;
   a.rw_log = rw_log_p; a.xcd_by_filter = xcd_by_filter_p; a.in_bytes = in_bytes_p;
   typedef PatchCfg<WS, WK, ST> Cfg;
@@ -356,11 +361,19 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   }
   if (tile >= a.tiles) return;
   const int f0blk = fblk * (32 * NI);
-  const int n0 = (tile / a.tiles_y) * a.TN, y0 = (tile % a.tiles_y) * a.TH;
+  // tile -> image group, row band, column tile (one column tile unless the rows are too wide)
+  const int TW = a.txw & 0xffff, ntx = a.txw >> 16;
+  const int n0 = (tile / a.tiles_y) * a.TN;
+  int band = tile % a.tiles_y, x0 = 0;
+  if (ntx > 1) {
+    x0 = (band % ntx) * TW;
+    band /= ntx;
+  }
+  const int y0 = band * a.TH;
   if constexpr (ST == 2) {
     if (fblk >= a.aux_fb0) {  // uniform for the workgroup
       if (SK && blockIdx.z != 0) return;  // the auxiliary blocks do not split K
-      patch_aux_1x1<T, OutT, WS, WK, NI>(a, smem, n0, y0, fblk - a.aux_fb0, threadIdx.x);
+      patch_aux_1x1<T, OutT, WS, WK, NI>(a, smem, n0, y0, x0, fblk - a.aux_fb0, threadIdx.x);
       return;
     }
   }
@@ -368,8 +381,8 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   // 2tx..2tx+2.  The patch keeps the even and the odd columns of a row apart (PWh pixels each), so
   // that the slots of consecutive output pixels stay consecutive in LDS for every tap.
   const int OH = ST == 1 ? a.H : a.OH, OW = ST == 1 ? a.W : a.OW;
-  const int PH = ST == 1 ? a.TH + 2 : 2 * a.TH + 1, PW = ST == 1 ? a.W + 2 : 2 * OW + 1;
-  const int PWh = OW + 1;
+  const int PH = ST == 1 ? a.TH + 2 : 2 * a.TH + 1, PW = ST == 1 ? TW + 2 : 2 * TW + 1;
+  const int PWh = TW + 1;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in an SGPR
@@ -393,12 +406,12 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   const unsigned ces = (unsigned)(a.C * ES);
   unsigned pvoff[kPasses];
   if (a.TN == 1) {  // one image per tile: patch row r is image row y0 - 1 + r
-    const int rowbase = (n0 * a.H + ST * y0 - 1) * a.W - 1;
+    const int rowbase = (n0 * a.H + ST * y0 - 1) * a.W + ST * x0 - 1;
 #pragma unroll
     for (int i = 0; i < kPasses; ++i) {
       const int q = i * (NT / 8) + p8;
       const int r = q >> a.rw_log, px = q & rwm;
-      const bool ok = (r < prows) & ((unsigned)(ST * y0 - 1 + r) < (unsigned)a.H) & ((unsigned)(px - 1) < (unsigned)a.W);
+      const bool ok = (r < prows) & ((unsigned)(ST * y0 - 1 + r) < (unsigned)a.H) & ((unsigned)(ST * x0 + px - 1) < (unsigned)a.W);
       const unsigned off = __umul24((unsigned)(rowbase + (int)__umul24(r, a.W) + px), ces) + pc;
       pvoff[i] = ok ? off : kOOBp;
     }
@@ -410,8 +423,8 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
       int py;
       const int n = n0 + fast_div(r, PH, a.inv_ph, &py);
       const int iy = ST * y0 + py - 1;
-      const bool ok = (r < prows) & (n < a.N) & ((unsigned)iy < (unsigned)a.H) & ((unsigned)(px - 1) < (unsigned)a.W);
-      const unsigned off = __umul24((unsigned)((n * a.H + iy) * a.W + px - 1), ces) + pc;
+      const bool ok = (r < prows) & (n < a.N) & ((unsigned)iy < (unsigned)a.H) & ((unsigned)(ST * x0 + px - 1) < (unsigned)a.W);
+      const unsigned off = __umul24((unsigned)((n * a.H + iy) * a.W + ST * x0 + px - 1), ces) + pc;
       pvoff[i] = ok ? off : kOOBp;
     }
   }
@@ -459,20 +472,20 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   ess.load(lane, f0blk, a.F, a.scale, a.shift);
 
   // ---- this lane's two pixel slots ----
-  const int nslots = a.TN * a.TH * OW;
+  const int nslots = a.TN * a.TH * TW;
   int sbase[2];  // byte offset of the slot's tap-(0,0) pixel in the patch
   int obase[2];  // element offset of the slot's output pixel row, or -1
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int sl = ws * 64 + j * 32 + lrow;
     int nl = 0, rem = sl, tx;
-    if (a.TN > 1) nl = fast_div(sl, a.TH * OW, a.inv_thw, &rem);
-    const int ty = fast_div(rem, OW, a.inv_w, &tx);
-    const bool ok = (sl < nslots) & ((n0 + nl) < a.N) & ((y0 + ty) < OH);
+    if (a.TN > 1) nl = fast_div(sl, a.TH * TW, a.inv_thw, &rem);
+    const int ty = fast_div(rem, TW, a.inv_w, &tx);
+    const bool ok = (sl < nslots) & ((n0 + nl) < a.N) & ((y0 + ty) < OH) & ((x0 + tx) < OW);
     // slots beyond the tile read pixel 0 of the patch; their results are never stored
     const int cell = ST == 1 ? __umul24(__umul24(nl, PH) + ty, PW) + tx : __umul24(__umul24(nl, PH) + 2 * ty, 2 * PWh) + tx;
     sbase[j] = (ok ? (int)__umul24(cell, kPitch) : 0) + (lchunk + 2 * wk * KPG) * 16;
-    obase[j] = ok ? (((n0 + nl) * OH + y0 + ty) * OW + tx) * a.F : -1;
+    obase[j] = ok ? (((n0 + nl) * OH + y0 + ty) * OW + x0 + tx) * a.F : -1;
   }
 
   floatx16 acc[2][2];  // [filter half][pixel half]; with NI = 1 only acc[0] is used
@@ -562,10 +575,13 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   }
 }
 
-// Tile choice for 64*ws slots: TN images x TH output rows x W output columns, patch of at most
-// `cap` pixels, which the loader walks as rows of 2^rw_log pixels, `cover` padded pixels at most.
-// H, W: output size (= input size at stride 1).
-static bool plan_tile(int st, int N, int H, int W, int slots, int cap, int cover, int* TN, int* TH, int* rw_log) {
+// Tile choice for 64*ws slots: TN images x TH output rows x TW output columns, patch of at most
+// `cap` cells, which the loader walks as rows of 2^rw_log <= 64 pixels, `cover` padded pixels at
+// most.  H, W: output size (= input size at stride 1).  Rows whose patch is wider than the loader
+// takes are cut into NTX column tiles of equal width.
+struct TilePlan { int TN, TH, TW, NTX, rw_log; };
+static bool plan_tile_ntx(int st, int N, int H, int W_full, int ntx, int slots, int cap, int cover, TilePlan* t) {
+  const int W = (W_full + ntx - 1) / ntx;
   const int PW = st == 1 ? W + 2 : 2 * W + 1;       // patch columns the loader walks
   const int cells = st == 1 ? W + 2 : 2 * (W + 1);  // LDS cells per patch row
   auto prow = [&](int th) { return st == 1 ? th + 2 : 2 * th + 1; };
@@ -578,22 +594,40 @@ static bool plan_tile(int st, int N, int H, int W, int slots, int cap, int cover
   for (int th = 1; th <= H; ++th)
     if (fits(1, th)) thmax = th;
   if (thmax == 0) return false;
-  *rw_log = lg;
+  t->rw_log = lg; t->TW = W; t->NTX = ntx; t->TN = 1;
   if (thmax < H) {
     const int nt = (H + thmax - 1) / thmax;
-    *TH = (H + nt - 1) / nt;  // balanced rows per tile
-    *TN = 1;
+    t->TH = (H + nt - 1) / nt;  // balanced rows per tile
     return true;
   }
-  int tn = 1;
-  while (tn + 1 <= N && fits(tn + 1, H)) ++tn;
-  *TN = tn;
-  *TH = H;
+  t->TH = H;
+  if (ntx == 1)
+    while (t->TN + 1 <= N && fits(t->TN + 1, H)) ++t->TN;
   return true;
 }
 
+static bool plan_tile(int st, int N, int H, int W, int slots, int cap, int cover, TilePlan* t) {
+  const int max_tw = std::min(slots, st == 1 ? 62 : 31);
+  const int ntx0 = (W + max_tw - 1) / max_tw;
+  if (ntx0 == 1) return plan_tile_ntx(st, N, H, W, 1, slots, cap, cover, t);
+  // Wide rows: the loader walks the patch as rows of a power of two, so the narrowest cut is not
+  // always the one that fills the slots best (64 columns: two tiles of 32 give a 34-wide patch walked
+  // as 64 and one row per tile; four tiles of 16 fill all 64 slots with four rows).  Try a few.
+  long long best_tiles = 0;
+  for (int ntx = ntx0; ntx <= ntx0 + 6 && ntx <= W; ++ntx) {
+    TilePlan c;
+    if (!plan_tile_ntx(st, N, H, W, ntx, slots, cap, cover, &c)) continue;
+    const long long tiles = (long long)((H + c.TH - 1) / c.TH) * ntx;
+    if (best_tiles == 0 || tiles < best_tiles) {
+      best_tiles = tiles;
+      *t = c;
+    }
+  }
+  return best_tiles > 0;
+}
+
 // Picks the wave arrangement: the largest pixel tile that still gives (about) every CU a workgroup.
-static bool plan_patch(int st, int N, int H, int W, int F, int slabs, int* WS, int* TN, int* TH, int* rw_log) {
+static bool plan_patch(int st, int N, int H, int W, int F, int slabs, int* WS, TilePlan* plan) {
   static const int force = [] {
     const char* e = getenv("NNCV_HIP_PATCH_WS");
     return e ? atoi(e) : 0;
@@ -614,15 +648,15 @@ static bool plan_patch(int st, int N, int H, int W, int F, int slabs, int* WS, i
       cap = ws == 2 ? PatchCfg<2, 2, 2>::cap : PatchCfg<1, 4, 2>::cap;
       cover = ws == 2 ? PatchCfg<2, 2, 2>::cover : PatchCfg<1, 4, 2>::cover;
     }
-    int tn, th, lg;
-    if (!plan_tile(st, N, H, W, 64 * ws, cap, cover, &tn, &th, &lg)) continue;
-    const long long tiles = (long long)((N + tn - 1) / tn) * ((H + th - 1) / th);
+    TilePlan t;
+    if (!plan_tile(st, N, H, W, 64 * ws, cap, cover, &t)) continue;
+    const long long tiles = (long long)((N + t.TN - 1) / t.TN) * ((H + t.TH - 1) / t.TH) * t.NTX;
     const double used = (double)N * H * W / ((double)tiles * 64 * ws);
     // "every CU busy" saturates at 7/8 of them: past that a narrower tile only adds halo re-reads
     const double fill = tiles * fb >= 224 ? 1.0 : (double)(tiles * fb) / 224.0;
     const double score = used * fill;
     if (score > best * 1.05) {
-      best = score; *WS = ws; *TN = tn; *TH = th; *rw_log = lg;
+      best = score; *WS = ws; *plan = t;
     }
   }
   return best > 0.0;
@@ -631,7 +665,8 @@ static bool plan_patch(int st, int N, int H, int W, int F, int slabs, int* WS, i
 bool conv3x3_patch_applicable(const IgemmArgs& a, int in_dt) {
   static const bool off = getenv("NNCV_HIP_NO_PATCH") != nullptr;
   const int slab = in_dt == kF16 ? 64 : 32;
-  int ws, tn, th, lg;
+  int ws;
+  TilePlan tp;
   static const bool off2 = getenv("NNCV_HIP_NO_PATCH_S2") != nullptr;
   const int st = a.stride_h;
   // auxiliary filters: the centre tap of a stride-2 launch, given fragment-major
@@ -643,7 +678,7 @@ bool conv3x3_patch_applicable(const IgemmArgs& a, int in_dt) {
          a.batch == 1 && a.pix_stride == 0 && a.C % slab == 0 && fmain % 8 == 0 && a.ldo == fmain &&
          (long long)a.N * a.OH * a.OW * std::max(fmain, faux) < (1ll << 31) && (long long)a.N * a.H * a.W < (1 << 24) && a.in_bytes < kOOBp &&
          (long long)((std::max(fmain, faux) + 63) / 64) * 64 * 9 * a.C * (long long)dtype_size(in_dt) < (1ll << 31) &&
-         plan_patch(st, a.N, a.OH, a.OW, fmain, a.C / slab, &ws, &tn, &th, &lg);
+         plan_patch(st, a.N, a.OH, a.OW, fmain, a.C / slab, &ws, &tp);
 }
 
 template <typename T, typename OutT, int WS, int WK, int NI, int ST = 1, bool SK = false>
@@ -662,7 +697,7 @@ static void launch_patch_cfg(const PatchArgs& a, double flops, double bytes, con
   if (b.xcd_by_filter && fblocks % kXcdsP != 0) b.xcd_by_filter = 0;
   dim3 grid((a.tiles + kXcdsP - 1) / kXcdsP * kXcdsP, fblocks, SK ? a.ksplit : 1);
   hipLaunchKernelGGL(kern, grid, dim3(Cfg::NT), Cfg::smem, s, b.in, b.tiles, b.tiles_y, b.TN, b.TH, b.N, b.H, b.W, b.C, b.rw_log,
-                     b.xcd_by_filter, b.in_bytes, b);
+                     b.xcd_by_filter, b.in_bytes, b.txw, b);
 }
 
 void launch_conv3x3_patch(const IgemmArgs& g, int in_dt, int out_dt, hipStream_t s) {
@@ -677,16 +712,18 @@ void launch_conv3x3_patch(const IgemmArgs& g, int in_dt, int out_dt, hipStream_t
   int ws = 0;
   const int st = g.stride_h;
   a.OH = g.OH; a.OW = g.OW;
-  NNCV_REQUIRE(plan_patch(st, a.N, a.OH, a.OW, a.F, a.C * (int)dtype_size(in_dt) / 128, &ws, &a.TN, &a.TH, &a.rw_log),
-               "conv3x3_patch: no tile fits");
-  a.tiles_y = (a.OH + a.TH - 1) / a.TH;
+  TilePlan tp;
+  NNCV_REQUIRE(plan_patch(st, a.N, a.OH, a.OW, a.F, a.C * (int)dtype_size(in_dt) / 128, &ws, &tp), "conv3x3_patch: no tile fits");
+  a.TN = tp.TN; a.TH = tp.TH; a.rw_log = tp.rw_log;
+  a.txw = tp.TW | (tp.NTX << 16);
+  a.tiles_y = ((a.OH + a.TH - 1) / a.TH) * tp.NTX;
   a.tiles = ((a.N + a.TN - 1) / a.TN) * a.tiles_y;
   a.in_bytes = g.in_bytes;
   a.wf_bytes = (unsigned)((size_t)((a.F + 63) / 64) * 64 * 9 * a.C * dtype_size(in_dt));
   a.xcd_by_filter = ((a.F + 63) / 64) % kXcdsP == 0 && a.wf_bytes > (2u << 20);
   a.inv_ph = 1.0f / (st == 1 ? a.TH + 2 : 2 * a.TH + 1);
-  a.inv_thw = 1.0f / (a.TH * a.OW);
-  a.inv_w = 1.0f / a.OW;
+  a.inv_thw = 1.0f / (a.TH * tp.TW);
+  a.inv_w = 1.0f / tp.TW;
   const double P = (double)a.N * a.OH * a.OW;
   const double flops = 2.0 * P * a.C * (9.0 * a.F + a.aux_F);
   const double es = dtype_size(in_dt), os = dtype_size(out_dt);

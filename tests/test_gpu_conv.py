@@ -38,7 +38,9 @@ CASES = [  # N, C, F, H, W, R, stride, pad
     (5, 256, 64, 14, 14, 3, 1, 1),    # few workgroups -> 2x4 waves, four slabs
     (9, 64, 128, 7, 7, 3, 1, 1),      # several images per tile, last tile short of images
     (2, 64, 72, 30, 62, 3, 1, 1),     # widest row the patch loader takes, F not a multiple of 64
-    (1, 64, 64, 20, 64, 3, 1, 1),     # too wide for the patch kernel: falls back to implicit GEMM
+    (1, 64, 64, 20, 64, 3, 1, 1),     # one row is wider than the patch loader takes: two column tiles of 32
+    (2, 64, 72, 11, 150, 3, 1, 1),    # three column tiles of 50, the halo columns come from the neighbouring tiles
+    (1, 128, 64, 40, 125, 3, 1, 1),   # column tiles of 42 + 42 + 41, two slabs
     (2, 64, 64, 23, 17, 3, 1, 1),     # ragged: H not a multiple of the row tile
     # stride 2 through the LDS-patch kernel (even / odd columns of the patch kept apart)
     (4, 64, 128, 56, 56, 3, 2, 1),    # 2x2 waves, TH=4, one slab
@@ -47,7 +49,8 @@ CASES = [  # N, C, F, H, W, R, stride, pad
     (9, 64, 72, 7, 7, 3, 2, 1),       # several images per tile, F not a multiple of 64
     (2, 64, 64, 23, 17, 3, 2, 1),     # odd sizes: the last input row / column is read by the last output only
     (2, 128, 64, 30, 62, 3, 2, 1),    # widest row the loader takes at stride 2
-    (1, 64, 64, 9, 63, 3, 2, 1),      # one column too wide: implicit GEMM
+    (1, 64, 64, 9, 63, 3, 2, 1),      # 32 output columns: two column tiles of 16
+    (2, 128, 64, 33, 99, 3, 2, 1),    # stride 2, odd width: 50 output columns in two tiles of 25
 ]
 
 

@@ -1,15 +1,19 @@
-// 3x3 stride-1 pad-1 convolution with the haloed input patch resident in LDS (gfx950).
+// 3x3 pad-1 convolution, stride 1 or 2, with the haloed input patch resident in LDS (gfx950).
+// The text below describes stride 1; what stride 2 changes (a 2TH+1 x 2TW+1 patch with its even and
+// odd columns kept apart, the 1x1 shortcut convolution of a down-sampling block as extra filter
+// blocks) is said where the code does it, and so is the split of K over workgroups that small
+// fp32 launches use (tile_reduce_store_splitk).
 //
 // The implicit-GEMM kernels gather every input pixel once per filter tap, i.e. nine times, from
 // L2, and need a workgroup barrier per K step.  Here a workgroup owns an output tile of TN images
 // x TH rows x TW columns (at most 64*WS pixel "slots"; TW is the full width unless a row is wider
 // than the 64 pixels the loader walks, in which case rows are cut into column tiles) and 64
 // filters, and per 128-byte channel slab (64 halves / 32 floats):
-//   * loads the (TH+2) x (W+2) haloed input patch ONCE into LDS (zero halo straight from the
+//   * loads the (TH+2) x (TW+2) haloed input patch ONCE into LDS (zero halo straight from the
 //     buffer-load range check; the reference materialises it with tensor.pad,
 //     tests/Nets/Res18.mlir:152-155),
 //   * walks the nine taps; a tap is a constant byte offset into the patch, so the MFMA pixel
-//     operand of tap (r,s) is read from the same LDS data at  slot_base + (r*(W+2)+s)*pitch,
+//     operand of tap (r,s) is read from the same LDS data at  slot_base + (r*(TW+2)+s)*pitch,
 //   * takes the MFMA weight operand straight from global memory into registers: the filters are
 //     stored fragment-major at model load (launch_weight_frag3x3), so each operand load of a wave
 //     is one contiguous kilobyte at a scalar offset, three taps of loads are always in flight,

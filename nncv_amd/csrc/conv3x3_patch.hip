@@ -58,6 +58,7 @@ struct PatchArgs {
   int TN, TH;            // tile: TN images x TH output rows x TW output columns
   int tiles_y;           // tiles per group of TN images: ceil(OH / TH) row bands x NTX column tiles
   int tiles;             // ceil(N / TN) * tiles_y
+  int ldo, pix;          // elements between pixels of out (and residual) / of in: F and C unless they are slices of wider tensors
   int txw;               // TW | NTX << 16.  NTX = 1 (TW = the full output width) unless a row is too wide for the loader
   int rw_log;            // patch loader: 2^rw_log >= patch columns per loader row
   int OH, OW;            // output size (stride 2; stride 1: H, W)
@@ -257,7 +258,7 @@ __device__ __forceinline__ void patch_aux_1x1(const PatchArgs& a, unsigned char*
     return (sl < nslots) & (*n < a.N) & (*oy < a.OH) & (*ox < a.OW);
   };
   const int p8 = tid >> 3, pc = (tid & 7) * 16;
-  const unsigned ces = (unsigned)(a.C * ES);
+  const unsigned ces = (unsigned)(a.pix * ES);
   unsigned aoff[AP];
 #pragma unroll
   for (int i = 0; i < AP; ++i) {
@@ -327,7 +328,9 @@ __device__ __forceinline__ void patch_aux_1x1(const PatchArgs& a, unsigned char*
                                          static_cast<const OutT*>(nullptr), static_cast<OutT*>(a.aux_out), a.aux_relu);
 }
 
-template <typename T, typename OutT, int WS, int WK, int NI, int ST, bool SK>
+// ACT: the epilogue knows every fused activation (and the residual-after-activation form); without
+// it only ReLU / none, which keeps the register-tight ResNet instances as they were.
+template <typename T, typename OutT, int WS, int WK, int NI, int ST, bool SK, bool ACT>
 __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv3x3_patch_kernel(
     // the values the patch addressing needs first, as plain leading arguments: those are preloaded
     // into SGPRs at wave launch, the struct behind them is fetched by a scalar load as usual
@@ -407,7 +410,7 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   const int p8 = tid >> 3, pc = (tid & 7) * 16;
   const int prows = a.TN * PH;
   const int rwm = (1 << a.rw_log) - 1;
-  const unsigned ces = (unsigned)(a.C * ES);
+  const unsigned ces = (unsigned)(a.pix * ES);
   unsigned pvoff[kPasses];
   if (a.TN == 1) {  // one image per tile: patch row r is image row y0 - 1 + r
     const int rowbase = (n0 * a.H + ST * y0 - 1) * a.W + ST * x0 - 1;
@@ -489,7 +492,7 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
     // slots beyond the tile read pixel 0 of the patch; their results are never stored
     const int cell = ST == 1 ? __umul24(__umul24(nl, PH) + ty, PW) + tx : __umul24(__umul24(nl, PH) + 2 * ty, 2 * PWh) + tx;
     sbase[j] = (ok ? (int)__umul24(cell, kPitch) : 0) + (lchunk + 2 * wk * KPG) * 16;
-    obase[j] = ok ? (((n0 + nl) * OH + y0 + ty) * OW + x0 + tx) * a.F : -1;
+    obase[j] = ok ? (((n0 + nl) * OH + y0 + ty) * OW + x0 + tx) * a.ldo : -1;
   }
 
   floatx16 acc[2][2];  // [filter half][pixel half]; with NI = 1 only acc[0] is used
@@ -574,8 +577,8 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
                                            static_cast<const OutT*>(a.residual), static_cast<OutT*>(a.out), a.relu,
                                            a.partial + (size_t)wg * a.ksplit * 4096, a.counters + wg, blockIdx.z, a.ksplit);
   } else {
-    tile_reduce_store<OutT, WK, NI, false>(acc, smem + ws * WK * kTileBytes, wk, lane, obase, f0blk, a.F, ess,
-                                           static_cast<const OutT*>(a.residual), static_cast<OutT*>(a.out), a.relu);
+    tile_reduce_store<OutT, WK, NI, ACT>(acc, smem + ws * WK * kTileBytes, wk, lane, obase, f0blk, a.F, ess,
+                                         static_cast<const OutT*>(a.residual), static_cast<OutT*>(a.out), a.relu);
   }
 }
 
@@ -613,15 +616,15 @@ static bool plan_tile_ntx(int st, int N, int H, int W_full, int ntx, int slots, 
 static bool plan_tile(int st, int N, int H, int W, int slots, int cap, int cover, TilePlan* t) {
   const int max_tw = std::min(slots, st == 1 ? 62 : 31);
   const int ntx0 = (W + max_tw - 1) / max_tw;
-  if (ntx0 == 1) return plan_tile_ntx(st, N, H, W, 1, slots, cap, cover, t);
-  // Wide rows: the loader walks the patch as rows of a power of two, so the narrowest cut is not
-  // always the one that fills the slots best (64 columns: two tiles of 32 give a 34-wide patch walked
-  // as 64 and one row per tile; four tiles of 16 fill all 64 slots with four rows).  Try a few.
+  // The loader walks the patch as rows of a power of two, so the widest cut is not always the one
+  // that fills the slots best (40 columns: a 42-wide patch is walked as 64 and leaves room for two
+  // output rows, 80 of 128 slots; two column tiles of 20 take six rows, 120 slots).  Try a few cuts
+  // and keep the one with the fewest tiles; ties go to the wider tile (less halo).
   long long best_tiles = 0;
   for (int ntx = ntx0; ntx <= ntx0 + 6 && ntx <= W; ++ntx) {
     TilePlan c;
     if (!plan_tile_ntx(st, N, H, W, ntx, slots, cap, cover, &c)) continue;
-    const long long tiles = (long long)((H + c.TH - 1) / c.TH) * ntx;
+    const long long tiles = (long long)((N + c.TN - 1) / c.TN) * ((H + c.TH - 1) / c.TH) * ntx;
     if (best_tiles == 0 || tiles < best_tiles) {
       best_tiles = tiles;
       *t = c;
@@ -638,7 +641,11 @@ static bool plan_patch(int st, int N, int H, int W, int F, int slabs, int* WS, T
   }();
   const int fb = (F + 63) / 64;
   // Score = fraction of the MFMA slots that carry real pixels x fraction of the 256 CUs that get
-  // a workgroup; ties go to the wider tile (fewer weight re-reads, no cross-wave reduction).
+  // a workgroup.  A narrower tile has to beat a wider one by a quarter: its workgroups re-read the
+  // weights more often, split K across waves and pay the fixed prologue / epilogue per fewer
+  // MFMAs (measured on 56x56x64 at batch 32: 15.8 / 17.1 / 20.7 us for 256 / 128 / 64 slots, and the
+  // same order on 28x28x128, 14x14x256, 80x80x64 and 40x40x128; 64 slots win where the wider tiles
+  // leave CUs idle, 7x7x512 and small batches).
   double best = 0.0;
   for (int ws : {4, 2, 1}) {
     if (force && ws != force) continue;
@@ -659,7 +666,7 @@ static bool plan_patch(int st, int N, int H, int W, int F, int slabs, int* WS, T
     // "every CU busy" saturates at 7/8 of them: past that a narrower tile only adds halo re-reads
     const double fill = tiles * fb >= 224 ? 1.0 : (double)(tiles * fb) / 224.0;
     const double score = used * fill;
-    if (score > best * 1.05) {
+    if (score > best * 1.25) {
       best = score; *WS = ws; *plan = t;
     }
   }
@@ -677,18 +684,30 @@ bool conv3x3_patch_applicable(const IgemmArgs& a, int in_dt) {
   const int fmain = a.aux_f0 ? a.aux_f0 : a.F, faux = a.F - fmain;
   const bool aux_ok = a.aux_f0 == 0 || (st == 2 && a.aux_tap == 4 && a.aux_wt_frag && a.aux_out && a.aux_relu <= kActRelu && a.aux_f0 % 64 == 0 &&
                                         faux % 8 == 0 && a.aux_ldo == faux);
-  return !off && aux_ok && a.relu <= kActRelu && a.wt_frag && a.R == 3 && a.S == 3 && (st == 1 || (st == 2 && !off2)) && a.stride_w == st &&
+  // other activations than ReLU (and the residual added after them): fp16 instances only
+  static const bool off_act = getenv("NNCV_HIP_NO_PATCH_ACT") != nullptr;
+  const bool act_ok = a.relu <= kActRelu || (in_dt == kF16 && !off_act && a.aux_f0 == 0 && (a.relu & 0xff) <= kActSigmoid &&
+                                             (a.relu & ~(0xff | kActResidualAfter)) == 0);
+  const int pix = a.pix_stride ? a.pix_stride : a.C;
+  // Stride 2 pays while the launch is small: its workgroups load four input pixels per output pixel
+  // in front of the same K walk, which the implicit-GEMM kernel overtakes once it has enough
+  // 128x128 tiles for several rounds per CU (measured at 15 GFLOP per launch: 29-34 us there, 35-38
+  // here; at 3.7 GFLOP: 13-17 us there, 10-11 here).
+  const double s2_flops = 2.0 * a.N * a.OH * a.OW * (double)fmain * 9.0 * a.C;
+  if (st == 2 && s2_flops > 8e9) return false;
+  return !off && aux_ok && act_ok && a.wt_frag && a.R == 3 && a.S == 3 && (st == 1 || (st == 2 && !off2)) && a.stride_w == st &&
          a.pad_h == 1 && a.pad_w == 1 && a.OH == (a.H - 1) / st + 1 && a.OW == (a.W - 1) / st + 1 &&
-         a.batch == 1 && a.pix_stride == 0 && a.C % slab == 0 && fmain % 8 == 0 && a.ldo == fmain &&
-         (long long)a.N * a.OH * a.OW * std::max(fmain, faux) < (1ll << 31) && (long long)a.N * a.H * a.W < (1 << 24) && a.in_bytes < kOOBp &&
+         a.batch == 1 && pix % (slab / 8) == 0 && a.C % slab == 0 && fmain % 8 == 0 && a.ldo >= fmain && a.ldo % (slab / 8) == 0 &&
+         (long long)a.N * a.OH * a.OW * std::max(a.ldo, faux) < (1ll << 31) && (long long)a.N * a.H * a.W < (1 << 24) && a.in_bytes < kOOBp &&
+         (long long)pix * (long long)dtype_size(in_dt) < (1 << 24) &&
          (long long)((std::max(fmain, faux) + 63) / 64) * 64 * 9 * a.C * (long long)dtype_size(in_dt) < (1ll << 31) &&
          plan_patch(st, a.N, a.OH, a.OW, fmain, a.C / slab, &ws, &tp);
 }
 
-template <typename T, typename OutT, int WS, int WK, int NI, int ST = 1, bool SK = false>
+template <typename T, typename OutT, int WS, int WK, int NI, int ST = 1, bool SK = false, bool ACT = false>
 static void launch_patch_cfg(const PatchArgs& a, double flops, double bytes, const char* tag, hipStream_t s) {
   typedef PatchCfg<WS, WK, ST> Cfg;
-  auto kern = conv3x3_patch_kernel<T, OutT, WS, WK, NI, ST, SK>;
+  auto kern = conv3x3_patch_kernel<T, OutT, WS, WK, NI, ST, SK, ACT>;
   static const bool attr = [&] {
     NNCV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::smem));
     return true;
@@ -708,6 +727,7 @@ void launch_conv3x3_patch(const IgemmArgs& g, int in_dt, int out_dt, hipStream_t
   PatchArgs a{};
   a.in = g.in; a.wf = g.wt_frag; a.out = g.out; a.scale = g.scale; a.shift = g.shift; a.residual = g.residual;
   a.N = g.N; a.H = g.H; a.W = g.W; a.C = g.C; a.F = g.aux_f0 ? g.aux_f0 : g.F; a.relu = g.relu;
+  a.ldo = g.ldo; a.pix = g.pix_stride ? g.pix_stride : g.C;
   if (g.aux_f0) {
     a.aux_F = g.F - g.aux_f0; a.aux_wf = g.aux_wt_frag; a.aux_out = g.aux_out; a.aux_relu = g.aux_relu;
     a.aux_scale = g.scale ? g.scale + g.aux_f0 : nullptr; a.aux_shift = g.shift ? g.shift + g.aux_f0 : nullptr;
@@ -761,7 +781,20 @@ void launch_conv3x3_patch(const IgemmArgs& g, int in_dt, int out_dt, hipStream_t
     a.partial = static_cast<float*>(g.splitk_ws);
     a.counters = g.splitk_counters;
   }
-  if (st == 2) {
+  const bool act = a.relu > kActRelu;
+  if (act) {
+    NNCV_REQUIRE(h, "conv3x3_patch: activations other than ReLU are fp16 only");
+    if (st == 2) {
+      if (ws == 2) launch_patch_cfg<half_t, half_t, 2, 2, 2, 2, false, true>(a, flops, bytes, "conv3x3s2_patch<f16,2,2,act>", s);
+      else if (halves) launch_patch_cfg<half_t, half_t, 1, 4, 1, 2, false, true>(a, flops, bytes, "conv3x3s2_patch<f16,1,4,half,act>", s);
+      else launch_patch_cfg<half_t, half_t, 1, 4, 2, 2, false, true>(a, flops, bytes, "conv3x3s2_patch<f16,1,4,act>", s);
+    } else {
+      if (ws == 4) launch_patch_cfg<half_t, half_t, 4, 1, 2, 1, false, true>(a, flops, bytes, "conv3x3_patch<f16,4,1,act>", s);
+      else if (ws == 2) launch_patch_cfg<half_t, half_t, 2, 2, 2, 1, false, true>(a, flops, bytes, "conv3x3_patch<f16,2,2,act>", s);
+      else if (halves) launch_patch_cfg<half_t, half_t, 1, 4, 1, 1, false, true>(a, flops, bytes, "conv3x3_patch<f16,1,4,half,act>", s);
+      else launch_patch_cfg<half_t, half_t, 1, 4, 2, 1, false, true>(a, flops, bytes, "conv3x3_patch<f16,1,4,act>", s);
+    }
+  } else if (st == 2) {
     if (h) {
       if (ws == 2) launch_patch_cfg<half_t, half_t, 2, 2, 2, 2>(a, flops, bytes, "conv3x3s2_patch<f16,2,2>", s);
       else if (halves) launch_patch_cfg<half_t, half_t, 1, 4, 1, 2>(a, flops, bytes, "conv3x3s2_patch<f16,1,4,half>", s);

@@ -249,6 +249,7 @@ void launch_maxpool_nhwc(const void* in, void* out, int dt, int N, int H, int W,
 // anchor_wh: A (w, h) pairs already multiplied by the stride.
 struct DetectArgs {
   const void* head; float* out; int N, H, W, A, F, ldc; long long box0, boxes_total; float stride; float anchor_wh[8];
+  float inv_f, inv_w;  // filled in by the launcher
 };
 void launch_yolo_detect(const DetectArgs& a, int dt, hipStream_t s);
 void launch_cast(const void* src, int src_dt, void* dst, int dst_dt, long long n, hipStream_t s);

@@ -550,13 +550,19 @@ __global__ __launch_bounds__(256) void yolo_detect_kernel(const DetectArgs a) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   const int HWF = a.H * a.W * a.F;
   if (i >= HWF) return;
-  const int pix = i / a.F, k = i - pix * a.F;
+  // i / F and pix / W by float reciprocal + correction (exact below 2^24, which the launcher checks):
+  // the integer-divide expansion was half of this kernel's instructions
+  int pix = (int)((float)i * a.inv_f), k = i - pix * a.F;
+  if (k >= a.F) { ++pix; k -= a.F; }
+  if (k < 0) { --pix; k += a.F; }
   const T* head = static_cast<const T*>(a.head);
   const float v = (float)head[((long long)n * a.H * a.W + pix) * a.ldc + an * a.F + k];
   const float sg = 1.0f / (expf(-v) + 1.0f);
   float o = sg;
   if (k < 4) {
-    const int y = pix / a.W, x = pix - y * a.W;
+    int y = (int)((float)pix * a.inv_w), x = pix - y * a.W;
+    if (x >= a.W) { ++y; x -= a.W; }
+    if (x < 0) { --y; x += a.W; }
     if (k < 2) {
       const float g = (float)(k == 0 ? x : y) - 0.5f;
       o = (sg * 2.0f + g) * a.stride;
@@ -570,14 +576,17 @@ __global__ __launch_bounds__(256) void yolo_detect_kernel(const DetectArgs a) {
 
 void launch_yolo_detect(const DetectArgs& a, int dt, hipStream_t s) {
   NNCV_REQUIRE(a.A >= 1 && a.A <= 4 && a.F >= 5 && a.A * a.F <= a.ldc && a.N >= 1 && a.H >= 1 && a.W >= 1, "yolo_detect: bad shape");
-  NNCV_REQUIRE((long long)a.H * a.W * a.F < (1ll << 31) && (long long)a.N * a.A <= 65535, "yolo_detect: level too large");
+  NNCV_REQUIRE((long long)a.H * a.W * a.F < (1ll << 24) && (long long)a.N * a.A <= 65535, "yolo_detect: level too large");
+  DetectArgs b = a;
+  b.inv_f = 1.0f / (float)a.F;
+  b.inv_w = 1.0f / (float)a.W;
   const long long work = (long long)a.N * a.A * a.H * a.W * a.F;
   ProfScope prof("yolo_detect", 0.0, (double)work * (dtype_size(dt) + 4.0), s);
   dim3 grid((unsigned)(((long long)a.H * a.W * a.F + 255) / 256), (unsigned)(a.N * a.A));
   if (dt == kF16)
-    hipLaunchKernelGGL((yolo_detect_kernel<half_t>), grid, dim3(256), 0, s, a);
+    hipLaunchKernelGGL((yolo_detect_kernel<half_t>), grid, dim3(256), 0, s, b);
   else
-    hipLaunchKernelGGL((yolo_detect_kernel<float>), grid, dim3(256), 0, s, a);
+    hipLaunchKernelGGL((yolo_detect_kernel<float>), grid, dim3(256), 0, s, b);
   NNCV_HIP_CHECK(hipGetLastError());
 }
 

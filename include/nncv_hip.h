@@ -114,6 +114,13 @@ int nncv_hip_conv_forward(nncv_hip_conv* c, const void* in, int N, int H, int W,
  * consecutive dispatches, so it reads slightly above a profiler's per-kernel time. */
 int nncv_hip_conv_time(nncv_hip_conv* c, const void* in, int N, int H, int W, const void* residual, void* out, int reps,
                        void* stream, float* avg_us);
+/* Diagnostic, host arithmetic only (works without a GPU): the tile plan of the 3x3 LDS-patch kernel for
+ * N x OH x OW output pixels at `stride` (1 | 2), F filters and `slabs` 128-byte channel slabs.
+ * plan[8] = {WS (64-slot groups per workgroup), TN images, TH rows, TW columns per tile, NTX column tiles per
+ * row band, log2 of the loader's row walk, LDS cells available, pixels the loader can walk}.  Returns 0, or 1 when
+ * no plan exists. No counterpart in the reference: it lets the CPU test suite check the planner's invariants
+ * (a plan that overflows LDS or the loader would fault on the device). */
+int nncv_hip_conv3x3_patch_plan(int stride, int N, int OH, int OW, int F, int slabs, int* plan);
 
 /* C += A.B, fp32 row-major, DEVICE pointers (K and N multiples of 4). */
 /* The reference driver's image preparation and top-1 scan on the device

@@ -472,6 +472,11 @@ void nncv_hip_profile_enable(int on) {
   guarded([&] { profiler_enable(on != 0); });
 }
 
+int nncv_hip_conv3x3_patch_plan(int stride, int N, int OH, int OW, int F, int slabs, int* plan) {
+  if (!plan) return 1;
+  return conv3x3_patch_plan(stride, N, OH, OW, F, slabs, plan) ? 0 : 1;
+}
+
 size_t nncv_hip_profile_report(char* buf, size_t cap) {
   std::string r;
   if (guarded([&] { r = profiler_report(); }) != 0) r = "{}";

@@ -138,6 +138,10 @@ void launch_igemm(const IgemmArgs& a, int in_dt, int out_dt, hipStream_t s);
 // 3x3 stride-1 pad-1 layers: direct convolution with the haloed input patch resident in LDS
 // (conv3x3_patch.hip); same arguments and epilogue as the igemm kernels.
 bool conv3x3_patch_applicable(const IgemmArgs& a, int in_dt);
+// The tile plan that kernel would use for N x OH x OW output pixels, F filters and `slabs` 128-byte
+// channel slabs: out = {WS, TN, TH, TW, NTX, rw_log, LDS cells available, loader coverage}.  Host
+// arithmetic only (no device needed); false = no plan.
+bool conv3x3_patch_plan(int stride, int N, int OH, int OW, int F, int slabs, int out[8]);
 void launch_conv3x3_patch(const IgemmArgs& a, int in_dt, int out_dt, hipStream_t s);
 bool igemm_fast_applicable(const IgemmArgs& a, int in_dt, int out_dt);
 void launch_igemm_fast(const IgemmArgs& a, int in_dt, int out_dt, hipStream_t s);

@@ -673,6 +673,22 @@ static bool plan_patch(int st, int N, int H, int W, int F, int slabs, int* WS, T
   return best > 0.0;
 }
 
+bool conv3x3_patch_plan(int stride, int N, int OH, int OW, int F, int slabs, int out[8]) {
+  int ws = 0;
+  TilePlan t{};
+  if ((stride != 1 && stride != 2) || N < 1 || OH < 1 || OW < 1 || F < 1 || slabs < 1 || !plan_patch(stride, N, OH, OW, F, slabs, &ws, &t))
+    return false;
+  out[0] = ws; out[1] = t.TN; out[2] = t.TH; out[3] = t.TW; out[4] = t.NTX; out[5] = t.rw_log;
+  if (stride == 1) {
+    out[6] = ws == 4 ? PatchCfg<4, 1>::cap : ws == 2 ? PatchCfg<2, 2>::cap : PatchCfg<1, 4>::cap;
+    out[7] = ws == 4 ? PatchCfg<4, 1>::cover : ws == 2 ? PatchCfg<2, 2>::cover : PatchCfg<1, 4>::cover;
+  } else {
+    out[6] = ws == 2 ? PatchCfg<2, 2, 2>::cap : PatchCfg<1, 4, 2>::cap;
+    out[7] = ws == 2 ? PatchCfg<2, 2, 2>::cover : PatchCfg<1, 4, 2>::cover;
+  }
+  return true;
+}
+
 bool conv3x3_patch_applicable(const IgemmArgs& a, int in_dt) {
   static const bool off = getenv("NNCV_HIP_NO_PATCH") != nullptr;
   const int slab = in_dt == kF16 ? 64 : 32;

@@ -50,6 +50,15 @@ constexpr int kActResidualAfter = 0x100;
 // `arith.cmpf ugt` + select: NaN is kept, everything not greater than zero becomes +0.
 __device__ __forceinline__ float relu_ugt(float x) { return (x <= 0.0f) ? 0.0f : x; }
 
+// 1 / (1 + exp(-x)) on the hardware's exp2 and reciprocal units (v_exp_f32, v_rcp_f32: about 1 ulp
+// each, so the result is within a few ulp of the correctly rounded one -- far inside the 1e-4 / 1e-2
+// parity bars).  The library expf plus an IEEE division is ~40 instructions per element, which made
+// the SiLU epilogue of YOLOv5's memory-bound layers cost as much as their memory traffic.
+// Limits: x -> -inf gives +0, x -> +inf gives 1, NaN stays NaN.
+__device__ __forceinline__ float sigmoid_fast(float x) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.44269504088896340736f));
+}
+
 __device__ __forceinline__ float act_apply(float x, int act) {
   switch (act) {
     case kActRelu: return relu_ugt(x);
@@ -63,8 +72,8 @@ __device__ __forceinline__ float act_apply(float x, int act) {
       t = 1.0f < t ? 1.0f : t;
       return 0.0f > t ? 0.0f : t;
     }
-    case kActSilu: return x * (1.0f / (1.0f + expf(-x)));
-    case kActSigmoid: return 1.0f / (1.0f + expf(-x));
+    case kActSilu: return x * sigmoid_fast(x);
+    case kActSigmoid: return sigmoid_fast(x);
     default: return x;
   }
 }

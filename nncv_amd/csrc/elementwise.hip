@@ -557,7 +557,7 @@ __global__ __launch_bounds__(256) void yolo_detect_kernel(const DetectArgs a) {
   if (k < 0) { --pix; k += a.F; }
   const T* head = static_cast<const T*>(a.head);
   const float v = (float)head[((long long)n * a.H * a.W + pix) * a.ldc + an * a.F + k];
-  const float sg = 1.0f / (expf(-v) + 1.0f);
+  const float sg = sigmoid_fast(v);
   float o = sg;
   if (k < 4) {
     int y = (int)((float)pix * a.inv_w), x = pix - y * a.W;

@@ -108,7 +108,7 @@ __global__ __launch_bounds__(128) void dwconv_kernel(const DwConvArgs a, int str
     if (ox0 + j >= a.OW) break;
     V o;
 #pragma unroll
-    for (int e = 0; e < VN; ++e) o[e] = (T)act_apply(acc[j][e] * sc[e] + sh[e], a.act);
+    for (int e = 0; e < VN; ++e) o[e] = (T)act_apply<sizeof(T) == 2>(acc[j][e] * sc[e] + sh[e], a.act);
     *reinterpret_cast<V*>(out + (long long)(ox0 + j) * a.C) = o;
   }
 }
@@ -398,7 +398,7 @@ __global__ __launch_bounds__(256) void eltwise_kernel(const T* __restrict__ a, c
   }
   V o;
 #pragma unroll
-  for (int e = 0; e < VN; ++e) o[e] = (T)act_apply(y[e], act);
+  for (int e = 0; e < VN; ++e) o[e] = (T)act_apply<sizeof(T) == 2>(y[e], act);
   *reinterpret_cast<V*>(out + p * ldo + c) = o;
 }
 

@@ -208,7 +208,7 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(const IgemmArgs a) {
           for (int e = 0; e < 4; ++e) y[e] = relu_ugt(y[e]);
         } else if (a.relu) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) y[e] = act_apply(y[e], a.relu & 0xff);
+          for (int e = 0; e < 4; ++e) y[e] = act_apply<sizeof(OutT) == 2>(y[e], a.relu & 0xff);
         }
         if (res && res_after) {
 #pragma unroll

@@ -187,26 +187,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // ---- scale/shift, ReLU, one rounding, tile to LDS; pixels outside the convolution output
     //      (and the spare slot) become the pooling halo ----
     const int cy0 = 2 * py0 - 1, cx0 = 2 * px0 - 1;
+    bool live[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int s = wave * 64 + j * 32 + lrow;
-      const bool live = (s < 255) & ((unsigned)(cy0 + cy[j]) < (unsigned)a.OH) & ((unsigned)(cx0 + cx[j]) < (unsigned)a.OW);
+      live[j] = (s < 255) & ((unsigned)(cy0 + cy[j]) < (unsigned)a.OH) & ((unsigned)(cx0 + cx[j]) < (unsigned)a.OW);
+    }
+    // scale / shift of a channel group are fetched once and used for both of the lane's pixels (the
+    // stores to the convolution tile in between keep the compiler from merging the reads itself;
+    // with the pixel loop outside, this stage took 38 % of the kernel, now 30 %)
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int c = i * 32 + 8 * q + 4 * lchunk;
-          const floatx4 sc = *reinterpret_cast<const floatx4*>(tab + c);
-          const floatx4 sh = *reinterpret_cast<const floatx4*>(tab + 64 + c);
+      for (int q = 0; q < 4; ++q) {
+        const int c = i * 32 + 8 * q + 4 * lchunk;
+        const floatx4 sc = *reinterpret_cast<const floatx4*>(tab + c);
+        const floatx4 sh = *reinterpret_cast<const floatx4*>(tab + 64 + c);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int s = wave * 64 + j * 32 + lrow;
           half4 o;
 #pragma unroll
           for (int e = 0; e < 4; ++e) o[e] = (half_t)relu_ugt(acc[i][j][4 * q + e] * sc[e] + sh[e]);
           typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
           u32x2 bits = __builtin_bit_cast(u32x2, o);
-          if (!live) bits = u32x2{0u, 0u};
+          if (!live[j]) bits = u32x2{0u, 0u};
           *reinterpret_cast<u32x2*>(conv_t + s * kConvPitch + c * 2) = bits;
         }
-    }
+      }
     __syncthreads();
 
     // ---- 3x3 stride-2 max over the convolution tile ----

@@ -215,3 +215,61 @@ def test_fp32_k_split_over_workgroups_is_exact_and_repeatable():
     assert max_rel(got2, oracle_layer(x2, w2, 2, 1, bn, None, relu=False)) < FP32_MAX_REL
     layer.close()
     l2.close()
+
+
+@pytest.mark.parametrize("dt", [abi.F32, abi.F16])
+def test_random_patch_kernel_layers(dt):
+    """40 seeded random 3x3 pad-1 layers per element type inside the LDS-patch kernel's domain (whole channel slabs):
+    stride 1 and 2, rows from 3 to 200 pixels wide (column tiles), batches that need several images per tile or the
+    half-block / K-split forms, filters that are not multiples of 64, and (fp16) every fused activation with the residual
+    before or after it.  Most of them must really have taken that kernel."""
+    f16 = dt == abi.F16
+    slab = 64 if f16 else 32
+    routes = {}
+    abi.profile_enable(True)
+    try:
+        abi.profile_report()
+        for seed in range(9500, 9540):
+            rng = np.random.default_rng(seed)
+            C = slab * int(rng.choice([1, 1, 2, 2, 3, 4]))
+            F = 8 * int(rng.choice([1, 4, 8, 8, 9, 16, 17, 32]))
+            stride = int(rng.choice([1, 2, 2]))
+            H, W = int(rng.integers(3, 48)), int(rng.integers(3, 200))
+            N = int(rng.integers(1, 10))
+            if N * H * W * C > 3e6:
+                N = 1
+            OH, OW = (H - 1) // stride + 1, (W - 1) // stride + 1
+            acts = [abi.ACT_NONE, abi.ACT_RELU, abi.ACT_RELU] + ([abi.ACT_SILU, abi.ACT_HARDSWISH] if f16 else [])
+            act = int(rng.choice(acts))
+            use_bn, use_res = rng.random() < 0.7, rng.random() < 0.4
+            x = synth.normal(seed, (N, C, H, W))
+            w = synth.normal(seed + 1, (F, C, 3, 3), std=float(np.sqrt(2.0 / (C * 9))))
+            bn = bn_params(seed + 2, F) if use_bn else None
+            res = synth.normal(seed + 6, (N, F, OH, OW)) if use_res else None
+            if f16:
+                x, w = synth.round_fp16(x), synth.round_fp16(w)
+                bn = tuple(synth.round_fp16(b) for b in bn) if bn else None
+                res = synth.round_fp16(res) if res is not None else None
+            print("seed", seed, (N, C, F, H, W, stride), "act", act, "bn", use_bn, "res", use_res, flush=True)
+            y = oracle.conv2d_nchw_fchw(oracle.pad_nchw(x, 1), w, stride)
+            if bn:
+                y = oracle.batchnorm(y, *bn)
+            if res is not None:
+                y = (y + res).astype(np.float32)
+            want = oracle.ACTIVATIONS[act](y)
+            conv = Conv(dt, w, stride, 1, bn=bn, relu=act, algo=abi.ALGO_IGEMM)
+            rd = dev(nhwc(res), dt) if res is not None else None
+            got = nchw(host(conv(dev(nhwc(x), dt), abi.NHWC, residual=rd)))
+            conv.close()
+            for k, v in abi.profile_report().items():
+                if "conv" in k or "igemm" in k:
+                    routes[k] = routes.get(k, 0) + v["launches"]
+            if f16:
+                assert rel_l2(got, want) < FP16_REL_L2, seed
+            else:
+                assert max_rel(got, want) < FP32_MAX_REL, seed
+    finally:
+        abi.profile_enable(False)
+    print("routes", routes, flush=True)
+    patch = sum(v for k, v in routes.items() if k.startswith("conv3x3"))
+    assert patch >= 0.8 * sum(routes.values()), routes

@@ -772,7 +772,8 @@ void launch_conv3x3_patch(const IgemmArgs& g, int in_dt, int out_dt, hipStream_t
   NNCV_REQUIRE(h || f, "conv3x3_patch: unsupported dtype combination");
   // Few workgroups (small batch on the deep layers: each streams its filter block's weights through
   // one CU's 64 B/clk vector-memory path): split the 64-filter blocks in two and use twice the CUs.
-  const bool halves = ws == 1 && (long long)a.tiles * ((a.F + 63) / 64 + (a.aux_F + 63) / 64) < 128 && a.F % 64 == 0;
+  // (measured on 7x7x512 -> 512: at 128 whole blocks, batch 16, halves take 10.1 us against 12.1; at 256, batch 32, 15.7 against 13.9)
+  const bool halves = ws == 1 && (long long)a.tiles * ((a.F + 63) / 64 + (a.aux_F + 63) / 64) <= 128 && a.F % 64 == 0;
   if (halves) a.xcd_by_filter = (a.F / 32) % kXcdsP == 0 && a.wf_bytes > (2u << 20);
   // fp32, still few workgroups, several slabs: split K over up to 256 / workgroups workgroups.  An
   // fp32 wave needs 64 cycles of the matrix pipe per 32x32x2 product, so a deep layer at batch 1

@@ -151,7 +151,7 @@ struct IgemmArgs {
 // Dispatches to the fast kernel (igemm_fast.hip) when C is a multiple of one K step and the
 // tensors are below 2 GiB, else to the generic one (igemm.hip).
 void launch_igemm(const IgemmArgs& a, int in_dt, int out_dt, hipStream_t s);
-// 3x3 stride-1 pad-1 layers: direct convolution with the haloed input patch resident in LDS
+// 3x3 pad-1 layers at stride 1 or 2: direct convolution with the haloed input patch resident in LDS
 // (conv3x3_patch.hip); same arguments and epilogue as the igemm kernels.
 bool conv3x3_patch_applicable(const IgemmArgs& a, int in_dt);
 // The tile plan that kernel would use for N x OH x OW output pixels, F filters and `slabs` 128-byte

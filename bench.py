@@ -14,6 +14,8 @@ Besides the headline images/s the line carries
                 workload, against the published dense fp16 MFMA peak;
   kernels       the same event-timed breakdown for every kernel tag (ms per step, share);
   batch1        images/s of the same network at batch 1;
+  conv3x3_sweep BASELINE config 5: each 3x3 layer shape of the network alone at batch 64, TFLOP/s and
+                the fraction of the fp16 matrix peak;
   cpu_baseline  the CPU restatement of the reference's HostWParallel schedule (oracle/, fp32,
                 OpenMP x AVX2) timed on this box's host cores on a bounded sample of the same
                 workload — a reported baseline, not a target.
@@ -54,7 +56,8 @@ def main():
     ap.add_argument("--batch", type=int, default=0, help="0 = the workload's default (32; yolov5s 16)")
     ap.add_argument("--algo", default="auto", choices=["auto", "winograd", "igemm"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-batch1", action="store_true", help="skip the batch-1 measurement (for per-kernel profiles)")
+    ap.add_argument("--no-batch1", action="store_true", help="skip the batch-1 measurement and the per-layer sweep (for per-kernel profiles)")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the per-layer 3x3 sweep at batch 64 (BASELINE config 5)")
     ap.add_argument("--profile-steps", type=int, default=5)
     ap.add_argument("--workload", default="resnet18", choices=["resnet18", "mobilenetv3", "yolov5s"],
                     help="resnet18 = the headline configuration; mobilenetv3 / yolov5s = the networks of tests/Nets/MobileNetV3.mlir "
@@ -200,6 +203,8 @@ def main():
         "device": L.nncv_hip_device_arch().decode(),
     }
 
+    if not (args.no_sweep or args.no_batch1):
+        out["conv3x3_sweep"] = conv3x3_sweep(L, stream)
     if args.copy_calibration:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
         dst = torch.empty_like(src)
@@ -209,6 +214,41 @@ def main():
         out["cpu_baseline"] = cpu_baseline(blob32, x)
     L.nncv_hip_resnet18_destroy(model)
     print(json.dumps(out))
+
+
+def conv3x3_sweep(L, stream, batch=64, reps=200):
+    """BASELINE config 5: the seven 3x3 layer shapes of ResNet-18 at batch 64, fp16, each fused with
+    BN + ReLU (+ the residual add on the stride-1 rows), one layer at a time: `reps` launches back to
+    back between one HIP event pair.  Weights and BN are the seeded ones of the parity tests; the
+    activations are device-side normals (the time does not depend on their values)."""
+    import ctypes
+    import numpy as np
+    import torch
+    from nncv_amd import abi, synth
+    rows = []
+    for i, (c, k, h, st) in enumerate(synth.CFG5_LAYERS):
+        seed = 5000 + 10 * i
+        w = synth.normal(seed + 1, (k, c, 3, 3), std=float(np.sqrt(2.0 / (c * 9)))).astype(np.float16)
+        bn = [synth.uniform(seed + 2, (k,), 0.5, 1.5), synth.normal(seed + 3, (k,), std=0.1),
+              synth.normal(seed + 4, (k,), std=0.1), synth.uniform(seed + 5, (k,), 0.5, 1.5)]
+        bn = [b.astype(np.float16) for b in bn]
+        conv = L.nncv_hip_conv_create(abi.F16, w.ctypes.data, k, c, 3, 3, st, 1, *[b.ctypes.data for b in bn], 1, abi.ALGO_AUTO)
+        if not conv:
+            raise RuntimeError(L.nncv_hip_last_error().decode())
+        oh = (h + 2 - 3) // st + 1
+        xin = torch.randn((batch, h, h, c), device="cuda", dtype=torch.float16)
+        res = torch.randn((batch, oh, oh, k), device="cuda", dtype=torch.float16) if st == 1 else None
+        yout = torch.empty((batch, oh, oh, k), device="cuda", dtype=torch.float16)
+        avg = ctypes.c_float(0.0)
+        abi.check(L.nncv_hip_conv_time(conv, xin.data_ptr(), batch, h, h, res.data_ptr() if res is not None else None,
+                                       yout.data_ptr(), reps, stream, ctypes.byref(avg)))
+        L.nncv_hip_conv_destroy(conv)
+        flops = 2.0 * batch * oh * oh * k * c * 9
+        tf = flops / (avg.value * 1e-6) / 1e12
+        rows.append({"layer": "%d->%d %dx%d s%d" % (c, k, h, h, st), "gflop": round(flops / 1e9, 2),
+                     "avg_launch_us": round(float(avg.value), 2), "tflops": round(tf, 1),
+                     "frac_of_fp16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4)})
+    return {"batch": batch, "dtype": "f16", "epilogue": "BN + ReLU (+ residual on stride-1 rows)", "launches": reps, "rows": rows}
 
 
 def bench_graph(args, L):

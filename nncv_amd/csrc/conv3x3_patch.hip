@@ -474,9 +474,13 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
 #pragma unroll
   for (int q = 0; q < NSET; ++q) wload(wregs[q], q);
 
-  // epilogue scale/shift of this lane's output channels: requested now, used at the very end
+  // epilogue scale/shift of this lane's output channels: requested now, used at the very end --
+  // except in the instances whose tap loop has no 16 registers to spare for them (they would be
+  // spilled to scratch memory around the loop: a wait for every load in flight at the loop's door
+  // and 13 KB of extra HBM writes per workgroup), which request them behind the loop instead
+  constexpr bool kLateScale = sizeof(T) == 2 && (WS == 4 || (ST == 2 && WS == 1 && NI == 2));
   EpiScale<OutT> ess;
-  ess.load(lane, f0blk, a.F, a.scale, a.shift);
+  if constexpr (!kLateScale) ess.load(lane, f0blk, a.F, a.scale, a.shift);
 
   // ---- this lane's two pixel slots ----
   const int nslots = a.TN * a.TH * TW;
@@ -569,6 +573,7 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
       prime(prime, std::integral_constant<int, 0>());
     }
   }
+  if constexpr (kLateScale) ess.load(lane, f0blk, a.F, a.scale, a.shift);
   __syncthreads();  // every wave is done with the patch: LDS becomes the output tiles
 
   if constexpr (SK) {

@@ -85,6 +85,37 @@ __device__ __forceinline__ float act_apply(float x, int act) {
   }
 }
 
+// The same for N values of one lane with ONE dispatch on the activation code.  Epilogues use this
+// form: calling act_apply per element inside an unrolled loop leaves a chain of scalar branches
+// per element in the code (some 400 taken branches per wave in a 64-value epilogue, which was most
+// of the run time of the memory-bound SiLU / hard-swish layers).
+template <bool HALF_OUT = false, int N>
+__device__ __forceinline__ void act_apply_n(float (&y)[N], int act) {
+  switch (act) {
+    case kActRelu:
+#pragma unroll
+      for (int e = 0; e < N; ++e) y[e] = act_apply<HALF_OUT>(y[e], kActRelu);
+      break;
+    case kActHardSwish:
+#pragma unroll
+      for (int e = 0; e < N; ++e) y[e] = act_apply<HALF_OUT>(y[e], kActHardSwish);
+      break;
+    case kActHardSigmoid:
+#pragma unroll
+      for (int e = 0; e < N; ++e) y[e] = act_apply<HALF_OUT>(y[e], kActHardSigmoid);
+      break;
+    case kActSilu:
+#pragma unroll
+      for (int e = 0; e < N; ++e) y[e] = act_apply<HALF_OUT>(y[e], kActSilu);
+      break;
+    case kActSigmoid:
+#pragma unroll
+      for (int e = 0; e < N; ++e) y[e] = act_apply<HALF_OUT>(y[e], kActSigmoid);
+      break;
+    default: break;
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Optional event timing of every launch (profiler.cpp).  `name` must be a string literal or
 // otherwise outlive the scope; flops / bytes are the ALGORITHMIC work of the launch.
@@ -159,6 +190,10 @@ bool conv3x3_patch_applicable(const IgemmArgs& a, int in_dt);
 // arithmetic only (no device needed); false = no plan.
 bool conv3x3_patch_plan(int stride, int N, int OH, int OW, int F, int slabs, int out[8]);
 void launch_conv3x3_patch(const IgemmArgs& a, int in_dt, int out_dt, hipStream_t s);
+// Stride-2 image convolutions over pixel pairs (C = 8, fp16, 6x3 and 3x2 windows, at most 64 filters):
+// the whole K axis in one step (conv_pairs.hip); same arguments and epilogue as the igemm kernels.
+bool conv_pairs_applicable(const IgemmArgs& a, int in_dt, int out_dt);
+void launch_conv_pairs(const IgemmArgs& a, hipStream_t s);
 bool igemm_fast_applicable(const IgemmArgs& a, int in_dt, int out_dt);
 void launch_igemm_fast(const IgemmArgs& a, int in_dt, int out_dt, hipStream_t s);
 

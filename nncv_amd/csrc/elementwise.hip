@@ -107,8 +107,12 @@ __global__ __launch_bounds__(128) void dwconv_kernel(const DwConvArgs a, int str
   for (int j = 0; j < OXT; ++j) {
     if (ox0 + j >= a.OW) break;
     V o;
+    float y[VN];
 #pragma unroll
-    for (int e = 0; e < VN; ++e) o[e] = (T)act_apply<sizeof(T) == 2>(acc[j][e] * sc[e] + sh[e], a.act);
+    for (int e = 0; e < VN; ++e) y[e] = acc[j][e] * sc[e] + sh[e];
+    act_apply_n<sizeof(T) == 2>(y, a.act);
+#pragma unroll
+    for (int e = 0; e < VN; ++e) o[e] = (T)y[e];
     *reinterpret_cast<V*>(out + (long long)(ox0 + j) * a.C) = o;
   }
 }
@@ -397,8 +401,9 @@ __global__ __launch_bounds__(256) void eltwise_kernel(const T* __restrict__ a, c
     for (int e = 0; e < VN; ++e) y[e] += (float)bv[e];
   }
   V o;
+  act_apply_n<sizeof(T) == 2>(y, act);
 #pragma unroll
-  for (int e = 0; e < VN; ++e) o[e] = (T)act_apply<sizeof(T) == 2>(y[e], act);
+  for (int e = 0; e < VN; ++e) o[e] = (T)y[e];
   *reinterpret_cast<V*>(out + p * ldo + c) = o;
 }
 

@@ -207,8 +207,9 @@ __global__ __launch_bounds__(kThreads) void igemm_kernel(const IgemmArgs a) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) y[e] = relu_ugt(y[e]);
         } else if (a.relu) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) y[e] = act_apply<sizeof(OutT) == 2>(y[e], a.relu & 0xff);
+          float t[4] = {y[0], y[1], y[2], y[3]};
+          act_apply_n<sizeof(OutT) == 2>(t, a.relu & 0xff);
+          y = floatx4{t[0], t[1], t[2], t[3]};
         }
         if (res && res_after) {
 #pragma unroll
@@ -282,6 +283,10 @@ void launch_igemm(const IgemmArgs& a_in, int in_dt, int out_dt, hipStream_t s) {
   NNCV_REQUIRE(a.OH >= 1 && a.OW >= 1 && a.OH <= (a.H + 2 * a.pad_h - a.R) / a.stride_h + 1 &&
                    a.OW <= (a.W + 2 * a.pad_w - a.S) / a.stride_w + 1,
                "igemm: output size does not match input/filter/stride/pad");
+  if (conv_pairs_applicable(a, in_dt, out_dt)) {
+    launch_conv_pairs(a, s);
+    return;
+  }
   if (in_dt == out_dt && conv3x3_patch_applicable(a, in_dt)) {
     launch_conv3x3_patch(a, in_dt, out_dt, s);
     return;

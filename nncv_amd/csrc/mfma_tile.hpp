@@ -173,8 +173,7 @@ __device__ __forceinline__ void tile_reduce_store(const floatx16 (&acc)[2][2], u
 #pragma unroll
       for (int e = 0; e < FPL; ++e) y[e] = relu_ugt(y[e]);
     } else if (ACT && relu) {
-#pragma unroll
-      for (int e = 0; e < FPL; ++e) y[e] = act_apply<sizeof(OutT) == 2>(y[e], relu & 0xff);
+      act_apply_n<sizeof(OutT) == 2>(y, relu & 0xff);
     }
     if (res && res_after) {
 #pragma unroll

@@ -420,3 +420,41 @@ def test_random_operator_lists(dt):
             assert err < (FP16_REL_L2 if f16 else FP32_MAX_REL), (seed, err)
         done += 1
     assert done >= 30
+
+
+@pytest.mark.parametrize("k,pad,F,act,shape", [
+    (6, 2, 32, abi.ACT_SILU, (2, 3, 64, 96)),         # YOLOv5s' first layer
+    (6, 2, 32, abi.ACT_SILU, (1, 3, 38, 50)),         # pixel count not a multiple of the 256-pixel tile
+    (6, 2, 64, abi.ACT_RELU, (3, 3, 20, 18)),         # two 32-filter halves per wave
+    (6, 2, 48, abi.ACT_NONE, (1, 3, 16, 16)),         # filters that end inside the second half
+    (3, 1, 16, abi.ACT_HARDSWISH, (2, 3, 64, 64)),    # MobileNetV3's first layer (half of the 32-filter block is padding)
+    (3, 1, 24, abi.ACT_RELU, (1, 3, 33, 46)),         # odd height
+    (3, 1, 64, abi.ACT_SILU, (2, 4, 12, 34)),         # four input channels
+    (3, 1, 8, abi.ACT_NONE, (1, 1, 9, 10)),           # one input channel
+])
+def test_fp16_image_convolution_over_pixel_pairs(k, pad, F, act, shape):
+    """A stride-2 convolution that is the only reader of an image with at most four channels and an even
+    width runs over pixel pairs; 6x6 pad 2 and 3x3 pad 1 windows take the kernel that loads the whole K
+    axis at once (`conv_pairs`).  One-operator graphs against the evaluator, with the route checked."""
+    N, C, H, W = shape
+    w = synth.normal(7900 + k, (F, C, k, k), std=float(np.sqrt(2.0 / (C * k * k))))
+    bnp = (synth.uniform(7902, (F,), 0.5, 1.5), synth.normal(7903, (F,), std=0.1), synth.normal(7904, (F,), std=0.1),
+           synth.uniform(7905, (F,), 0.5, 1.5))
+    blob = r16(np.concatenate([w.ravel()] + list(bnp)))
+    o = F * C * k * k
+    ops = [abi.graph_op(abi.OP_CONV, [0, -1], 1, F=F, K=k, stride=2, pad=pad, act=act, eps=1e-3, w=0,
+                        bn=(o, o + F, o + 2 * F, o + 3 * F))]
+    x = r16(synth.uniform(7906, shape, -1.0, 1.0))
+    print("pair stem", k, pad, F, act, shape, flush=True)
+    g = Graph(ops, C, blob, abi.F16)
+    abi.profile_enable(True)
+    abi.profile_report()
+    got = host(g(dev(x, abi.F16)))
+    tags = abi.profile_report()
+    abi.profile_enable(False)
+    want = oracle.run_graph(ops, x, blob, C)
+    g.close()
+    assert any(t.startswith("conv_pairs<f16,%s" % ("6x3" if k == 6 else "3x2")) for t in tags), sorted(tags)
+    assert got.shape == want.shape
+    assert rel_l2(got, want) < 2e-3  # one layer: only the rounding of the result to half
+    assert np.abs(got - want).max() < 2e-2 * max(1.0, np.abs(want).max())

@@ -1,19 +1,22 @@
-// Image convolution over pixel pairs: the stride-2 first layer of a network whose input has at most
-// four channels, once the graph executor has packed the image as [N][H][W/2][2 pixels x 4 channels]
-// (fp16).  The horizontal walk is then stride 1 over S pairs, every filter tap is one 16-byte chunk
-// and the whole K axis is R*S chunks, 18 for YOLOv5s' 6x6 window, 6 for MobileNetV3's 3x3.
+// Convolutions whose whole K axis is a handful of 16-byte chunks (fp16), in two forms:
+//  * the stride-2 first layer of a network whose input has at most four channels, once the graph
+//    executor has packed the image as [N][H][W/2][2 pixels x 4 channels]: the horizontal walk is
+//    stride 1 over S pairs, every filter tap is one chunk and K is R*S chunks, 18 for YOLOv5s'
+//    6x6 window, 6 for MobileNetV3's 3x3 (tests/Nets/Yolov5s.mlir, tests/Nets/MobileNetV3.mlir);
+//  * 1x1 convolutions over at most 144 channels in multiples of 8 (MobileNetV3's expansion and
+//    projection layers, 16..144 channels: none of them a multiple of the 64-byte K step of the
+//    pipelined kernel), with the residual add of an inverted-residual block.
 // Replaces the compiler's tiling of linalg.conv_2d_nchw_fchw for those layers
-// (src/nncv/compiler/Conversion/CodeGen/LlvmCpu/ModernTile.cpp:124-286; the layers are
-// tests/Nets/Yolov5s.mlir's and tests/Nets/MobileNetV3.mlir's first convolutions).
+// (src/nncv/compiler/Conversion/CodeGen/LlvmCpu/ModernTile.cpp:124-286).
 //
 // K is so short that a pipelined K walk through LDS only adds barriers.  A wave owns 64 pixels x 32
 // or 64 filters and needs no staging at all: lane (pixel l%32, chunk half l/32) of MFMA step kk reads
-// chunk 2*kk + l/32 of its pixel straight from global memory (half a wave reads 32 consecutive
-// pairs = 512 contiguous bytes), ALL steps requested back to back (one latency), the filters sit in
-// registers.  The epilogue (scale/shift, activation, one rounding) runs on the accumulators; the
-// halves pass through a small LDS tile only to leave as whole pixel rows, 16 bytes per lane.  With
-// 5-10 KB of LDS per wave tile the kernel runs at the occupancy its registers allow.  HBM bound:
-// the packed image is read once (window overlap is served by the caches), the result written once.
+// chunk 2*kk + l/32 of its pixel straight from global memory, ALL steps requested back to back (one
+// latency), the filters sit in registers.  The epilogue (scale/shift, residual, activation, one
+// rounding) runs on the accumulators; the halves pass through a small LDS tile only to leave as
+// whole pixel rows, 16 bytes per lane.  With 5-10 KB of LDS per wave tile the kernel runs at the
+// occupancy its registers allow.  HBM bound: input read once (window overlap and the re-reads of
+// further filter blocks are served by the caches), result written once.
 #include "mfma_tile.hpp"
 
 namespace nncv_hip {
@@ -24,52 +27,72 @@ namespace {
 constexpr unsigned kOOBc = 0x7fff0000u;  // byte offset beyond any buffer this kernel accepts
 }
 
-template <int R, int S, int NI>
-__global__ __launch_bounds__(256) void conv_pairs_kernel(const IgemmArgs a) {
-  constexpr int NCH = R * S, KST = NCH / 2;
+// PW = false: R x S window over pixel pairs (C = 8), KST = R*S/2.
+// PW = true : 1x1 window over C = 8*nch channels, nch <= 2*KST chunks (chunks past nch read as zero).
+// WV waves per workgroup, 64 pixels each (1 for small launches: more, smaller workgroups).
+template <bool PW, int R, int S, int KST, int NI, int WV>
+__global__ __launch_bounds__(64 * WV) void conv_pairs_kernel(const IgemmArgs a) {
   constexpr int TP = 64 * NI + 16;  // bytes per pixel row of the output tile: 32*NI halves + pad
-  static_assert(NCH % 2 == 0, "an MFMA step takes two chunks");
-  __shared__ __align__(16) unsigned char smem[4 * 64 * TP];
+  static_assert(PW || R * S == 2 * KST, "an MFMA step takes two chunks");
+  __shared__ __align__(16) unsigned char smem[WV * 64 * TP];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lrow = lane & 31, lchunk = lane >> 5;
   const int P = a.N * a.OH * a.OW;
   const int f0 = blockIdx.y * (32 * NI);
-  const int p0 = blockIdx.x * 256 + wave * 64;
+  const int p0 = blockIdx.x * (64 * WV) + wave * 64;
+  const int nch = PW ? a.C / 8 : R * S;  // chunks per pixel = chunks per filter row
   const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(a.in, a.in_bytes);
   const __amdgpu_buffer_rsrc_t rs_wt = make_rsrc(a.wt, a.wt_bytes);
 
   // ---- this lane's two pixels and its chunk of every step, requested back to back ----
-  int base[2], iy0[2], ix0[2];
-  const int ohow = a.OH * a.OW;
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int p = p0 + j * 32 + lrow;
-    const int n = p / ohow, rem = p - n * ohow;
-    const int oy = rem / a.OW, ox = rem - oy * a.OW;
-    iy0[j] = p < P ? oy * a.stride_h - a.pad_h : -(1 << 28);  // pixels past the end: never inside the image
-    ix0[j] = ox * a.stride_w - a.pad_w;
-    base[j] = (n * a.H + iy0[j]) * a.W + ix0[j];  // in pairs; only used when the tap is in bounds
-  }
   u32x4 b[KST][2];
+  if constexpr (PW) {
+    const int pix = a.pix_stride ? a.pix_stride : a.C;
 #pragma unroll
-  for (int kk = 0; kk < KST; ++kk) {
-    const int c = 2 * kk + lchunk, r = c / S, s = c - r * S;
+    for (int kk = 0; kk < KST; ++kk) {
+      const int c = 2 * kk + lchunk;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int p = p0 + j * 32 + lrow;
+        const bool ok = (p < P) & (c < nch);
+        b[kk][j] = __builtin_amdgcn_raw_buffer_load_b128(rs_in, ok ? (unsigned)(p * pix + c * 8) * 2u : kOOBc, 0, 0);
+      }
+    }
+  } else {
+    int base[2], iy0[2], ix0[2];
+    const int ohow = a.OH * a.OW;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const bool ok = ((unsigned)(iy0[j] + r) < (unsigned)a.H) & ((unsigned)(ix0[j] + s) < (unsigned)a.W);
-      b[kk][j] = __builtin_amdgcn_raw_buffer_load_b128(rs_in, ok ? (unsigned)(base[j] + r * a.W + s) * 16u : kOOBc, 0, 0);
+      const int p = p0 + j * 32 + lrow;
+      const int n = p / ohow, rem = p - n * ohow;
+      const int oy = rem / a.OW, ox = rem - oy * a.OW;
+      iy0[j] = p < P ? oy * a.stride_h - a.pad_h : -(1 << 28);  // pixels past the end: never inside the image
+      ix0[j] = ox * a.stride_w - a.pad_w;
+      base[j] = (n * a.H + iy0[j]) * a.W + ix0[j];  // in pairs; only used when the tap is in bounds
+    }
+#pragma unroll
+    for (int kk = 0; kk < KST; ++kk) {
+      const int c = 2 * kk + lchunk, r = c / S, s = c - r * S;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const bool ok = ((unsigned)(iy0[j] + r) < (unsigned)a.H) & ((unsigned)(ix0[j] + s) < (unsigned)a.W);
+        b[kk][j] = __builtin_amdgcn_raw_buffer_load_b128(rs_in, ok ? (unsigned)(base[j] + r * a.W + s) * 16u : kOOBc, 0, 0);
+      }
     }
   }
-  // ---- the filters: row f is R*S chunks; lane (filter l%32, chunk half l/32) of step kk holds
+  // ---- the filters: row f is nch chunks; lane (filter l%32, chunk half l/32) of step kk holds
   //      chunk 2*kk + l/32.  Rows past the tensor read as zero. ----
   u32x4 w[KST][NI];
 #pragma unroll
   for (int kk = 0; kk < KST; ++kk)
 #pragma unroll
-    for (int i = 0; i < NI; ++i)
-      w[kk][i] = __builtin_amdgcn_raw_buffer_load_b128(rs_wt, (unsigned)(((f0 + i * 32 + lrow) * NCH + 2 * kk + lchunk) * 16), 0, 0);
-  // scale/shift of this lane's accumulator channels f0 + 32 i + 8 q + 4 (l/32) .. + 3
+    for (int i = 0; i < NI; ++i) {
+      const int c = 2 * kk + lchunk;
+      w[kk][i] = __builtin_amdgcn_raw_buffer_load_b128(rs_wt, c < nch ? (unsigned)(((f0 + i * 32 + lrow) * nch + c) * 16) : kOOBc, 0, 0);
+    }
+  // scale/shift of this lane's accumulator channels f0 + 32 i + 8 q + 4 (l/32) .. + 3, and the
+  // residual values at the same places (element offsets; rows past the end read element 0)
   floatx4 sc[NI][4], sh[NI][4];
 #pragma unroll
   for (int i = 0; i < NI; ++i)
@@ -80,6 +103,20 @@ __global__ __launch_bounds__(256) void conv_pairs_kernel(const IgemmArgs a) {
       sc[i][q] = (a.scale && fin) ? *reinterpret_cast<const floatx4*>(a.scale + f) : floatx4{1.f, 1.f, 1.f, 1.f};
       sh[i][q] = (a.shift && fin) ? *reinterpret_cast<const floatx4*>(a.shift + f) : floatx4{0.f, 0.f, 0.f, 0.f};
     }
+  const half_t* res = static_cast<const half_t*>(a.residual);
+  half4 rv[NI][2][4];
+  if (res) {
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int p = p0 + j * 32 + lrow, f = f0 + i * 32 + 8 * q + 4 * lchunk;
+          const long long off = (p < P && f < a.F) ? (long long)p * a.ldo + f : 0;
+          rv[i][j][q] = *reinterpret_cast<const half4*>(res + off);
+        }
+  }
 
   floatx16 acc[NI][2];
 #pragma unroll
@@ -98,6 +135,7 @@ __global__ __launch_bounds__(256) void conv_pairs_kernel(const IgemmArgs a) {
   // ---- epilogue on the accumulators, halves to this wave's tile [pixel][channel] ----
   unsigned char* tile = smem + wave * (64 * TP);
   const int act = a.relu & 0xff;
+  const bool res_after = a.relu & kActResidualAfter;  // y = act(conv) + residual instead of act(conv + residual)
 #pragma unroll
   for (int i = 0; i < NI; ++i)
 #pragma unroll
@@ -107,7 +145,15 @@ __global__ __launch_bounds__(256) void conv_pairs_kernel(const IgemmArgs a) {
         float y[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) y[e] = acc[i][j][4 * q + e] * sc[i][q][e] + sh[i][q][e];
+        if (res && !res_after) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) y[e] += (float)rv[i][j][q][e];
+        }
         act_apply_n<true>(y, act);
+        if (res && res_after) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) y[e] += (float)rv[i][j][q][e];
+        }
         half4 h;
 #pragma unroll
         for (int e = 0; e < 4; ++e) h[e] = (half_t)y[e];
@@ -128,31 +174,57 @@ __global__ __launch_bounds__(256) void conv_pairs_kernel(const IgemmArgs a) {
 
 bool conv_pairs_applicable(const IgemmArgs& a, int in_dt, int out_dt) {
   static const bool off = getenv("NNCV_HIP_NO_CONV_PAIRS") != nullptr;
-  const bool window = (a.R == 6 && a.S == 3) || (a.R == 3 && a.S == 2);
+  static const bool off_pw = getenv("NNCV_HIP_NO_CONV_SHORTK") != nullptr;
+  const int pix = a.pix_stride ? a.pix_stride : a.C;
   const long long P = (long long)a.N * a.OH * a.OW;
-  return !off && in_dt == kF16 && out_dt == kF16 && window && a.C == 8 && (a.pix_stride == 0 || a.pix_stride == 8) && a.batch == 1 &&
-         a.aux_f0 == 0 && a.residual == nullptr && (a.relu & ~0xff) == 0 && a.F % 8 == 0 && a.F <= 64 && a.ldo % 8 == 0 && a.ldo >= a.F && P * a.ldo < (1ll << 31) &&
-         (long long)a.N * a.H * a.W * 16 < (long long)kOOBc && a.in_bytes > 0 && a.in_bytes < kOOBc && a.wt_bytes > 0;
+  const bool common = in_dt == kF16 && out_dt == kF16 && a.batch == 1 && a.aux_f0 == 0 && a.F % 8 == 0 && a.ldo % 8 == 0 && a.ldo >= a.F &&
+                      P * a.ldo < (1ll << 31) && a.in_bytes > 0 && a.in_bytes < kOOBc && a.wt_bytes > 0 && a.wt_bytes < kOOBc &&
+                      (a.relu & ~(0xff | kActResidualAfter)) == 0;
+  if (!common) return false;
+  const bool window = (a.R == 6 && a.S == 3) || (a.R == 3 && a.S == 2);
+  if (window)
+    return !off && a.C == 8 && pix == 8 && a.F <= 64 && (long long)a.N * a.H * a.W * 16 < (long long)kOOBc;
+  // 1x1, stride 1, no padding: the output pixel is the input pixel
+  return !off_pw && a.R == 1 && a.S == 1 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 0 && a.pad_w == 0 && a.OH == a.H &&
+         a.OW == a.W && a.C % 8 == 0 && a.C % 32 != 0 && a.C <= 144 && pix % 8 == 0 && P * pix * 2 < (long long)kOOBc;
 }
 
-template <int R, int S, int NI>
+template <bool PW, int R, int S, int KST, int NI>
 static void launch_pairs_cfg(const IgemmArgs& a, const char* tag, hipStream_t s) {
-  auto kern = conv_pairs_kernel<R, S, NI>;
   const long long P = (long long)a.N * a.OH * a.OW;
-  const double flops = a.alg_flops > 0 ? a.alg_flops : 2.0 * P * a.F * R * S * 8.0;
-  const double bytes = 2.0 * ((double)a.N * a.H * a.W * 8 + (double)a.F * R * S * 8 + (double)P * a.F * (a.residual ? 2 : 1));
+  const double flops = a.alg_flops > 0 ? a.alg_flops : 2.0 * P * a.F * a.R * a.S * a.C;
+  const double bytes = 2.0 * ((double)a.N * a.H * a.W * a.C + (double)a.F * a.R * a.S * a.C + (double)P * a.F * (a.residual ? 2 : 1));
   ProfScope prof(tag, flops, bytes, s);
-  dim3 grid((unsigned)((P + 255) / 256), (unsigned)((a.F + 32 * NI - 1) / (32 * NI)));
-  hipLaunchKernelGGL(kern, grid, dim3(256), 0, s, a);
+  const unsigned gy = (unsigned)((a.F + 32 * NI - 1) / (32 * NI));
+  // fewer four-wave workgroups than CUs: one wave per workgroup instead
+  if ((P + 255) / 256 * gy < 256)
+    hipLaunchKernelGGL((conv_pairs_kernel<PW, R, S, KST, NI, 1>), dim3((unsigned)((P + 63) / 64), gy), dim3(64), 0, s, a);
+  else
+    hipLaunchKernelGGL((conv_pairs_kernel<PW, R, S, KST, NI, 4>), dim3((unsigned)((P + 255) / 256), gy), dim3(256), 0, s, a);
 }
 
 void launch_conv_pairs(const IgemmArgs& a, hipStream_t s) {
   if (a.R == 6) {
-    if (a.F > 32) launch_pairs_cfg<6, 3, 2>(a, "conv_pairs<f16,6x3,64>", s);
-    else launch_pairs_cfg<6, 3, 1>(a, "conv_pairs<f16,6x3,32>", s);
+    if (a.F > 32) launch_pairs_cfg<false, 6, 3, 9, 2>(a, "conv_pairs<f16,6x3,64>", s);
+    else launch_pairs_cfg<false, 6, 3, 9, 1>(a, "conv_pairs<f16,6x3,32>", s);
+  } else if (a.R == 3) {
+    if (a.F > 32) launch_pairs_cfg<false, 3, 2, 3, 2>(a, "conv_pairs<f16,3x2,64>", s);
+    else launch_pairs_cfg<false, 3, 2, 3, 1>(a, "conv_pairs<f16,3x2,32>", s);
   } else {
-    if (a.F > 32) launch_pairs_cfg<3, 2, 2>(a, "conv_pairs<f16,3x2,64>", s);
-    else launch_pairs_cfg<3, 2, 1>(a, "conv_pairs<f16,3x2,32>", s);
+    // K steps in registers: 1 (16 channels), 3 (..48), 6 (..96), 9 (..144); 64 filters per wave tile
+    // while the registers allow it
+    const int kst = (a.C / 8 + 1) / 2;
+    if (kst <= 1) {
+      if (a.F > 32) launch_pairs_cfg<true, 1, 1, 1, 2>(a, "conv1x1_shortk<f16,16,64>", s);
+      else launch_pairs_cfg<true, 1, 1, 1, 1>(a, "conv1x1_shortk<f16,16,32>", s);
+    } else if (kst <= 3) {
+      if (a.F > 32) launch_pairs_cfg<true, 1, 1, 3, 2>(a, "conv1x1_shortk<f16,48,64>", s);
+      else launch_pairs_cfg<true, 1, 1, 3, 1>(a, "conv1x1_shortk<f16,48,32>", s);
+    } else if (kst <= 6) {
+      launch_pairs_cfg<true, 1, 1, 6, 1>(a, "conv1x1_shortk<f16,96,32>", s);
+    } else {
+      launch_pairs_cfg<true, 1, 1, 9, 1>(a, "conv1x1_shortk<f16,144,32>", s);
+    }
   }
   NNCV_HIP_CHECK(hipGetLastError());
 }

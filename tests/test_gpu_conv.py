@@ -273,3 +273,40 @@ def test_random_patch_kernel_layers(dt):
     print("routes", routes, flush=True)
     patch = sum(v for k, v in routes.items() if k.startswith("conv3x3"))
     assert patch >= 0.8 * sum(routes.values()), routes
+
+
+@pytest.mark.parametrize("C,F,N,H,W,act,res", [
+    (16, 72, 2, 56, 56, abi.ACT_RELU, False),       # MobileNetV3 expansion: one K step, two 64-filter blocks
+    (16, 16, 3, 9, 7, abi.ACT_NONE, True),          # projection with the block's residual, ragged pixel count
+    (24, 88, 2, 28, 28, abi.ACT_RELU, False),       # 3 chunks: the second step's upper half is padding
+    (40, 240, 1, 14, 14, abi.ACT_HARDSWISH, False),
+    (48, 288, 2, 14, 14, abi.ACT_HARDSWISH, False),
+    (72, 24, 2, 28, 28, abi.ACT_NONE, False),
+    (88, 24, 2, 28, 28, abi.ACT_NONE, True),
+    (120, 48, 2, 14, 14, abi.ACT_NONE, False),
+    (144, 48, 3, 14, 14, abi.ACT_SILU, True),       # 18 chunks, activation before ... the residual is added first here
+    (136, 40, 1, 5, 5, abi.ACT_RELU, True),         # 17 chunks: odd, the last step is half padding
+])
+def test_fp16_1x1_convolutions_with_a_short_k_axis(C, F, N, H, W, act, res):
+    """1x1 layers whose channel count is a multiple of 8 but not of 32, up to 144: the kernel that holds the whole
+    K axis in registers (`conv1x1_shortk`), against the oracle, with the route checked."""
+    x = synth.round_fp16(synth.normal(7600 + C, (N, C, H, W)))
+    w = synth.round_fp16(synth.normal(7601 + C, (F, C, 1, 1), std=float(np.sqrt(2.0 / C))))
+    bn = tuple(synth.round_fp16(b) for b in bn_params(7602 + C, F))
+    r = synth.round_fp16(synth.normal(7606 + C, (N, F, H, W))) if res else None
+    y = oracle.batchnorm(oracle.conv2d_nchw_fchw(x, w, 1), *bn)
+    if r is not None:
+        y = (y + r).astype(np.float32)
+    want = oracle.ACTIVATIONS[act](y)
+    conv = Conv(abi.F16, w, 1, 0, bn=bn, relu=act, algo=abi.ALGO_IGEMM)
+    rd = dev(nhwc(r), abi.F16) if r is not None else None
+    print("1x1 short K", (C, F, N, H, W), act, res, flush=True)
+    abi.profile_enable(True)
+    abi.profile_report()
+    got = nchw(host(conv(dev(nhwc(x), abi.F16), abi.NHWC, residual=rd)))
+    tags = abi.profile_report()
+    abi.profile_enable(False)
+    conv.close()
+    assert any(t.startswith("conv1x1_shortk<f16") for t in tags), sorted(tags)
+    assert rel_l2(got, want) < 2e-3
+    assert np.abs(got - want).max() < 2e-2 * max(1.0, np.abs(want).max())

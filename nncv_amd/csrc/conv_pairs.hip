@@ -30,7 +30,8 @@ constexpr unsigned kOOBc = 0x7fff0000u;  // byte offset beyond any buffer this k
 // PW = false: R x S window over pixel pairs (C = 8), KST = R*S/2.
 // PW = true : 1x1 window over C = 8*nch channels, nch <= 2*KST chunks (chunks past nch read as zero).
 // WV waves per workgroup, 64 pixels each (1 for small launches: more, smaller workgroups).
-template <bool PW, int R, int S, int KST, int NI, int WV>
+// RES: the launch has a residual input (instances without one carry no registers or code for it).
+template <bool PW, int R, int S, int KST, int NI, int WV, bool RES>
 __global__ __launch_bounds__(64 * WV) void conv_pairs_kernel(const IgemmArgs a) {
   constexpr int TP = 64 * NI + 16;  // bytes per pixel row of the output tile: 32*NI halves + pad
   static_assert(PW || R * S == 2 * KST, "an MFMA step takes two chunks");
@@ -105,7 +106,7 @@ __global__ __launch_bounds__(64 * WV) void conv_pairs_kernel(const IgemmArgs a) 
     }
   const half_t* res = static_cast<const half_t*>(a.residual);
   half4 rv[NI][2][4];
-  if (res) {
+  if constexpr (RES) {
 #pragma unroll
     for (int i = 0; i < NI; ++i)
 #pragma unroll
@@ -145,12 +146,12 @@ __global__ __launch_bounds__(64 * WV) void conv_pairs_kernel(const IgemmArgs a) 
         float y[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) y[e] = acc[i][j][4 * q + e] * sc[i][q][e] + sh[i][q][e];
-        if (res && !res_after) {
+        if (RES && !res_after) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) y[e] += (float)rv[i][j][q][e];
         }
         act_apply_n<true>(y, act);
-        if (res && res_after) {
+        if (RES && res_after) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) y[e] += (float)rv[i][j][q][e];
         }
@@ -183,7 +184,8 @@ bool conv_pairs_applicable(const IgemmArgs& a, int in_dt, int out_dt) {
   if (!common) return false;
   const bool window = (a.R == 6 && a.S == 3) || (a.R == 3 && a.S == 2);
   if (window)
-    return !off && a.C == 8 && pix == 8 && a.F <= 64 && (long long)a.N * a.H * a.W * 16 < (long long)kOOBc;
+    return !off && a.C == 8 && pix == 8 && a.F <= 64 && a.residual == nullptr && (a.relu & ~0xff) == 0 &&
+           (long long)a.N * a.H * a.W * 16 < (long long)kOOBc;
   // 1x1, stride 1, no padding: the output pixel is the input pixel
   return !off_pw && a.R == 1 && a.S == 1 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 0 && a.pad_w == 0 && a.OH == a.H &&
          a.OW == a.W && a.C % 8 == 0 && a.C % 32 != 0 && a.C <= 144 && pix % 8 == 0 && P * pix * 2 < (long long)kOOBc;
@@ -197,10 +199,17 @@ static void launch_pairs_cfg(const IgemmArgs& a, const char* tag, hipStream_t s)
   ProfScope prof(tag, flops, bytes, s);
   const unsigned gy = (unsigned)((a.F + 32 * NI - 1) / (32 * NI));
   // fewer four-wave workgroups than CUs: one wave per workgroup instead
-  if ((P + 255) / 256 * gy < 256)
-    hipLaunchKernelGGL((conv_pairs_kernel<PW, R, S, KST, NI, 1>), dim3((unsigned)((P + 63) / 64), gy), dim3(64), 0, s, a);
-  else
-    hipLaunchKernelGGL((conv_pairs_kernel<PW, R, S, KST, NI, 4>), dim3((unsigned)((P + 255) / 256), gy), dim3(256), 0, s, a);
+  const bool small = (P + 255) / 256 * gy < 256;
+  const dim3 grid(small ? (unsigned)((P + 63) / 64) : (unsigned)((P + 255) / 256), gy), block(small ? 64 : 256);
+  if constexpr (PW) {
+    if (a.residual && small) hipLaunchKernelGGL((conv_pairs_kernel<PW, R, S, KST, NI, 1, true>), grid, block, 0, s, a);
+    else if (a.residual) hipLaunchKernelGGL((conv_pairs_kernel<PW, R, S, KST, NI, 4, true>), grid, block, 0, s, a);
+    else if (small) hipLaunchKernelGGL((conv_pairs_kernel<PW, R, S, KST, NI, 1, false>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((conv_pairs_kernel<PW, R, S, KST, NI, 4, false>), grid, block, 0, s, a);
+  } else {  // the image layers have no residual input (conv_pairs_applicable)
+    if (small) hipLaunchKernelGGL((conv_pairs_kernel<PW, R, S, KST, NI, 1, false>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((conv_pairs_kernel<PW, R, S, KST, NI, 4, false>), grid, block, 0, s, a);
+  }
 }
 
 void launch_conv_pairs(const IgemmArgs& a, hipStream_t s) {

@@ -186,9 +186,12 @@ bool conv_pairs_applicable(const IgemmArgs& a, int in_dt, int out_dt) {
   if (window)
     return !off && a.C == 8 && pix == 8 && a.F <= 64 && a.residual == nullptr && (a.relu & ~0xff) == 0 &&
            (long long)a.N * a.H * a.W * 16 < (long long)kOOBc;
-  // 1x1, stride 1, no padding: the output pixel is the input pixel
+  // 1x1, stride 1, no padding: the output pixel is the input pixel.  Channel counts that the pipelined
+  // kernel takes as well (multiples of 32) come here only for small launches, where its barriers per K
+  // step are all latency (MobileNetV3's 96-channel layers at 14x14 and 7x7: 0.449 -> 0.444 ms per
+  // batch of 32); on YOLOv5s' large 1x1 layers it is the faster one (1.27 against 1.32 ms).
   return !off_pw && a.R == 1 && a.S == 1 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 0 && a.pad_w == 0 && a.OH == a.H &&
-         a.OW == a.W && a.C % 8 == 0 && a.C % 32 != 0 && a.C <= 144 && pix % 8 == 0 && P * pix * 2 < (long long)kOOBc;
+         a.OW == a.W && a.C % 8 == 0 && (a.C % 32 != 0 || P <= 8192) && a.C <= 144 && pix % 8 == 0 && P * pix * 2 < (long long)kOOBc;
 }
 
 template <bool PW, int R, int S, int KST, int NI>

@@ -579,6 +579,50 @@ __global__ __launch_bounds__(256) void yolo_detect_kernel(const DetectArgs a) {
   a.out[((long long)n * a.boxes_total + a.box0 + (long long)an * a.H * a.W) * a.F + i] = o;
 }
 
+// The same with four consecutive values per thread and one 16-byte store (the launcher uses it when
+// H*W*F is a multiple of 4 and the level's first output value is 16-byte aligned): a quarter of the
+// index arithmetic and store instructions per value.
+template <typename T>
+__global__ __launch_bounds__(256) void yolo_detect4_kernel(const DetectArgs a) {
+  const int n = blockIdx.y / a.A, an = blockIdx.y - n * a.A;
+  const int i = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  const int HWF = a.H * a.W * a.F;
+  if (i >= HWF) return;
+  int pix = (int)((float)i * a.inv_f), k = i - pix * a.F;
+  if (k >= a.F) { ++pix; k -= a.F; }
+  if (k < 0) { --pix; k += a.F; }
+  const T* head = static_cast<const T*>(a.head) + (long long)n * a.H * a.W * a.ldc + an * a.F;
+  float v[4];
+  int kk[4], pp[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    kk[e] = k;
+    pp[e] = pix;
+    v[e] = (float)head[(long long)pix * a.ldc + k];
+    if (++k == a.F) { k = 0; ++pix; }
+  }
+  float o[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float sg = sigmoid_fast(v[e]);
+    o[e] = sg;
+    if (kk[e] < 4) {
+      int y = (int)((float)pp[e] * a.inv_w), x = pp[e] - y * a.W;
+      if (x >= a.W) { ++y; x -= a.W; }
+      if (x < 0) { --y; x += a.W; }
+      if (kk[e] < 2) {
+        const float g = (float)(kk[e] == 0 ? x : y) - 0.5f;
+        o[e] = (sg * 2.0f + g) * a.stride;
+      } else {
+        const float t = sg * 2.0f;
+        o[e] = (t * t) * a.anchor_wh[an * 2 + (kk[e] - 2)];
+      }
+    }
+  }
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  *reinterpret_cast<f4*>(a.out + ((long long)n * a.boxes_total + a.box0 + (long long)an * a.H * a.W) * a.F + i) = f4{o[0], o[1], o[2], o[3]};
+}
+
 void launch_yolo_detect(const DetectArgs& a, int dt, hipStream_t s) {
   NNCV_REQUIRE(a.A >= 1 && a.A <= 4 && a.F >= 5 && a.A * a.F <= a.ldc && a.N >= 1 && a.H >= 1 && a.W >= 1, "yolo_detect: bad shape");
   NNCV_REQUIRE((long long)a.H * a.W * a.F < (1ll << 24) && (long long)a.N * a.A <= 65535, "yolo_detect: level too large");
@@ -587,6 +631,19 @@ void launch_yolo_detect(const DetectArgs& a, int dt, hipStream_t s) {
   b.inv_w = 1.0f / (float)a.W;
   const long long work = (long long)a.N * a.A * a.H * a.W * a.F;
   ProfScope prof("yolo_detect", 0.0, (double)work * (dtype_size(dt) + 4.0), s);
+  // four values per thread when every (image, anchor) block of the output starts on a 16-byte boundary
+  const long long hwf = (long long)a.H * a.W * a.F;
+  const bool vec4 = hwf % 4 == 0 && (a.boxes_total * a.F) % 4 == 0 && (a.box0 * a.F) % 4 == 0 &&
+                    reinterpret_cast<uintptr_t>(a.out) % 16 == 0;
+  if (vec4) {
+    dim3 grid4((unsigned)((hwf / 4 + 255) / 256), (unsigned)(a.N * a.A));
+    if (dt == kF16)
+      hipLaunchKernelGGL((yolo_detect4_kernel<half_t>), grid4, dim3(256), 0, s, b);
+    else
+      hipLaunchKernelGGL((yolo_detect4_kernel<float>), grid4, dim3(256), 0, s, b);
+    NNCV_HIP_CHECK(hipGetLastError());
+    return;
+  }
   dim3 grid((unsigned)(((long long)a.H * a.W * a.F + 255) / 256), (unsigned)(a.N * a.A));
   if (dt == kF16)
     hipLaunchKernelGGL((yolo_detect_kernel<half_t>), grid, dim3(256), 0, s, b);

@@ -297,6 +297,11 @@ void launch_concat_slice(const void* x, void* out, int dt, long long P, int C, i
 // nearest-neighbour 2x up-sampling [N,H,W,C] -> [N,2H,2W,C], written at channel offset c0 of pitch ldo
 void launch_upsample2x(const void* x, void* out, int dt, int N, int H, int W, int C, int ldo, int c0, hipStream_t s, int ldi = 0);
 // max-pool K x K, any stride / padding (-inf halo), NHWC
+// y1 = m(x), y2 = m(y1), y3 = m(y2) with m = max-pool 5x5 stride 1 pad 2, all three kept, in one launch
+// (maps of at most 1600 pixels); ld*: elements between pixels of each tensor.
+bool maxpool5_chain3_applicable(int dt, int H, int W, int C);
+void launch_maxpool5_chain3(const void* in, void* o1, void* o2, void* o3, int dt, int N, int H, int W, int C, int ldi, int ld1, int ld2,
+                            int ld3, hipStream_t s);
 void launch_maxpool_nhwc(const void* in, void* out, int dt, int N, int H, int W, int C, int K, int stride, int pad,
                          hipStream_t s, int ldi = 0, int ldo = 0);  // pixel pitches of in / out, 0 = C
 // YOLOv5 Detect decode of one level: head [N,H,W,ldc] (A*F used channels, anchor-major) ->

@@ -542,6 +542,84 @@ void launch_maxpool_nhwc(const void* in, void* out, int dt, int N, int H, int W,
 }
 
 // ---------------------------------------------------------------------------------------------
+// Three 5x5 stride-1 pad-2 max-pools in a row, each result kept (YOLOv5's SPPF block,
+// Yolov5s.mlir: y1 = m(x), y2 = m(y1), y3 = m(y2), all four concatenated): one launch instead of
+// three.  A workgroup owns one image x one 16-byte channel vector: the H*W map sits in LDS, each
+// stage reads its 25 neighbours there (the -inf halo is a skipped tap) and writes its result both
+// to memory and to the other LDS buffer.  The maps are 20x20 for a 640x640 input, so the three
+// stand-alone launches were nothing but latency (16 us each for 3 MB).
+// ---------------------------------------------------------------------------------------------
+constexpr int kPoolChainMaxHW = 1600;
+
+template <typename T>
+__global__ __launch_bounds__(256) void maxpool5_chain3_kernel(const T* __restrict__ in, T* __restrict__ o1, T* __restrict__ o2,
+                                                              T* __restrict__ o3, int H, int W, int CG, int ldi, int ld1, int ld2,
+                                                              int ld3) {
+  constexpr int VN = V16<T>::n;
+  typedef typename V16<T>::type V;
+  __shared__ V buf[2][kPoolChainMaxHW];
+  const int n = blockIdx.x / CG, cg = blockIdx.x - n * CG;
+  const int HW = H * W, tid = threadIdx.x;
+  const float inv_w = 1.0f / (float)W;
+  in += (long long)n * HW * ldi + cg * VN;
+  for (int p = tid; p < HW; p += 256) buf[0][p] = *reinterpret_cast<const V*>(in + (long long)p * ldi);
+  __syncthreads();
+#pragma unroll
+  for (int stage = 0; stage < 3; ++stage) {
+    const V* src = buf[stage & 1];
+    V* dst = buf[(stage + 1) & 1];
+    T* out = (stage == 0 ? o1 : stage == 1 ? o2 : o3) + ((long long)n * HW * (stage == 0 ? ld1 : stage == 1 ? ld2 : ld3) + cg * VN);
+    const int ldo = stage == 0 ? ld1 : stage == 1 ? ld2 : ld3;
+    for (int p = tid; p < HW; p += 256) {
+      int y = (int)((float)p * inv_w), x = p - y * W;  // exact for p < 2^24 after the correction
+      if (x >= W) { ++y; x -= W; }
+      if (x < 0) { --y; x += W; }
+      float m[VN];
+#pragma unroll
+      for (int e = 0; e < VN; ++e) m[e] = -INFINITY;
+#pragma unroll
+      for (int r = -2; r <= 2; ++r)
+#pragma unroll
+        for (int q = -2; q <= 2; ++q) {
+          const bool ok = ((unsigned)(y + r) < (unsigned)H) & ((unsigned)(x + q) < (unsigned)W);
+          const V v = src[ok ? p + r * W + q : p];  // outside the map: the centre again, which changes nothing
+#pragma unroll
+          for (int e = 0; e < VN; ++e) m[e] = max_nan(m[e], (float)v[e]);
+        }
+      V o;
+#pragma unroll
+      for (int e = 0; e < VN; ++e) o[e] = (T)m[e];
+      dst[p] = o;
+      *reinterpret_cast<V*>(out + (long long)p * ldo) = o;
+    }
+    __syncthreads();
+  }
+}
+
+bool maxpool5_chain3_applicable(int dt, int H, int W, int C) {
+  static const bool off = getenv("NNCV_HIP_NO_POOL_CHAIN") != nullptr;
+  const int vn = dt == kF16 ? 8 : 4;
+  return !off && H >= 1 && W >= 1 && H * W <= kPoolChainMaxHW && C % vn == 0;
+}
+
+void launch_maxpool5_chain3(const void* in, void* o1, void* o2, void* o3, int dt, int N, int H, int W, int C, int ldi, int ld1, int ld2,
+                            int ld3, hipStream_t s) {
+  const int vn = dt == kF16 ? 8 : 4;
+  NNCV_REQUIRE(maxpool5_chain3_applicable(dt, H, W, C) && ldi % vn == 0 && ld1 % vn == 0 && ld2 % vn == 0 && ld3 % vn == 0 &&
+                   ldi >= C && ld1 >= C && ld2 >= C && ld3 >= C && (long long)N * (C / vn) < (1ll << 31),
+               "maxpool chain: shape not covered");
+  ProfScope prof("maxpool5_chain3", 0.0, (double)dtype_size(dt) * N * C * 4.0 * H * W, s);
+  const dim3 grid((unsigned)((long long)N * (C / vn)));
+  if (dt == kF16)
+    hipLaunchKernelGGL((maxpool5_chain3_kernel<half_t>), grid, dim3(256), 0, s, (const half_t*)in, (half_t*)o1, (half_t*)o2, (half_t*)o3,
+                       H, W, C / vn, ldi, ld1, ld2, ld3);
+  else
+    hipLaunchKernelGGL((maxpool5_chain3_kernel<float>), grid, dim3(256), 0, s, (const float*)in, (float*)o1, (float*)o2, (float*)o3, H, W,
+                       C / vn, ldi, ld1, ld2, ld3);
+  NNCV_HIP_CHECK(hipGetLastError());
+}
+
+// ---------------------------------------------------------------------------------------------
 // YOLOv5 Detect decode, one level (Yolov5s.mlir:1348-1448): expand [N,A*F,H,W] to [N,A,H,W,F],
 // sigmoid, xy = (2 s + (x, y) - 0.5) * stride, wh = (2 s)^2 * anchor (powf(., 2) is the square),
 // everything else the sigmoid itself; boxes ordered (anchor, y, x).  One thread per output value,

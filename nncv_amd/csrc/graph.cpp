@@ -388,6 +388,19 @@ const Graph::Plan& Graph::plan_of(int N, int H, int W) const {
     life[t] = TensorLife{i + 1, std::max(i + 1, last_use_[t] + 1), (size_t)N * d.H * d.W * d.C * es, 0};
     if (nodes_[i].op.kind == NNCV_HIP_OP_YOLO_DETECT) life[t].bytes = 256;  // written straight to the caller's buffer
   }
+  // three chained 5x5 stride-1 pad-2 max-pools may run as one launch that writes all three results at
+  // the first one's step (forward()): the later two are live from there
+  {
+    auto pool5 = [&](int k, int in) {
+      return k < n && !nodes_[k].skip && nodes_[k].op.kind == NNCV_HIP_OP_MAXPOOL && nodes_[k].op.K == 5 && nodes_[k].op.stride == 1 &&
+             nodes_[k].op.pad == 2 && (in < 0 || nodes_[k].op.in[0] == in);
+    };
+    for (int i = 0; i + 2 < n; ++i)
+      if (pool5(i, -1) && pool5(i + 1, nodes_[i].op.out) && pool5(i + 2, nodes_[i + 1].op.out)) {
+        life[nodes_[i + 1].op.out].first_op = i + 1;
+        life[nodes_[i + 2].op.out].first_op = i + 1;
+      }
+  }
   life[nodes_[n - 1].op.out].last_op = n + 1;
   // a tensor that lives inside a concatenated one has no memory of its own; the concatenated
   // tensor is live from its first such input to the last reader of any of them
@@ -492,10 +505,23 @@ void Graph::forward(const void* src, int N, int H, int W, float* out, void* ws, 
         launch_dwconv(d, dt_, s);
         break;
       }
-      case NNCV_HIP_OP_MAXPOOL:
+      case NNCV_HIP_OP_MAXPOOL: {
+        // three 5x5 stride-1 pad-2 pools in a row (SPPF): one launch that keeps all three results
+        auto pool5 = [&](size_t k, int in) {
+          return k < nodes_.size() && !nodes_[k].skip && nodes_[k].op.kind == NNCV_HIP_OP_MAXPOOL && nodes_[k].op.K == 5 &&
+                 nodes_[k].op.stride == 1 && nodes_[k].op.pad == 2 && (in < 0 || nodes_[k].op.in[0] == in);
+        };
+        if (pool5(i, -1) && pool5(i + 1, op.out) && pool5(i + 2, nodes_[i + 1].op.out) && maxpool5_chain3_applicable(dt_, a.H, a.W, a.C)) {
+          const int t2 = nodes_[i + 1].op.out, t3 = nodes_[i + 2].op.out;
+          launch_maxpool5_chain3(at(op.in[0]), at(op.out), at(t2), at(t3), dt_, N, a.H, a.W, a.C, pitch(op.in[0]), pitch(op.out),
+                                 pitch(t2), pitch(t3), s);
+          i += 2;
+          break;
+        }
         launch_maxpool_nhwc(at(op.in[0]), at(op.out), dt_, N, a.H, a.W, a.C, op.K, op.stride, op.pad, s, pitch(op.in[0]),
                             pitch(op.out));
         break;
+      }
       case NNCV_HIP_OP_GAVGPOOL:
         launch_global_avgpool_nhwc(at(op.in[0]), at(op.out), dt_, N, a.H * a.W, a.C, s);
         break;

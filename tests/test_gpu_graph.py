@@ -458,3 +458,55 @@ def test_fp16_image_convolution_over_pixel_pairs(k, pad, F, act, shape):
     assert got.shape == want.shape
     assert rel_l2(got, want) < 2e-3  # one layer: only the rounding of the result to half
     assert np.abs(got - want).max() < 2e-2 * max(1.0, np.abs(want).max())
+
+
+@pytest.mark.parametrize("dt", [abi.F32, abi.F16])
+@pytest.mark.parametrize("shape,concat", [((2, 3, 20, 20), True), ((3, 3, 7, 13), True), ((1, 3, 40, 40), False), ((1, 3, 41, 40), True)])
+def test_three_chained_5x5_max_pools_run_as_one_launch(dt, shape, concat):
+    """SPPF: y1 = m(x), y2 = m(y1), y3 = m(y2), concatenated with x (or only y3 kept).  Maps of at most 1600 pixels take
+    the fused kernel, larger ones three launches; both must equal the evaluator exactly (max of copies of the input)."""
+    C = 16
+    sizes, ops = [], []
+
+    def take(n):
+        off = sum(sizes)
+        sizes.append(n)
+        return off
+
+    w = take(C * 3)
+    ops.append(abi.graph_op(abi.OP_CONV, [0, -1], 1, F=C, K=1, stride=1, pad=0, act=abi.ACT_NONE, w=w, bias=take(C)))
+    ops.append(abi.graph_op(abi.OP_MAXPOOL, [1], 2, K=5, stride=1, pad=2))
+    ops.append(abi.graph_op(abi.OP_MAXPOOL, [2], 3, K=5, stride=1, pad=2))
+    ops.append(abi.graph_op(abi.OP_MAXPOOL, [3], 4, K=5, stride=1, pad=2))
+    if concat:
+        ops.append(abi.graph_op(abi.OP_CONCAT, [1, 2, 3, 4], 5))
+    blob = synth.normal(7950, (sum(sizes),), std=0.5)
+    x = synth.normal(7951, shape)
+    if dt == abi.F16:
+        blob, x = r16(blob), r16(x)
+    g = Graph(ops, 3, blob, dt)
+    abi.profile_enable(True)
+    abi.profile_report()
+    got = host(g(dev(x, dt)))
+    tags = abi.profile_report()
+    abi.profile_enable(False)
+    want = oracle.run_graph(ops, x, blob, 3)
+    fused = shape[2] * shape[3] <= 1600
+    assert ("maxpool5_chain3" in tags) == fused and ("maxpool" in tags) == (not fused), sorted(tags)
+    assert got.shape == want.shape
+    if dt == abi.F32:
+        assert max_rel(got, want) < FP32_MAX_REL
+    else:
+        assert rel_l2(got, want) < 2e-3
+    # the pools themselves are exact: every pooled channel must be the maximum of the unpooled ones it covers
+    if concat:
+        y0, y1 = got[:, :C], got[:, C:2 * C]
+        assert np.array_equal(y1, oracle.maxpool_nchw(y0, 5, 1, 2))
+        assert np.array_equal(got[:, 2 * C:3 * C], oracle.maxpool_nchw(y1, 5, 1, 2))
+        assert np.array_equal(got[:, 3 * C:], oracle.maxpool_nchw(got[:, 2 * C:3 * C], 5, 1, 2))
+    # replays of the captured graph reproduce the eager result
+    xd = dev(x, dt)
+    first = host(g(xd))
+    for it in range(3):
+        assert np.array_equal(host(g(xd)), first), it
+    g.close()

@@ -545,8 +545,8 @@ void launch_maxpool_nhwc(const void* in, void* out, int dt, int N, int H, int W,
 // Three 5x5 stride-1 pad-2 max-pools in a row, each result kept (YOLOv5's SPPF block,
 // Yolov5s.mlir: y1 = m(x), y2 = m(y1), y3 = m(y2), all four concatenated): one launch instead of
 // three.  A workgroup owns one image x one 16-byte channel vector: the H*W map sits in LDS, each
-// stage reads its 25 neighbours there (the -inf halo is a skipped tap) and writes its result both
-// to memory and to the other LDS buffer.  The maps are 20x20 for a 640x640 input, so the three
+// stage takes five row maxima and then five of those down the column (the -inf halo is a skipped
+// tap) and writes its result both to memory and to the other LDS map.  The maps are 20x20 for a 640x640 input, so the three
 // stand-alone launches were nothing but latency (16 us each for 3 MB).
 // ---------------------------------------------------------------------------------------------
 constexpr int kPoolChainMaxHW = 1600;
@@ -557,19 +557,22 @@ __global__ __launch_bounds__(256) void maxpool5_chain3_kernel(const T* __restric
                                                               int ld3) {
   constexpr int VN = V16<T>::n;
   typedef typename V16<T>::type V;
-  __shared__ V buf[2][kPoolChainMaxHW];
-  const int n = blockIdx.x / CG, cg = blockIdx.x - n * CG;
+  extern __shared__ __align__(16) unsigned char pool_smem[];
   const int HW = H * W, tid = threadIdx.x;
+  V* bufs = reinterpret_cast<V*>(pool_smem);  // two maps that take turns + the row maxima of the current stage
+  V* rowmax = bufs + 2 * HW;
+  const int n = blockIdx.x / CG, cg = blockIdx.x - n * CG;
   const float inv_w = 1.0f / (float)W;
   in += (long long)n * HW * ldi + cg * VN;
-  for (int p = tid; p < HW; p += 256) buf[0][p] = *reinterpret_cast<const V*>(in + (long long)p * ldi);
+  for (int p = tid; p < HW; p += 256) bufs[p] = *reinterpret_cast<const V*>(in + (long long)p * ldi);
   __syncthreads();
 #pragma unroll
   for (int stage = 0; stage < 3; ++stage) {
-    const V* src = buf[stage & 1];
-    V* dst = buf[(stage + 1) & 1];
-    T* out = (stage == 0 ? o1 : stage == 1 ? o2 : o3) + ((long long)n * HW * (stage == 0 ? ld1 : stage == 1 ? ld2 : ld3) + cg * VN);
+    const V* src = bufs + (stage & 1) * HW;
+    V* dst = bufs + ((stage + 1) & 1) * HW;
     const int ldo = stage == 0 ? ld1 : stage == 1 ? ld2 : ld3;
+    T* out = (stage == 0 ? o1 : stage == 1 ? o2 : o3) + ((long long)n * HW * ldo + cg * VN);
+    // the 5x5 maximum as five columns of row maxima (the maximum does not depend on the order, NaN included)
     for (int p = tid; p < HW; p += 256) {
       int y = (int)((float)p * inv_w), x = p - y * W;  // exact for p < 2^24 after the correction
       if (x >= W) { ++y; x -= W; }
@@ -578,14 +581,27 @@ __global__ __launch_bounds__(256) void maxpool5_chain3_kernel(const T* __restric
 #pragma unroll
       for (int e = 0; e < VN; ++e) m[e] = -INFINITY;
 #pragma unroll
-      for (int r = -2; r <= 2; ++r)
+      for (int q = -2; q <= 2; ++q) {
+        const V v = src[(unsigned)(x + q) < (unsigned)W ? p + q : p];  // outside the map: the centre again, which changes nothing
 #pragma unroll
-        for (int q = -2; q <= 2; ++q) {
-          const bool ok = ((unsigned)(y + r) < (unsigned)H) & ((unsigned)(x + q) < (unsigned)W);
-          const V v = src[ok ? p + r * W + q : p];  // outside the map: the centre again, which changes nothing
+        for (int e = 0; e < VN; ++e) m[e] = max_nan(m[e], (float)v[e]);
+      }
+      V o;
 #pragma unroll
-          for (int e = 0; e < VN; ++e) m[e] = max_nan(m[e], (float)v[e]);
-        }
+      for (int e = 0; e < VN; ++e) o[e] = (T)m[e];
+      rowmax[p] = o;
+    }
+    __syncthreads();
+    for (int p = tid; p < HW; p += 256) {
+      float m[VN];
+#pragma unroll
+      for (int e = 0; e < VN; ++e) m[e] = -INFINITY;
+#pragma unroll
+      for (int r = -2; r <= 2; ++r) {
+        const V v = rowmax[(unsigned)(p + r * W) < (unsigned)HW ? p + r * W : p];
+#pragma unroll
+        for (int e = 0; e < VN; ++e) m[e] = max_nan(m[e], (float)v[e]);
+      }
       V o;
 #pragma unroll
       for (int e = 0; e < VN; ++e) o[e] = (T)m[e];
@@ -610,11 +626,20 @@ void launch_maxpool5_chain3(const void* in, void* o1, void* o2, void* o3, int dt
                "maxpool chain: shape not covered");
   ProfScope prof("maxpool5_chain3", 0.0, (double)dtype_size(dt) * N * C * 4.0 * H * W, s);
   const dim3 grid((unsigned)((long long)N * (C / vn)));
+  static const bool once = [] {
+    NNCV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(maxpool5_chain3_kernel<half_t>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 3 * kPoolChainMaxHW * 16));
+    NNCV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(maxpool5_chain3_kernel<float>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 3 * kPoolChainMaxHW * 16));
+    return true;
+  }();
+  (void)once;
+  const size_t smem = (size_t)3 * H * W * 16;
   if (dt == kF16)
-    hipLaunchKernelGGL((maxpool5_chain3_kernel<half_t>), grid, dim3(256), 0, s, (const half_t*)in, (half_t*)o1, (half_t*)o2, (half_t*)o3,
+    hipLaunchKernelGGL((maxpool5_chain3_kernel<half_t>), grid, dim3(256), smem, s, (const half_t*)in, (half_t*)o1, (half_t*)o2, (half_t*)o3,
                        H, W, C / vn, ldi, ld1, ld2, ld3);
   else
-    hipLaunchKernelGGL((maxpool5_chain3_kernel<float>), grid, dim3(256), 0, s, (const float*)in, (float*)o1, (float*)o2, (float*)o3, H, W,
+    hipLaunchKernelGGL((maxpool5_chain3_kernel<float>), grid, dim3(256), smem, s, (const float*)in, (float*)o1, (float*)o2, (float*)o3, H, W,
                        C / vn, ldi, ld1, ld2, ld3);
   NNCV_HIP_CHECK(hipGetLastError());
 }

@@ -218,6 +218,17 @@ int nncv_hip_graph_output_shape(const nncv_hip_graph* g, int H, int W, int* shap
  * shape, out_elems = N*C*OH*OW (checked). */
 int nncv_hip_graph_forward(nncv_hip_graph* g, const void* src, int N, int H, int W, float* out, int64_t out_elems,
                            void* stream);
+/* The workspace plan nncv_hip_graph_forward would use for an [N,in_channels,H,W] input, computed on the
+ * HOST (no device is touched, no parameters are needed): the planner is the greedy-by-size offset
+ * calculation of the reference's MemSolver (src/nncv/compiler/Utils/MemSolver.cpp:15-47) over tensor
+ * lifetimes that follow the launches actually issued (merged operators write at the merged launch).
+ * tensor_info[4*t .. 4*t+3] = {id of the tensor whose memory block t lives in (itself unless it is a
+ * slice of a concatenated tensor), byte offset of t, bytes of that block, channel offset of t in it};
+ * launch_dst[i] = tensor the launch of operator i writes, -1 if the operator is merged into another
+ * launch or writes the caller's buffer. Refuses (-1) a plan in which a launch would write over memory
+ * it reads. Returns the workspace bytes. */
+int64_t nncv_hip_graph_plan(const nncv_hip_graph_op* ops, int n_ops, int in_channels, int dtype, int N, int H, int W,
+                            int64_t* tensor_info, int tensor_cap, int32_t* launch_dst);
 /* The operator list of torchvision's MobileNetV3-small as exported in tests/Nets/MobileNetV3.mlir
  * (parameters in state_dict order without num_batches_tracked). Writes at most `cap` operators,
  * returns their number; *n_elems receives the parameter count. _mlir_ciface_forward serves this

@@ -40,7 +40,7 @@ EXPORTS = [
     "nncv_hip_matmul_f32", "nncv_hip_wino43_filter", "nncv_hip_wino43_input", "nncv_hip_wino43_gemm",
     "nncv_hip_wino43_output", "nncv_hip_maxpool3x3s2", "nncv_hip_global_avgpool",
     "nncv_hip_graph_create", "nncv_hip_graph_destroy", "nncv_hip_graph_output_shape", "nncv_hip_graph_forward",
-    "nncv_hip_mobilenetv3_small_ops", "nncv_hip_dwconv", "nncv_hip_scale_channels", "nncv_hip_eltwise",
+    "nncv_hip_graph_plan", "nncv_hip_mobilenetv3_small_ops", "nncv_hip_dwconv", "nncv_hip_scale_channels", "nncv_hip_eltwise",
     "nncv_hip_concat_slice", "nncv_hip_upsample2x", "nncv_hip_maxpool",
 ]
 
@@ -128,6 +128,8 @@ def lib():
         L.nncv_hip_graph_destroy.restype = None
         L.nncv_hip_graph_output_shape.argtypes = [vp, i, i, P(i)]
         L.nncv_hip_graph_forward.argtypes = [vp, vp, i, i, i, vp, i64, vp]
+        L.nncv_hip_graph_plan.argtypes = [P(GraphOp), i, i, i, i, i, i, P(i64), i, P(ctypes.c_int32)]
+        L.nncv_hip_graph_plan.restype = i64
         L.nncv_hip_mobilenetv3_small_ops.argtypes = [P(GraphOp), i, P(i64)]
         L.nncv_hip_dwconv.argtypes = [i, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, i, vp]
         L.nncv_hip_scale_channels.argtypes = [i, vp, vp, vp, i, i, i, vp]
@@ -252,6 +254,18 @@ def graph_create(ops, in_channels, params_blob):
     if not h:
         raise NncvHipError(lib().nncv_hip_last_error().decode())
     return h
+
+
+def graph_plan(ops, in_channels, dt, N, H, W):
+    """nncv_hip_graph_plan (host only) -> (total bytes, [(root, offset, root_bytes, c0)] per tensor, [dst] per operator)."""
+    arr = (GraphOp * len(ops))(*ops)
+    n_t = max(o.out for o in ops) + 1
+    info = (ctypes.c_int64 * (4 * n_t))()
+    dst = (ctypes.c_int32 * len(ops))()
+    total = lib().nncv_hip_graph_plan(arr, len(ops), in_channels, dt, N, H, W, info, n_t, dst)
+    if total < 0:
+        raise NncvHipError(lib().nncv_hip_last_error().decode())
+    return int(total), [tuple(int(v) for v in info[4 * t:4 * t + 4]) for t in range(n_t)], [int(d) for d in dst]
 
 
 def graph_output_shape(h, H, W):

@@ -837,6 +837,22 @@ int nncv_hip_graph_forward(nncv_hip_graph* g, const void* src, int N, int H, int
   });
 }
 
+int64_t nncv_hip_graph_plan(const nncv_hip_graph_op* ops, int n_ops, int in_channels, int dtype, int N, int H, int W,
+                            int64_t* tensor_info, int tensor_cap, int32_t* launch_dst) {
+  int64_t total = -1;
+  const int rc = guarded([&] {
+    NNCV_REQUIRE(ops && n_ops > 0 && tensor_info && launch_dst, "null or empty argument");
+    const Graph g(ops, n_ops, in_channels, nullptr, 0, dtype, nullptr);  // structure only: no device work
+    NNCV_REQUIRE(g.num_tensors() <= tensor_cap, "graph_plan: tensor_info holds fewer tensors than the graph has");
+    std::vector<long long> info((size_t)4 * g.num_tensors());
+    std::vector<int> dst((size_t)n_ops);
+    total = (int64_t)g.describe_plan(N, H, W, info.data(), dst.data());
+    for (size_t k = 0; k < info.size(); ++k) tensor_info[k] = info[k];
+    for (int i = 0; i < n_ops; ++i) launch_dst[i] = dst[i];
+  });
+  return rc == 0 ? total : -1;
+}
+
 int nncv_hip_mobilenetv3_small_ops(nncv_hip_graph_op* ops, int cap, int64_t* n_elems) {
   long long n = 0;
   const std::vector<GraphOp> v = mobilenetv3_small_ops(&n);

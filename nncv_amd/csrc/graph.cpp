@@ -51,7 +51,7 @@ int n_inputs(int kind) {
 }  // namespace
 
 Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, long long n_elems, int dt, hipStream_t s)
-    : dt_(dt), c_in_(in_channels) {
+    : dt_(dt), c_in_(in_channels), dry_(params == nullptr) {
   NNCV_REQUIRE(dt == kF32 || dt == kF16, "graph: dtype must be 1 (fp32) or 2 (fp16)");
   NNCV_REQUIRE(ops && n > 0 && in_channels > 0, "graph: empty operator list");
   const int vn = dt == kF16 ? 8 : 4;
@@ -70,7 +70,7 @@ Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, lon
   nodes_.resize(n);
 
   auto param = [&](long long off, long long count, const std::string& what) -> const void* {
-    NNCV_REQUIRE(off >= 0 && off + count <= n_elems, "graph: " + what + " lies outside the parameter blob");
+    NNCV_REQUIRE(off >= 0 && (dry_ || off + count <= n_elems), "graph: " + what + " lies outside the parameter blob");
     return blob + (size_t)off * es;
   };
 
@@ -116,6 +116,7 @@ Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, lon
         Cstored = round_up(op.F, vn);
         const int Cl = logical_[op.in[0]];  // channels the filters really have
         const void* w = param(op.w, (long long)op.F * Cl * op.K * op.K, where + "w");
+        if (dry_) break;
         nd.wt.reset((size_t)Cstored * op.K * op.K * C * es);
         NNCV_HIP_CHECK(hipMemsetAsync(nd.wt.get(), 0, nd.wt.bytes(), s));
         launch_weight_frsc(w, dt, nd.wt.get(), dt, op.F, Cl, op.K, op.K, C, s);
@@ -129,6 +130,7 @@ Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, lon
         NNCV_REQUIRE(op.K == 3 || op.K == 5, where + "K must be 3 or 5");
         NNCV_REQUIRE(op.stride >= 1 && op.pad >= 0, where + "bad geometry");
         const void* w = param(op.w, (long long)C * op.K * op.K, where + "w");
+        if (dry_) break;
         nd.wt.reset((size_t)C * op.K * op.K * es);
         launch_weight_dw(w, dt, nd.wt.get(), dt, C, op.K, s);
         break;
@@ -157,6 +159,9 @@ Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, lon
         const void* an = param(op.w, (long long)levels * op.K * 2, where + "anchors");
         const void* st = param(op.bias, levels, where + "strides");
         std::vector<float> anchors((size_t)levels * op.K * 2), strides(levels);
+        Cout = op.F;
+        Cstored = op.F;
+        if (dry_) break;
         DeviceBuffer tmp((anchors.size() + strides.size()) * 4);
         launch_cast(an, dt, tmp.get(), kF32, (long long)anchors.size(), s);
         launch_cast(st, dt, tmp.as<float>() + anchors.size(), kF32, levels, s);
@@ -167,13 +172,11 @@ Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, lon
         detect_anchor_wh_.resize(anchors.size());
         for (int l = 0; l < levels; ++l)
           for (int q = 0; q < op.K * 2; ++q) detect_anchor_wh_[l * op.K * 2 + q] = anchors[l * op.K * 2 + q] * strides[l];
-        Cout = op.F;
-        Cstored = op.F;
         break;
       }
       default: break;
     }
-    if (op.kind == NNCV_HIP_OP_CONV || op.kind == NNCV_HIP_OP_DWCONV) {
+    if (!dry_ && (op.kind == NNCV_HIP_OP_CONV || op.kind == NNCV_HIP_OP_DWCONV)) {
       const int F = Cout, Fs = Cstored > 0 ? Cstored : Cout;
       if (op.gamma >= 0) {
         NNCV_REQUIRE(op.beta >= 0 && op.mean >= 0 && op.var >= 0, where + "BatchNorm needs gamma, beta, mean and var");
@@ -236,10 +239,11 @@ Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, lon
       if (ops[i].kind == NNCV_HIP_OP_CONV && ops[i].in[0] == 0 && ops[i].stride == 2 && ops[i].in[1] < 0) {
         const GraphOp& o = ops[i];
         const int Fp = channels_[o.out], S2 = (o.K + (o.pad & 1) + 1) / 2;
+        pair_stem_ = i;
+        if (dry_) continue;
         nodes_[i].wt_pairs.reset((size_t)Fp * o.K * S2 * 8 * es);
         launch_weight_pairs(param(o.w, (long long)o.F * c_in_ * o.K * o.K, "pair stem w"), dt, nodes_[i].wt_pairs.get(), o.F, Fp, c_in_,
                             o.K, o.pad, s);
-        pair_stem_ = i;
       }
 
   // x + act(conv(.)): the ADD rides in the convolution's epilogue
@@ -388,8 +392,16 @@ const Graph::Plan& Graph::plan_of(int N, int H, int W) const {
     life[t] = TensorLife{i + 1, std::max(i + 1, last_use_[t] + 1), (size_t)N * d.H * d.W * d.C * es, 0};
     if (nodes_[i].op.kind == NNCV_HIP_OP_YOLO_DETECT) life[t].bytes = 256;  // written straight to the caller's buffer
   }
-  // three chained 5x5 stride-1 pad-2 max-pools may run as one launch that writes all three results at
-  // the first one's step (forward()): the later two are live from there
+  // Operators that were merged into an earlier launch write their result at that launch's step, so the
+  // result is live from there: the tail of a squeeze-excitation block (written by the block's one launch
+  // at the pooling operator's step), the ADD of a convolution + ADD pair (written by the convolution),
+  // the later two of three chained 5x5 stride-1 pad-2 max-pools (one launch writes all three results).
+  // Without this the planner sees the merged result and an input of the earlier launch as disjoint in
+  // time and may lay one over the other.
+  for (int i = 0; i < n; ++i) {
+    if (nodes_[i].se_head && i + 3 < n) life[nodes_[i + 3].op.out].first_op = i + 1;
+    if (nodes_[i].add_out >= 0) life[nodes_[i].add_out].first_op = std::min(life[nodes_[i].add_out].first_op, i + 1);
+  }
   {
     auto pool5 = [&](int k, int in) {
       return k < n && !nodes_[k].skip && nodes_[k].op.kind == NNCV_HIP_OP_MAXPOOL && nodes_[k].op.K == 5 && nodes_[k].op.stride == 1 &&
@@ -417,14 +429,90 @@ const Graph::Plan& Graph::plan_of(int N, int H, int W) const {
     if (nodes_[i].add_out >= 0) life[nodes_[i].op.out] = TensorLife{i + 1, i + 1, 0, 0};
   p.total = plan_offsets(life, 256);
   p.offset.resize(n_tensors_);
+  p.root_bytes.resize(n_tensors_);
   for (int t = 0; t < n_tensors_; ++t) {
     int root, c0;
     root_of(t, &root, &c0);
     p.offset[t] = life[root].offset + (size_t)c0 * es;
+    p.root_bytes[t] = life[root].bytes;
   }
+  check_plan(p);
   if (plans_.size() >= 8) plans_.erase(plans_.begin());
   plans_.push_back(std::move(p));
   return plans_.back();
+}
+
+// The tensors one launch of forward() touches: what it writes and what it reads.
+void Graph::launch_io(int i, std::vector<int>* writes, std::vector<int>* reads) const {
+  writes->clear();
+  reads->clear();
+  const int n = (int)nodes_.size();
+  const Node& nd = nodes_[i];
+  const GraphOp& op = nd.op;
+  if (nd.skip) return;
+  if (nd.se_head) {
+    reads->push_back(op.in[0]);
+    writes->push_back(nodes_[i + 3].op.out);
+    return;
+  }
+  for (int k = 0; k < 4; ++k)  // inputs of a CONCAT that already live in its result are not copied
+    if (op.in[k] >= 0 && !(op.kind == NNCV_HIP_OP_CONCAT && view_of_[op.in[k]] == op.out)) reads->push_back(op.in[k]);
+  if (nd.add_res >= 0) reads->push_back(nd.add_res);
+  if (op.kind == NNCV_HIP_OP_YOLO_DETECT) return;  // writes the caller's buffer
+  writes->push_back(nd.add_out >= 0 ? nd.add_out : op.out);
+  auto pool5 = [&](int k, int in) {
+    return k < n && !nodes_[k].skip && nodes_[k].op.kind == NNCV_HIP_OP_MAXPOOL && nodes_[k].op.K == 5 && nodes_[k].op.stride == 1 &&
+           nodes_[k].op.pad == 2 && (in < 0 || nodes_[k].op.in[0] == in);
+  };
+  if (pool5(i, -1) && pool5(i + 1, op.out) && pool5(i + 2, nodes_[i + 1].op.out)) {
+    writes->push_back(nodes_[i + 1].op.out);
+    writes->push_back(nodes_[i + 2].op.out);
+  }
+}
+
+// No launch may write memory that it also reads (a 3x3 convolution in place is a race between
+// workgroups on the halo rows) or that another tensor it writes occupies.  Two tensors inside the same
+// concatenated tensor are channel slices of the same rows and must not share channels; everything
+// else is compared as whole byte ranges.
+void Graph::check_plan(const Plan& p) const {
+  const size_t es = dtype_size(dt_);
+  auto clash = [&](int a, int b) {
+    int ra, ca, rb, cb;
+    root_of(a, &ra, &ca);
+    root_of(b, &rb, &cb);
+    if (ra == rb) return a == b || (ca < cb + channels_[b] && cb < ca + channels_[a]);
+    const size_t a0 = p.offset[a] - (size_t)ca * es, b0 = p.offset[b] - (size_t)cb * es;
+    return p.root_bytes[a] > 0 && p.root_bytes[b] > 0 && a0 < b0 + p.root_bytes[b] && b0 < a0 + p.root_bytes[a];
+  };
+  std::vector<int> w, r;
+  for (int i = 0; i < (int)nodes_.size(); ++i) {
+    launch_io(i, &w, &r);
+    for (size_t x = 0; x < w.size(); ++x) {
+      for (int t : r)
+        NNCV_REQUIRE(!clash(w[x], t), "graph: workspace plan lays the result of operator " + std::to_string(i) + " (tensor " +
+                                          std::to_string(w[x]) + ") over its input tensor " + std::to_string(t));
+      for (size_t y = x + 1; y < w.size(); ++y)
+        NNCV_REQUIRE(!clash(w[x], w[y]), "graph: workspace plan lays two results of operator " + std::to_string(i) + " over each other");
+    }
+  }
+}
+
+size_t Graph::describe_plan(int N, int H, int W, long long* tensor_info, int* launch_dst) const {
+  const Plan& p = plan_of(N, H, W);
+  for (int t = 0; t < n_tensors_; ++t) {
+    int root, c0;
+    root_of(t, &root, &c0);
+    tensor_info[4 * t + 0] = root;
+    tensor_info[4 * t + 1] = (long long)p.offset[t];
+    tensor_info[4 * t + 2] = (long long)p.root_bytes[t];
+    tensor_info[4 * t + 3] = c0;
+  }
+  std::vector<int> w, r;
+  for (int i = 0; i < (int)nodes_.size(); ++i) {
+    launch_io(i, &w, &r);
+    launch_dst[i] = w.empty() ? -1 : w[0];
+  }
+  return p.total;
 }
 
 void Graph::output_shape(int H, int W, int* C, int* OH, int* OW) const {

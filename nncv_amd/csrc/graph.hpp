@@ -21,6 +21,8 @@ class Graph {
   // channels); every other tensor is the `out` of exactly one operator and may only be read by
   // later ones.  The `out` of the last operator is the network output.
   // params_dev: flat device blob of n_elems elements of type dt that the operators' offsets index.
+  // params_dev == nullptr builds the structure only (shapes, merged launches, concatenation views, the
+  // workspace plan): no device is touched and forward() must not be called.
   Graph(const GraphOp* ops, int n, int in_channels, const void* params_dev, long long n_elems, int dt, hipStream_t s);
   int dtype() const { return dt_; }
   int in_channels() const { return c_in_; }
@@ -28,6 +30,12 @@ class Graph {
   // channels / height / width of the network output for an H x W input
   void output_shape(int H, int W, int* C, int* OH, int* OW) const;
   size_t workspace_bytes(int N, int H, int W) const;
+  int num_tensors() const { return n_tensors_; }
+  // The workspace plan for an input shape, for inspection: tensor_info[4*t..] = {tensor whose memory t
+  // lives in, byte offset of t, bytes of that memory block, channel offset of t inside it}; launch_dst[i]
+  // = the tensor operator i's launch writes first, -1 when the operator was merged into another launch
+  // or writes no workspace tensor.  Returns the workspace size.  Host arithmetic only.
+  size_t describe_plan(int N, int H, int W, long long* tensor_info, int* launch_dst) const;
   // src: NCHW [N,in_channels,H,W] of type dt; out: NCHW fp32 of the output shape (both device)
   void forward(const void* src, int N, int H, int W, float* out, void* ws, hipStream_t s) const;
 
@@ -51,11 +59,15 @@ class Graph {
     int N, H, W;
     std::vector<Dims> dims;      // per tensor
     std::vector<size_t> offset;  // per tensor, in the workspace (tensor 0: its NHWC copy)
+    std::vector<size_t> root_bytes;  // per tensor: size of the memory block it lives in
     size_t total;
   };
   const Plan& plan_of(int N, int H, int W) const;
+  void launch_io(int i, std::vector<int>* writes, std::vector<int>* reads) const;
+  void check_plan(const Plan& p) const;
 
   int dt_, c_in_, n_tensors_ = 0;
+  bool dry_ = false;
   std::vector<Node> nodes_;
   std::vector<int> channels_;  // per tensor, as stored (padded to a whole 16-byte vector)
   std::vector<int> logical_;   // per tensor, as the network defines it

@@ -68,6 +68,29 @@ def test_yolov5s_fp16(blob):
     g.close()
 
 
+def test_yolov5s_fp16_batch8_at_640_every_image(blob):
+    """Launches of several rounds of workgroups per CU (batch 8 at 640x640): a launch that wrote over
+    its own input would only show at such sizes, where the workgroups of one launch no longer all run
+    at the same time.  Image 0 of the batch against the oracle, every image against the same image
+    sent alone (images are independent of each other)."""
+    b16 = synth.round_fp16(blob)
+    g = Graph(spec.graph_ops(), 3, b16, abi.F16)
+    x = synth.round_fp16(synth.uniform(8203, (8, 3, 640, 640), 0.0, 1.0))
+    print("yolov5s fp16 batch 8 at 640", flush=True)
+    got = host(g(dev(x, abi.F16))).reshape(8, 25200, 85)
+    assert np.isfinite(got).all()
+    for n in range(8):
+        alone = host(g(dev(x[n:n + 1], abi.F16))).reshape(25200, 85)
+        e = rel_l2(got[n], alone)
+        print("image", n, "batched vs alone rel_l2", e, flush=True)
+        assert e < 2e-3, n
+    want = oracle.run_graph(spec.graph_ops(), x[:1], b16, 3, conv=oracle.hwp_conv2d)[0]
+    e_box, e_sc = rel_l2(got[0][:, :4], want[:, :4]), rel_l2(got[0][:, 4:], want[:, 4:])
+    print("image 0 vs oracle: box rel_l2", e_box, "score rel_l2", e_sc, flush=True)
+    assert e_box < FP16_REL_L2 and e_sc < FP16_REL_L2
+    g.close()
+
+
 def test_detect_refuses_being_in_the_middle(blob):
     ops = spec.graph_ops()
     extra = abi.graph_op(abi.OP_ACT, [ops[-1].out], ops[-1].out + 1, stride=0)

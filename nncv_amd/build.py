@@ -14,6 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "lib", "libnncv_hip.so")
 RT_LIB = os.path.join(HERE, "lib", "libnncv_rt.so")
+DRIVER = os.path.join(HERE, "lib", "res18_main")
 
 DEVICE_SOURCES = ["igemm.hip", "igemm_fast.hip", "conv3x3_patch.hip", "conv_pairs.hip", "stem_pool.hip", "gemm_nn.hip", "winograd.hip", "pool_layout.hip", "elementwise.hip"]
 HOST_SOURCES = ["model.cpp", "capi.cpp", "datatype.cpp", "profiler.cpp", "arena_plan.cpp", "graph.cpp"]
@@ -61,6 +62,10 @@ def build(force=False, verbose=True):
     # host-only runtime library (model.bin reader/writer), the counterpart of the reference's nncv_rt
     subprocess.check_call(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-I" + os.path.join(ROOT, "include"),
                            "-o", RT_LIB, os.path.join(CSRC, "datatype.cpp")])
+    # the example driver (the flow of the reference's examples/Res18/main.cpp): the C++ caller of the C ABI
+    subprocess.check_call(["g++", "-O2", "-std=c++17", os.path.join(ROOT, "examples", "res18_main.cpp"),
+                           "-I" + os.path.join(ROOT, "include"), "-L" + os.path.dirname(LIB), "-lnncv_hip",
+                           "-Wl,-rpath,$ORIGIN", "-Wl,-rpath-link,/opt/rocm/lib", "-o", DRIVER])
     if verbose:
         print("built", LIB)
     return LIB

@@ -34,8 +34,26 @@ void Context::init(int device) {
   // the code objects in this library exist for gfx950 only; anything else cannot run them
   NNCV_REQUIRE(arch_.rfind("gfx950", 0) == 0, "this library is built for gfx950 (MI355X); found " + arch_);
   NNCV_HIP_CHECK(hipStreamCreate(&stream_));  // default priority
+  NNCV_HIP_CHECK(hipEventCreateWithFlags(&tail_event_, hipEventDisableTiming));
   device_ = device;
   ready_ = true;
+}
+
+void Context::order_after_previous(hipStream_t s) {
+  if (!tail_pending_ || tail_stream_ == s) return;
+  // the previous caller stream may have been destroyed since: then wait for the whole device instead
+  if (hipEventRecord(tail_event_, tail_stream_) == hipSuccess && hipStreamWaitEvent(s, tail_event_, 0) == hipSuccess) {
+    tail_pending_ = false;
+    return;
+  }
+  (void)hipGetLastError();
+  NNCV_HIP_CHECK(hipDeviceSynchronize());
+  tail_pending_ = false;
+}
+
+void Context::note_stream(hipStream_t s, bool pending) {
+  tail_stream_ = s;
+  tail_pending_ = pending;
 }
 
 }  // namespace nncv_hip
@@ -68,12 +86,26 @@ void guarded_abort(const char* what, const std::function<void()>& fn) {
   }
 }
 
-struct Sync {  // NULL stream -> library stream + synchronise on exit
+// NULL stream -> library stream + synchronise on exit.  Workspace (one arena), split-K tickets and the
+// pinned staging buffers are shared by every call, and the mutex only serialises the enqueueing: work
+// left pending on one caller stream must not overlap work enqueued next on another.  So a call that
+// arrives on a different stream than the previous one first makes its stream wait for everything the
+// previous stream was given (an event recorded there now: the mutex is held, so that is exactly the
+// earlier calls' work).  Calls that stay on one stream pay nothing.
+struct Sync {
   hipStream_t s;
   bool own;
-  explicit Sync(void* user) : s(user ? static_cast<hipStream_t>(user) : Context::get().stream()), own(user == nullptr) {}
+  explicit Sync(void* user) : s(user ? static_cast<hipStream_t>(user) : Context::get().stream()), own(user == nullptr) {
+    Context::get().order_after_previous(s);
+  }
+  bool done = false;
   void finish() {
     if (own) NNCV_HIP_CHECK(hipStreamSynchronize(s));
+    Context::get().note_stream(s, /*pending=*/!own);
+    done = true;
+  }
+  ~Sync() {  // left early by an exception: whatever was enqueued may still be running
+    if (!done) Context::get().note_stream(s, true);
   }
 };
 
@@ -156,6 +188,7 @@ std::vector<CachedModel>& model_cache() {
 
 // cheap change detector for a parameter blob that lives at the same address: 4096 strided samples
 uint64_t fingerprint(const void* p, long long n, size_t es) {
+  NNCV_REQUIRE(p && n > 0, "params: empty memref");
   const unsigned char* b = static_cast<const unsigned char*>(p);
   uint64_t h = 1469598103934665603ull ^ (uint64_t)n;
   const long long step = std::max<long long>(1, n / 4096);
@@ -324,6 +357,7 @@ void forward_abi(nncv_memref2d* dst, nncv_memref4d* src, void* params, int dt) {
   Context& ctx = Context::get();
   ctx.init(-1);
   hipStream_t s = ctx.stream();
+  ctx.order_after_previous(s);
   const size_t es = dtype_size(dt);
   const nncv_memref1d* p = static_cast<const nncv_memref1d*>(params);
   NNCV_REQUIRE(p->aligned && p->strides[0] == 1, "params must be a dense rank-1 memref");
@@ -406,6 +440,7 @@ void _mlir_ciface_matmul(nncv_memref2d* res, nncv_memref2d* a, nncv_memref2d* b,
     Context& ctx = Context::get();
     ctx.init(-1);
     hipStream_t s = ctx.stream();
+    ctx.order_after_previous(s);
     const int M = (int)a->sizes[0], K = (int)a->sizes[1], N = (int)b->sizes[1];
     NNCV_REQUIRE(b->sizes[0] == K && c->sizes[0] == M && c->sizes[1] == N, "matmul: shapes do not agree");
     const size_t ab = align256((size_t)M * K * 4), bb = align256((size_t)K * N * 4), cb = align256((size_t)M * N * 4);
@@ -428,6 +463,7 @@ void _mlir_ciface_batch_nchw_conv(nncv_memref4d* res, nncv_memref4d* in, nncv_me
     Context& ctx = Context::get();
     ctx.init(-1);
     hipStream_t s = ctx.stream();
+    ctx.order_after_previous(s);
     const int N = (int)in->sizes[0], C = (int)in->sizes[1], H = (int)in->sizes[2], W = (int)in->sizes[3];
     const int F = (int)filter->sizes[0], R = (int)filter->sizes[2], S = (int)filter->sizes[3];
     const int OH = (int)out->sizes[2], OW = (int)out->sizes[3];

@@ -97,11 +97,17 @@ class Context {
   Arena arena;
   PinnedBuffer pin_in, pin_out;
   std::recursive_mutex mu;
+  // Cross-stream ordering of consecutive calls (they share the arena): see Sync in capi.cpp.
+  void order_after_previous(hipStream_t s);
+  void note_stream(hipStream_t s, bool pending);
 
  private:
   bool ready_ = false;
   int device_ = -1;
   hipStream_t stream_ = nullptr;
+  hipStream_t tail_stream_ = nullptr;  // stream of the previous call; tail_pending_: it was left with work in flight
+  hipEvent_t tail_event_ = nullptr;
+  bool tail_pending_ = false;
   std::string arch_;
 };
 

@@ -71,7 +71,8 @@ def test_conv_bn_relu_residual_nhwc(N, C, F, H, W, R, stride, pad, dt, algo):
         bn = tuple(synth.round_fp16(b) for b in bn)
     want = oracle_layer(x, w, stride, pad, bn, res, relu=True)
     layer = Conv(dt, w, stride, pad, bn=bn, relu=True, algo=algo)
-    assert layer.algo == algo
+    # a request for fp16 Winograd is served by the direct form (F(4,3) in half misses the fp16 bar)
+    assert layer.algo == (abi.ALGO_IGEMM if (dt == abi.F16 and algo == abi.ALGO_WINOGRAD) else algo)
     got = nchw(host(layer(dev(nhwc(x), dt), abi.NHWC, residual=dev(nhwc(res), dt))))
     if dt == abi.F32:
         assert max_rel(got, want) < FP32_MAX_REL
@@ -175,7 +176,7 @@ def test_random_layers(dt):
         got = nchw(host(conv(dev(nhwc(x), dt), abi.NHWC, residual=rd)))
         conv.close()
         if f16:
-            assert rel_l2(got, want) < (3e-2 if wino else FP16_REL_L2), seed  # F(4,3) in half costs about 10x the rounding error
+            assert rel_l2(got, want) < FP16_REL_L2, seed
         else:
             assert max_rel(got, want) < FP32_MAX_REL, seed
         done += 1

@@ -1,0 +1,132 @@
+"""The callers the C ABI exists for, run on the GPU as child processes and from several threads.
+
+ * examples/res18_main.cpp (this repository's driver with the flow of the reference's
+   examples/Res18/main.cpp:18-23, :79-114, built by nncv_amd/build.py) reads a model.bin, calls
+   _mlir_ciface_forward and prints the top-1 index per image: compared with the oracle.
+ * oracle/_ref/res18_ref_driver is the reference's own examples/Res18/main.cpp, compiled unchanged
+   (with its own DataType.cpp and the stb_image.h it vendors) and linked against libnncv_hip.so in
+   place of the compiled model object.  It reads ./model.bin and ./cat_256x256.jpg (the photo of the
+   reference's example, kept as tests/golden/cat_256x256.jpg) and prints its top-1 index, which must
+   be the oracle's on the pixels the same decoder produces.  Skipped where that build is absent.
+ * _mlir_ciface_forward from two threads at once: each result equals the one a serial call gives.
+"""
+import os
+import shutil
+import subprocess
+import threading
+
+import numpy as np
+import pytest
+
+import oracle
+from nncv_amd import abi, build, modelbin, synth
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+REF_DRIVER = os.path.join(ROOT, "oracle", "_ref", "res18_ref_driver")
+STB_DECODE = os.path.join(ROOT, "oracle", "_ref", "stb_decode")
+PHOTO = os.path.join(ROOT, "tests", "golden", "cat_256x256.jpg")
+
+
+@pytest.fixture(scope="module")
+def blob():
+    return synth.resnet18_params()
+
+
+def _run(cmd, cwd):
+    print("running", cmd, "in", cwd, flush=True)
+    r = subprocess.run(cmd, cwd=cwd, capture_output=True, text=True, timeout=110)
+    print(r.stdout, r.stderr, flush=True)
+    assert r.returncode == 0, (r.returncode, r.stderr)
+    return r.stdout.split("\n")
+
+
+def test_example_driver_prints_the_oracles_top1(blob, tmp_path):
+    assert os.path.exists(build.DRIVER), "nncv_amd/lib/res18_main is missing: run python -m nncv_amd.build"
+    modelbin.write_resnet18(str(tmp_path / "model.bin"), blob)
+    B, H, W = 2, 96, 64
+    x = synth.uniform(9100, (B, 3, H, W), 0.0, 1.0)
+    x.tofile(str(tmp_path / "image.f32"))
+    lines = _run([build.DRIVER, "model.bin", "image.f32", str(B), str(H), str(W)], str(tmp_path))
+    got = [int(l) for l in lines if l.strip().isdigit()]
+    # the driver normalises with the ImageNet mean / std, each step in fp32
+    mean = np.array([0.485, 0.456, 0.406], np.float32).reshape(1, 3, 1, 1)
+    std = np.array([0.229, 0.224, 0.225], np.float32).reshape(1, 3, 1, 1)
+    want = oracle.resnet18_forward(((x - mean) / std).astype(np.float32), blob)
+    assert got == [int(i) for i in want.argmax(1)], (got, want.argmax(1))
+
+
+@pytest.mark.skipif(not (os.path.exists(REF_DRIVER) and os.path.exists(STB_DECODE)),
+                    reason="oracle/_ref holds no build of the reference's driver")
+def test_the_references_own_driver_runs_on_this_library(blob, tmp_path):
+    modelbin.write_resnet18(str(tmp_path / "model.bin"), blob)
+    shutil.copy(PHOTO, str(tmp_path / "cat_256x256.jpg"))
+    lines = [l for l in _run([REF_DRIVER], str(tmp_path)) if l.strip()]
+    assert lines[0].split() == ["256", "256", "3"]
+    assert lines[1].startswith("Time: ")
+    got = int(lines[2])
+    raw = subprocess.run([STB_DECODE, PHOTO], capture_output=True, check=True).stdout
+    head, _, pixels = raw.partition(b"\n")
+    w, h, c = (int(v) for v in head.split())
+    img = np.frombuffer(pixels, np.uint8).reshape(1, h, w, c)
+    logits = oracle.resnet18_forward(oracle.preprocess_u8(img), blob)
+    want = int(oracle.top1_scan(logits)[0])
+    print("reference driver top-1", got, "oracle", want, flush=True)
+    assert got == want
+
+
+def test_forward_from_two_threads_at_once(blob):
+    """The reference's object is re-entrant; here calls serialise on the library's mutex and share one
+    arena and one weight cache.  Two threads, different inputs and shapes, several rounds: every result
+    must be bit-equal to what the same call returns alone."""
+    xs = [synth.uniform(9200, (1, 3, 64, 64), 0.0, 1.0), synth.uniform(9201, (3, 3, 96, 64), 0.0, 1.0)]
+    serial = [abi.forward(x, blob) for x in xs]
+    for x, got in zip(xs, serial):
+        want = oracle.resnet18_forward(x, blob)
+        assert np.abs(got - want).max() / np.abs(want).max() < 1e-4
+    results = [[], []]
+    errors = []
+
+    def work(k):
+        try:
+            for _ in range(6):
+                results[k].append(abi.forward(xs[k], blob))
+        except Exception as e:  # noqa: BLE001 - reported below
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(k,)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(100)
+        assert not t.is_alive()
+    assert not errors, errors
+    for k in range(2):
+        assert len(results[k]) == 6
+        for r in results[k]:
+            assert np.array_equal(r.view(np.uint32), serial[k].view(np.uint32))
+
+
+def test_device_calls_on_two_streams_do_not_overlap_in_the_shared_workspace(blob):
+    """The device entry point on two caller streams alternately, without synchronising in between: the
+    library orders the second stream behind the first (they share the activation arena), so both
+    results equal the serial ones."""
+    import torch
+    from gpu_util import Model, dev, host
+    m = Model(synth.round_fp16(blob), abi.F16, abi.ALGO_AUTO)
+    L = abi.lib()
+    xa = dev(synth.round_fp16(synth.uniform(9300, (8, 3, 224, 224), 0.0, 1.0)), abi.F16)
+    xb = dev(synth.round_fp16(synth.uniform(9301, (8, 3, 224, 224), 0.0, 1.0)), abi.F16)
+    want_a, want_b = host(m(xa)), host(m(xb))
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    oa = torch.empty((8, 1000), dtype=torch.float32, device="cuda")
+    ob = torch.empty((8, 1000), dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    for _ in range(5):
+        abi.check(L.nncv_hip_resnet18_forward(m.h, xa.data_ptr(), 8, 224, 224, oa.data_ptr(), s1.cuda_stream))
+        abi.check(L.nncv_hip_resnet18_forward(m.h, xb.data_ptr(), 8, 224, 224, ob.data_ptr(), s2.cuda_stream))
+    torch.cuda.synchronize()
+    assert np.array_equal(oa.cpu().numpy(), want_a)
+    assert np.array_equal(ob.cpu().numpy(), want_b)
+    m.close()

@@ -73,8 +73,7 @@ def test_fp16_small_batch(blob):
         err = rel_l2(got, want)
         print("fp16 algo", algo, "rel_l2", err, "top1", got.argmax(1), want.argmax(1), flush=True)
         assert err < FP16_REL_L2
-        if algo == abi.ALGO_IGEMM:
-            assert (got.argmax(1) == want.argmax(1)).all()
+        assert (got.argmax(1) == want.argmax(1)).all()
 
 
 def test_fp16_layers_take_the_kernels_they_are_measured_on(blob):

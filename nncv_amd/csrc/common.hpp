@@ -161,6 +161,7 @@ struct IgemmArgs {
                      // contiguous elements = 4 packed pixel pairs at a pixel pitch of 8)
   unsigned in_bytes, wt_bytes;  // size of one batch slice of in / wt; 0 = derived from the geometry
   const void* wt_frag;  // the same 3x3 filters in fragment-major order (launch_weight_frag3x3), or null
+  const void* wt_frag32;  // fp16 3x3 stride-1 filters in the stream kernel's order (launch_weight_frag32), or null
   // Auxiliary filters fused into the same launch (the 1x1 stride-2 shortcut convolution of a
   // down-sampling block rides on the 3x3 stride-2 one: same input pixels, centre tap only).
   // Filters [aux_f0, F) are auxiliary: their rows of `wt` are zero outside tap `aux_tap`
@@ -190,6 +191,16 @@ bool conv3x3_patch_applicable(const IgemmArgs& a, int in_dt);
 // arithmetic only (no device needed); false = no plan.
 bool conv3x3_patch_plan(int stride, int N, int OH, int OW, int F, int slabs, int out[8]);
 void launch_conv3x3_patch(const IgemmArgs& a, int in_dt, int out_dt, hipStream_t s);
+// fp16 3x3 stride-1 pad-1 layers over whole 128-byte channel slabs and whole 32-filter groups: persistent
+// workgroups, double-buffered LDS patch, 128 x 32 wave tiles (conv3x3_f16.hip).  launch returns false when no
+// tile plan exists for the shape (nothing launched).
+bool conv3x3_stream_applicable(const IgemmArgs& a, int in_dt, int out_dt);
+bool launch_conv3x3_stream(const IgemmArgs& a, hipStream_t s);
+// The stream kernel's tile plan for N images of H x W: out = {TH, S, top, aligned, vstart, tiles, patch cells, PW};
+// host arithmetic only (no device needed); false = no plan.
+bool conv3x3_stream_plan(int N, int H, int W, int out[8]);
+size_t weight_frag32_bytes(int F, int C);
+void launch_weight_frag32(const void* w, int w_dt, void* dst, int F, int C, hipStream_t s);
 // Stride-2 image convolutions over pixel pairs (C = 8, fp16, 6x3 and 3x2 windows, at most 64 filters):
 // the whole K axis in one step (conv_pairs.hip); same arguments and epilogue as the igemm kernels.
 bool conv_pairs_applicable(const IgemmArgs& a, int in_dt, int out_dt);

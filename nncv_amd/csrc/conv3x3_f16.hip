@@ -1,0 +1,671 @@
+// fp16 3x3 stride-1 pad-1 convolution + BN/residual/activation for gfx950: the stream form of the LDS-patch
+// kernel (conv3x3_patch.hip keeps every other case: fp32, stride 2, odd channel counts, wide rows).
+// Replaces what ModernTile.cpp:184-199 + ModernVec.cpp:54-62 emit for linalg.conv_2d_nchw_fchw
+// (tests/Nets/Res18.mlir:157 ...) together with the BN / add / ReLU generics behind it (:127-142, :193-203).
+//
+// What is different from conv3x3_patch.hip, and why:
+//  * A workgroup is persistent: it owns one block of filters and walks a list of pixel tiles.  The
+//    haloed input patch of the NEXT (tile, channel slab) is requested before the taps of the current one
+//    and goes from global memory straight into the other of two LDS buffers (buffer_load ... lds, 16 bytes
+//    per lane: no staging registers, no LDS store instructions), so a slab change costs one barrier and no
+//    wait, and the weight stream (fragment-major, straight from global memory into registers, nine K steps
+//    ahead) never stops at a tile boundary.
+//  * A wave owns 128 pixel slots x 32 filters (four 32x32x16 MFMAs per K step share ONE weight fragment):
+//    per MFMA the vector-memory path carries 256 bytes of weights instead of 512, and LDS (256 B/clk
+//    on this chip) carries the pixels.  The 64 B/clk vector-memory path was what a 2x2 blocking saturated.
+//  * All addressing is arithmetic on the block and lane ids with host-computed reciprocals: no tables in
+//    memory, no dependent loads before the first patch request, no divisions.
+//  * Rows of all images are stacked into one column of "virtual rows"; a tile is TH consecutive virtual
+//    rows.  Either every image takes a whole number of tiles (aligned form), or the images are one zero
+//    row apart and tiles run across image borders (gap form: that shared row is the halo of both images);
+//    14x14 and 7x7 images fill 126 of 128 slots that way instead of 98.
+//  * Patch cells are 128 bytes apart and their eight 16-byte chunks are stored XOR-swizzled with bits 1..3
+//    of the cell number: the direct-to-LDS load needs whole kilobytes per wave instruction, and the
+//    swizzle keeps the 16-byte reads of 16 neighbouring cells on distinct banks.
+//  * The filters of a wave are stored permuted (row 8q+4h+e of the MFMA holds filter 16h+4q+e), so a
+//    lane ends up with 16 consecutive output channels of a pixel: results go from the accumulators to
+//    memory with two 16-byte stores, without a transposing pass through LDS.  K groups (the waves that
+//    split the channel slab) exchange half of their partial sums through LDS once per tile.
+#include <algorithm>
+
+#include "mfma_tile.hpp"
+#include "runtime.hpp"
+
+namespace nncv_hip {
+
+using namespace mt;
+
+namespace {
+
+constexpr int kSlots = 128;                       // pixel slots per workgroup tile
+constexpr int kPitchS = 144;                      // LDS bytes per patch cell: 128 payload + 16 pad (conflict-free 16-byte reads)
+constexpr int kSegCells = 7;                      // patch cells one load instruction fills: 63 lanes x 16 bytes = 7 x 144
+constexpr int kSegB = kSegCells * kPitchS;        // 1008 bytes
+constexpr int kLoadsPerWave = 10;                 // patch load instructions per wave and stage, always all issued
+constexpr int kSegCap = 36;                       // row segments per patch buffer
+constexpr int kPatchB = (kSegCap + 1) * kSegB + 64;  // 37360 bytes: the segments, one more that takes the loads of
+                                                     // rows past the patch, and the 16 bytes an idle lane points at
+constexpr unsigned kOOBs = 0x80000000u;           // buffer offsets at or above this are out of range
+constexpr int kRing = 9;                          // weight fragments in flight per wave (K steps ahead)
+constexpr int kXcds = 8;
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// s_waitcnt immediate that waits for all but the n youngest vector-memory operations and for nothing else
+constexpr int vmcnt_only(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0070 | 0x0f00; }
+
+struct StreamArgs {
+  // ---- what the first requests need: these 16 dwords arrive preloaded in SGPRs, ahead of the scalar load
+  //      that brings the rest ----
+  const void* in;         // NHWC [N][H][W][pix]
+  const void* wf;         // launch_weight_frag32 order
+  unsigned in_bytes, wf_bytes;
+  unsigned G, div, mdiv;  // workgroup -> (filter block, first tile): see launch_conv3x3_stream
+  unsigned mS32;          // ceil(2^32 / S)
+  unsigned n_tiles;
+  unsigned tstep_nslab_flags;  // tile step | channel slabs << 16 | by_filter << 24 | aligned << 25 | top << 26
+  unsigned N_TH;               // N | TH << 24
+  unsigned geom;               // H | W << 8 | S << 16 | NSEG << 24
+  unsigned pixB;               // bytes between input pixels
+  unsigned spare;
+  // ---- the end of a tile needs these ----
+  void* out;              // NHWC [N][H][W][ldo]
+  const float* scale;     // [F] or null
+  const float* shift;     // [F] or null
+  const void* residual;   // like out, or null
+  unsigned out_bytes, mW16;  // mW16 = ceil(2^16 / W)
+  int F, act, ldo;
+#ifdef NNCV_STREAM_STAMPS
+  long long* stamps;
+#endif
+};
+static_assert(offsetof(StreamArgs, out) == 64, "sixteen preloaded dwords");
+
+// Geometry: rows of all images are stacked into virtual rows, image n's row y being v = n*S + top + y; tile t
+// covers virtual rows [top + t*TH, +TH) and W columns.  The patch of a tile is its TH + 2 rows of W + 2 cells,
+// each row padded to NSEG segments of 7 cells in LDS.
+//
+// WF x WK waves: WF filter groups of 32 (the workgroup's filter block is 32*WF filters) x WK K groups.
+template <int WF, int WK, bool ACT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv3x3_f16_stream_kernel(const StreamArgs a) {
+  static_assert(WF * WK == 4, "four waves");
+  constexpr int KPG = 4 / WK;        // 32-byte K sub-steps of a tap per K group
+  constexpr int kSteps = 9 * KPG;    // K steps per (tile, slab) stage and wave
+  constexpr int NOWN = 4 / WK;       // pixel groups of 32 slots a wave finishes in the epilogue
+  constexpr int BF = 32 * WF;        // filters per workgroup
+  static_assert(kSteps % kRing == 0 || kRing % kSteps == 0, "the weight ring must tile a stage");
+  constexpr int kPieceSteps = KPG >= 2 ? 10 : 5;  // K steps of a stage that carry the next patch's load instructions
+  static_assert(kLoadsPerWave % kPieceSteps == 0 && kPieceSteps < kSteps, "patch pieces per step");
+  // weight refills younger than the last patch piece at the end of a stage: what the wait for the patch may leave in flight
+  constexpr int kYoung = kSteps - kPieceSteps < kRing ? kSteps - kPieceSteps : kRing;
+  extern __shared__ __align__(16) unsigned char smem[];
+#ifdef NNCV_STREAM_STAMPS
+  long long ts[8] = {clock64(), 0, 0, 0, 0, 0, 0, 0};
+  const long long wall0 = wall_clock64();
+#endif
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wf = wave % WF, wk = wave / WF;
+  const int lrow = lane & 31, lchunk = lane >> 5;
+
+  const int tstep = (int)(a.tstep_nslab_flags & 0xffffu), nslab = (int)((a.tstep_nslab_flags >> 16) & 0xffu);
+  const bool by_filter = (a.tstep_nslab_flags >> 24) & 1u, aligned = (a.tstep_nslab_flags >> 25) & 1u;
+  const unsigned top = (a.tstep_nslab_flags >> 26) & 1u;
+  const unsigned N = a.N_TH & 0xffffffu, TH = a.N_TH >> 24;
+  const unsigned H = a.geom & 0xffu, W = (a.geom >> 8) & 0xffu, S = (a.geom >> 16) & 0xffu, NSEG = a.geom >> 24;
+  const int PWp = (int)NSEG * kSegCells;  // cells per patch row in LDS
+
+  // ---- workgroup -> filter block and tile list.  Hardware deals workgroups to the 8 XCDs round-robin by
+  //      linear id; `logical` makes an XCD's workgroups neighbours in the (filter block, tile) order ----
+  const unsigned bid = blockIdx.x;
+  const unsigned logical = (bid & (kXcds - 1)) * ((a.G + kXcds - 1) / kXcds) + (bid / kXcds);
+  if (logical >= a.G) return;
+  const unsigned qd = a.div == 1 ? logical : __umulhi(logical, a.mdiv);
+  const unsigned rd = logical - qd * a.div;
+  const int fb = (int)(by_filter ? qd : rd);
+  int tile = (int)(by_filter ? rd : qd);
+  const int tend = (int)a.n_tiles;
+  if (tile >= tend) return;
+#ifdef NNCV_STREAM_STAMPS
+  ts[6] = clock64();
+#endif
+
+  const __amdgpu_buffer_rsrc_t rs_wf = make_rsrc(a.wf, a.wf_bytes);
+
+  // ---- weights: fragment (filter group g, iteration it = slab*9 + tap, sub-step kk) is the kilobyte at
+  //      ((g*niter + it)*4 + kk)*1024; a wave streams its KPG sub-steps of every iteration ----
+  const int niter = nslab * 9;
+  const int wbase = ((fb * WF + wf) * niter * 4 + wk * KPG) * 1024;
+  const unsigned wlane = lane * 16;
+  const int wwrap = niter * 4096;
+  u32x4 wring[kRing];
+  // step L (counted over the whole stream of the wave, KPG per iteration) lives at wbase + (L / KPG) * 4096 + (L % KPG) * 1024
+  auto wload_at = [&](int soff) { return __builtin_amdgcn_raw_buffer_load_b128(rs_wf, wlane, wbase + soff, 0); };
+  auto ring_fill = [&](auto q_c) {
+    constexpr int q = decltype(q_c)::value;
+    int it = q / KPG;
+    if (it >= niter) it -= niter;  // a one-slab layer wraps inside the first ring fill
+    wring[q] = wload_at(it * 4096 + (q % KPG) * 1024);
+  };
+  // the first fragments go out ahead of the patch request (they gate the first MFMA as much as the patch
+  // does); the rest follow it, so that the patch is not queued behind 72 KB of weights per CU
+  ring_fill(std::integral_constant<int, 0>());
+  ring_fill(std::integral_constant<int, 1>());
+  ring_fill(std::integral_constant<int, 2>());
+
+  // ---- patch loader.  One load instruction (buffer_load ... lds: global memory straight into LDS, lane l
+  //      to the instruction's LDS base + 16*l) fills one row segment: 63 lanes = chunk l % 9 of cell l / 9
+  //      of the segment's 7 cells, chunk 8 being the pad of the 144-byte cell pitch.  The buffer descriptor
+  //      of the instruction is the image row the segment belongs to, W pixels long: cells left and right of
+  //      the image, the pad chunk and whole rows above / below the image (a descriptor of no bytes) come
+  //      back as zeros from the range check, and the per-tile addressing is scalar arithmetic, once per row.
+  //      Wave w loads patch rows w, w + 4, ...; its m-th instruction is segment m % NSEG of its row m / NSEG.
+  //      Every wave issues all kLoadsPerWave instructions in every stage (those past the patch load nothing
+  //      into a spare segment): a fixed count, so the compiler's wait for a weight fragment older than a
+  //      patch request never includes the request.  The pieces are spread over the first K steps of a
+  //      stage, between its MFMAs: an instruction outside the tap loop costs its wave four idle cycles
+  //      of the matrix pipe, one inside it costs nothing. ----
+  const unsigned lcell = ((unsigned)lane * 57u) >> 9, lch = (unsigned)lane - lcell * 9u;  // lane / 9, lane % 9
+  // offset in the row of this lane's unit for a segment starting at cell 0: cell c is image column c - 1
+  const unsigned uoff = lch == 8u ? kOOBs : (lcell - 1u) * a.pixB + lch * 16u;
+  const unsigned segstep = kSegCells * a.pixB;
+  const bool dma_lane = lane < 63;
+  // the loader's cursor: first virtual row of the patch and image of the tile, byte offset of the channel slab in a
+  // pixel, LDS offset of the buffer; this wave's row counter and segment in the row; descriptor of the current
+  // row, lane offset and LDS offset of the current segment
+  unsigned pc_v0m1 = 0, pc_nt = 0, pc_slabB = 0, pc_i = 0, pc_j = 0, pc_vo = 0;
+  int pc_dst = 0, pc_lds = 0, pc_ldstep = 0;
+  bool pc_live = false;
+  __amdgpu_buffer_rsrc_t pc_rs = make_rsrc(a.in, 0u);
+  auto patch_begin = [&](int t, int slab, int dstbuf, bool live) {
+    const unsigned v0 = top + (unsigned)t * TH;
+    pc_v0m1 = v0 - 1u;  // wraps for the row above the first image: fails n < N
+    pc_nt = __umulhi(v0, a.mS32);
+    pc_slabB = (unsigned)slab * 128u;
+    pc_dst = dstbuf;
+    pc_live = live;
+    pc_i = 0;
+    pc_j = 0;
+  };
+  auto patch_piece = [&]() {
+    if (pc_j == 0) {  // a new row
+      const unsigned r = (unsigned)wave + 4u * pc_i;
+      const unsigned v = pc_v0m1 + r;
+      const unsigned n = __umulhi(v, a.mS32);
+      const unsigned y = v - n * S - top;
+      const bool ok = pc_live & (y < H) & (n < N) & (r < TH + 2u) & (!aligned | (n == pc_nt));
+      const unsigned long long rowB = (unsigned long long)((n * H + y) * W) * a.pixB;
+      pc_rs = make_rsrc(static_cast<const unsigned char*>(a.in) + (ok ? rowB : 0ull), ok ? W * a.pixB : 0u);
+      pc_vo = uoff + pc_slabB;
+      // rows past the patch: every piece into the one spare segment
+      pc_lds = pc_dst + (int)((r < TH + 2u ? r * NSEG : (unsigned)kSegCap) * kSegB);
+      pc_ldstep = r < TH + 2u ? kSegB : 0;
+    }
+    if (dma_lane) __builtin_amdgcn_raw_ptr_buffer_load_lds(pc_rs, (lds_ptr_t)(smem + pc_lds), 16, pc_vo, 0, 0, 0);
+    // a lane left of the row wraps to a huge offset, one right of it passes W pixels: both out of range
+    pc_vo += segstep;
+    pc_lds += pc_ldstep;
+    if (++pc_j == NSEG) {
+      pc_j = 0;
+      ++pc_i;
+    }
+  };
+
+  patch_begin(tile, 0, 0, true);
+#pragma unroll
+  for (int m = 0; m < kLoadsPerWave; ++m) patch_piece();
+  __builtin_amdgcn_sched_barrier(0);
+  ring_fill(std::integral_constant<int, 3>());
+  ring_fill(std::integral_constant<int, 4>());
+  ring_fill(std::integral_constant<int, 5>());
+  ring_fill(std::integral_constant<int, 6>());
+  ring_fill(std::integral_constant<int, 7>());
+  ring_fill(std::integral_constant<int, 8>());
+  __builtin_amdgcn_sched_barrier(0);
+#ifdef NNCV_STREAM_STAMPS
+  ts[1] = clock64();
+#endif
+
+  // ---- everything below needs the rest of the arguments ----
+  const __amdgpu_buffer_rsrc_t rs_out = make_rsrc(a.out, a.out_bytes);
+  const __amdgpu_buffer_rsrc_t rs_res = make_rsrc(a.residual ? a.residual : a.out, a.residual ? a.out_bytes : 0u);
+
+  // Scale and shift of the block's filters wait in LDS behind the patch buffers (32 registers less across
+  // the taps).  They are requested here and written at the end of the first stage: writing them now would
+  // wait for the youngest requests, i.e. for everything.
+  const int sse = tid & (BF / 2 - 1);
+  const bool ss_shift = sse >= BF / 4;
+  floatx4 vsc, vsh;
+  {
+    const unsigned off = (unsigned)(fb * BF + 4 * (ss_shift ? sse - BF / 4 : sse)) * 4u;
+    // a missing vector is a buffer of no bytes: the load returns zeros and the select later fills in 1 / 0
+    const __amdgpu_buffer_rsrc_t rs_sc = make_rsrc(a.scale ? a.scale : a.in, a.scale ? (unsigned)a.F * 4u : 0u);
+    const __amdgpu_buffer_rsrc_t rs_sh = make_rsrc(a.shift ? a.shift : a.in, a.shift ? (unsigned)a.F * 4u : 0u);
+    vsc = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rs_sc, off, 0, 0));
+    vsh = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rs_sh, off, 0, 0));
+  }
+  bool ss_pending = true;
+
+  // ---- this lane's four pixel slots: LDS address of tap (r, 0) (static) and output offset (per tile) ----
+  int rowbase[3][4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const unsigned s = (unsigned)(j * 32 + lrow);
+    const unsigned ty = (s * a.mW16) >> 16, tx = s - ty * W;
+    const int cell = ty < TH ? (int)(ty * (unsigned)PWp + tx) : 0;
+#pragma unroll
+    for (int r = 0; r < 3; ++r) rowbase[r][j] = (cell + r * PWp) * kPitchS + (lchunk + 2 * wk * KPG) * 16;
+  }
+  const int f0 = fb * BF + wf * 32 + 16 * lchunk;    // this lane's 16 consecutive output channels
+  unsigned obase[NOWN];  // of the slot groups wk*NOWN .. +NOWN-1, the ones this wave finishes
+  auto tile_outputs = [&](int t) {
+    const unsigned v0 = top + (unsigned)t * TH;
+#pragma unroll
+    for (int j = 0; j < NOWN; ++j) {
+      const unsigned s = (unsigned)((wk * NOWN + j) * 32 + lrow);
+      const unsigned ty = (s * a.mW16) >> 16, tx = s - ty * W;
+      const unsigned v = v0 + ty;
+      const unsigned n = __umulhi(v, a.mS32);
+      const unsigned y = v - n * S - top;
+      const unsigned bad = (unsigned)(ty >= TH) | (unsigned)(y >= H) | (unsigned)(n >= N);
+      const unsigned pixel = (n * H + y) * W + tx;
+      obase[j] = ((pixel * (unsigned)a.ldo + (unsigned)f0) * 2u) | (bad ? kOOBs : 0u);
+    }
+  };
+  tile_outputs(tile);
+
+  floatx16 acc[4];
+  // the first patch is older than the six fragments and the two scale / shift loads requested after it
+  __builtin_amdgcn_s_waitcnt(vmcnt_only(8));
+  __syncthreads();
+#ifdef NNCV_STREAM_STAMPS
+  ts[2] = clock64();
+#endif
+
+  int cur = 0;      // LDS offset of the buffer the taps read
+  int wo = 0;       // byte offset of the current stage's first iteration in the weight stream
+  u32x4 pr[2][4];   // pixel operands of two K steps
+
+  for (;;) {
+    const int next_tile = tile + tstep;
+    for (int slab = 0; slab < nslab; ++slab) {
+      const bool last = slab + 1 == nslab;
+      // The patch of the next stage goes into the other buffer.  After the last tile the same instructions
+      // are issued with descriptors of no bytes (same count on every path; no memory traffic).
+      const bool more = !last || next_tile < tend;
+      patch_begin(last ? next_tile : tile, last ? 0 : slab + 1, cur ^ kPatchB, more);
+      u32x4 rv[NOWN][2];
+      __builtin_amdgcn_sched_barrier(0);
+      int wo_next = wo + 9 * 4096;
+      if (wo_next >= wwrap) wo_next = 0;
+
+      // ---- taps: 9*KPG K steps, fully unrolled; pixel operands one step ahead, weights kRing steps ahead ----
+      auto ldp = [&](auto step_c) {
+        constexpr int st = decltype(step_c)::value;
+        constexpr int t = st / KPG, k = st % KPG;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          pr[st & 1][j] = *reinterpret_cast<const u32x4*>(smem + rowbase[t / 3][j] + (t % 3) * kPitchS + k * 32);
+      };
+      ldp(std::integral_constant<int, 0>());
+      auto steps = [&](auto self, auto step_c) -> void {
+        constexpr int st = decltype(step_c)::value;
+        if constexpr (st < kSteps) {
+          if constexpr (st + 1 < kSteps) ldp(std::integral_constant<int, st + 1>());
+          __builtin_amdgcn_sched_barrier(0);
+          if constexpr (st == 0) {
+            // the first step of a tile starts the sums: a zero C operand instead of 64 cleared registers
+            if (slab == 0) {
+              const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+              for (int j = 0; j < 4; ++j)
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, wring[0]), __builtin_bit_cast(half8, pr[0][j]), zero, 0, 0, 0);
+            } else {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) Mma<half_t>::run(wring[0], pr[0][j], acc[j]);
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) Mma<half_t>::run(wring[st % kRing], pr[st & 1][j], acc[j]);
+          }
+          // the next patch: kLoadsPerWave pieces over the first K steps of the stage
+          if constexpr (st < kPieceSteps) {
+#pragma unroll
+            for (int q = 0; q < kLoadsPerWave / kPieceSteps; ++q) patch_piece();
+          }
+          // the residual rows this wave finishes go out in the tile's last stage, behind the patch pieces (no
+          // residual: a buffer of no bytes, the loads return zeros without touching memory)
+          if constexpr (st == kPieceSteps) {
+            if (last) {
+#pragma unroll
+              for (int o = 0; o < NOWN; ++o) {
+                rv[o][0] = __builtin_amdgcn_raw_buffer_load_b128(rs_res, obase[o], 0, 0);
+                rv[o][1] = __builtin_amdgcn_raw_buffer_load_b128(rs_res, obase[o], 16, 0);
+              }
+            }
+          }
+          // refill this ring slot with the fragment kRing steps further down the stream
+          constexpr int nx = st + kRing, nt = nx / KPG, nk = nx % KPG;
+          static_assert(nt < 18, "the ring reaches at most into the next stage");
+          if constexpr (nt < 9) {
+            wring[st % kRing] = wload_at(wo + nt * 4096 + nk * 1024);
+          } else {
+            wring[st % kRing] = wload_at(wo_next + (nt - 9) * 4096 + nk * 1024);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          self(self, std::integral_constant<int, st + 1>());
+        }
+      };
+      steps(steps, std::integral_constant<int, 0>());
+      wo = wo_next;
+
+      // The next patch (requested before this stage's kSteps >= kRing weight refills) must have landed, and
+      // every wave must be past its taps, before the buffers change roles.
+      __builtin_amdgcn_sched_barrier(0);
+      if (ss_pending) {
+        asm volatile("" : "+v"(vsc), "+v"(vsh));  // keeps this arithmetic (and its wait for the two loads) here
+        const float one = a.scale ? 0.0f : 1.0f;  // added to the zeros of a missing scale vector
+        floatx4 ssv;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) ssv[q] = ss_shift ? vsh[q] : vsc[q] + one;
+        *reinterpret_cast<floatx4*>(smem + 2 * kPatchB + sse * 16) = ssv;
+        ss_pending = false;
+      }
+      __builtin_amdgcn_s_waitcnt(vmcnt_only(kYoung));
+      __syncthreads();
+      const int done = cur;  // the buffer this stage's taps read: free until the end of the next stage's request
+      const int delta = cur ? -kPatchB : kPatchB;
+      cur ^= kPatchB;
+#pragma unroll
+      for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) rowbase[r][j] += delta;
+      if (!last) continue;
+#ifdef NNCV_STREAM_STAMPS
+      if (ts[3] == 0) ts[3] = clock64();
+#endif
+
+      // ---- end of a tile: K groups exchange partial sums through the buffer the taps just left, then
+      //      scale/shift, residual, activation, one rounding, two 16-byte stores per pixel ----
+      constexpr int FPL = 16;
+      if constexpr (WK > 1) {
+        // Wave (wf, wk) finishes slot groups [wk*NOWN, (wk+1)*NOWN); the other groups' partial sums go to
+        // their owners, lane-linear (kilobytes of 64 lanes x 16 bytes: no bank conflicts, no address math).
+        // Two rounds when the partial sums of all four groups do not fit one patch buffer (WK = 4).
+        constexpr int NR = WK == 4 ? 2 : 1;
+        unsigned char* xb = smem + done;
+#pragma unroll
+        for (int round = 0; round < NR; ++round) {
+          if (round > 0) __syncthreads();  // the previous round's readers are done
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int owner = j / NOWN;
+            if ((NR == 1 || j / 2 == round) && owner != wk) {
+              const int rank = wk < owner ? wk : wk - 1;  // position among the WK-1 senders
+              const int jx = NR == 1 ? j : (j & 1), nj = NR == 1 ? 4 : 2;
+              unsigned char* dst = xb + (((wf * nj + jx) * (WK - 1) + rank) * 4) * 1024 + lane * 16;
+#pragma unroll
+              for (int q = 0; q < 4; ++q)
+                *reinterpret_cast<floatx4*>(dst + q * 1024) = floatx4{acc[j][4 * q], acc[j][4 * q + 1], acc[j][4 * q + 2], acc[j][4 * q + 3]};
+            }
+          }
+          __syncthreads();
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            if (j / NOWN == wk && (NR == 1 || j / 2 == round)) {
+              const int jx = NR == 1 ? j : (j & 1), nj = NR == 1 ? 4 : 2;
+              const unsigned char* src = xb + (((wf * nj + jx) * (WK - 1)) * 4) * 1024 + lane * 16;
+#pragma unroll
+              for (int r = 0; r < WK - 1; ++r)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                  const floatx4 p = *reinterpret_cast<const floatx4*>(src + (r * 4 + q) * 1024);
+#pragma unroll
+                  for (int e = 0; e < 4; ++e) acc[j][4 * q + e] += p[e];
+                }
+            }
+          }
+        }
+      }
+#ifdef NNCV_STREAM_STAMPS
+      if (ts[4] == 0) ts[4] = clock64();
+#endif
+      floatx4 sc4[4], sh4[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        sc4[q] = *reinterpret_cast<const floatx4*>(smem + 2 * kPatchB + (wf * 32 + 16 * lchunk + 4 * q) * 4);
+        sh4[q] = *reinterpret_cast<const floatx4*>(smem + 2 * kPatchB + (BF + wf * 32 + 16 * lchunk + 4 * q) * 4);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (j / NOWN != wk) continue;
+        const int o = j % NOWN;
+        float y[FPL];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) y[4 * q + e] = acc[j][4 * q + e] * sc4[q][e] + sh4[q][e];
+        const bool res_after = ACT && (a.act & kActResidualAfter);
+        float rf[FPL];
+        if (a.residual) {
+          const half8 r0 = __builtin_bit_cast(half8, rv[o][0]), r1 = __builtin_bit_cast(half8, rv[o][1]);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            rf[e] = (float)r0[e];
+            rf[8 + e] = (float)r1[e];
+          }
+          if (!res_after) {
+#pragma unroll
+            for (int e = 0; e < FPL; ++e) y[e] += rf[e];
+          }
+        }
+        if (a.act == kActRelu) {
+#pragma unroll
+          for (int e = 0; e < FPL; ++e) y[e] = relu_ugt(y[e]);
+        } else if (ACT && a.act) {
+          act_apply_n<true>(y, a.act & 0xff);
+        }
+        if (a.residual && res_after) {
+#pragma unroll
+          for (int e = 0; e < FPL; ++e) y[e] += rf[e];
+        }
+        half8 o0, o1;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          o0[e] = (half_t)y[e];
+          o1[e] = (half_t)y[8 + e];
+        }
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o0), rs_out, obase[o], 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o1), rs_out, obase[o], 16, 0);
+      }
+      if constexpr (WK > 1) __syncthreads();  // the exchange buffer takes a patch again at the start of the next stage
+    }
+    if (next_tile >= tend) break;
+    tile = next_tile;
+    tile_outputs(tile);
+  }
+#ifdef NNCV_STREAM_STAMPS
+  ts[5] = clock64();
+  if (a.stamps && tid == 0) {
+    long long* d = a.stamps + 16 * (long long)blockIdx.x;
+    for (int i = 0; i < 6; ++i) d[i] = ts[i];
+    d[6] = ts[6] - ts[0];
+    d[7] = 0;
+    d[8] = wall0;
+    d[9] = wall_clock64();
+  }
+#endif
+}
+
+// ---- host side: tile plan ---------------------------------------------------------------------------
+
+struct StreamGeom {
+  int TH = 0, NSEG = 0, S = 0, top = 0, aligned = 0, n_tiles = 0;
+};
+
+unsigned recip32(unsigned d) { return d == 1 ? 0u : (unsigned)(0xffffffffull / d + 1); }  // ceil(2^32 / d) for d >= 2
+
+// TH consecutive virtual rows of W columns per tile: at most kSlots pixels, and a patch of TH + 2 rows of
+// NSEG segments within kSegCap.  Aligned form: S = bands * TH >= H virtual rows per image, tiles never
+// leave their image.  Gap form: S = H + 1 (one shared zero row between images), tiles of the largest TH
+// that fits.  The form with fewer tiles wins; aligned on a tie (it wastes no slot on the zero rows).
+bool stream_geometry(int N, int H, int W, StreamGeom* g) {
+  if (N < 1 || H < 1 || W < 1 || W > kSlots || H > 254 || N >= (1 << 24)) return false;
+  const int NSEG = (W + 2 + kSegCells - 1) / kSegCells;
+  int thmax = 0;
+  for (int th = 1; th <= H + 1; ++th)
+    if (th * W <= kSlots && (th + 2) * NSEG <= kSegCap && (th + 2 + 3) / 4 * NSEG <= kLoadsPerWave) thmax = th;
+  if (thmax == 0) return false;
+  const int tha0 = std::min(thmax, H);
+  const int bands = (H + tha0 - 1) / tha0, tha = (H + bands - 1) / bands;
+  const long long tiles_a = (long long)N * bands;
+  const long long rows_g = (long long)N * (H + 1) - 1;  // virtual rows 1 .. N*(H+1)-1
+  const long long tiles_g = (rows_g + thmax - 1) / thmax;
+  const bool gap = tiles_g < tiles_a;
+  g->NSEG = NSEG;
+  if (gap) {
+    g->TH = thmax; g->S = H + 1; g->top = 1; g->aligned = 0; g->n_tiles = (int)tiles_g;
+  } else {
+    g->TH = tha; g->S = bands * tha; g->top = 0; g->aligned = 1; g->n_tiles = (int)tiles_a;
+  }
+  if (g->S < 2 || g->S > 255) return false;  // the reciprocal of 1 does not exist; S travels in 8 bits
+  // the reciprocal multiplications are exact while x * d < 2^32 (x the dividend, d the divisor)
+  const long long vmax = (long long)N * g->S + g->TH + 2;
+  return (gap ? tiles_g : tiles_a) < (1ll << 24) && vmax * g->S < (1ll << 31);
+}
+
+// 3x3 weights FCHW -> the stream kernel's order: per 32-filter group, per 128-byte channel slab, per tap,
+// four kilobyte fragments (K sub-steps), each the 64 lanes' 16-byte MFMA A operands in lane order.
+// Row rho = 8q + 4h + e of the MFMA holds filter 16h + 4q + e of the group, so that the accumulator
+// registers of a lane are 16 consecutive filters.  Filters beyond F are zero.
+template <typename Ts>
+__global__ void weight_frag32_kernel(const Ts* __restrict__ w, half_t* __restrict__ dst, int F, int C, int Fp) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;  // one 16-byte chunk each
+  const int nslab = C / 64;
+  const long long total = (long long)(Fp / 32) * nslab * 9 * 4 * 64;
+  if (idx >= total) return;
+  const int L = (int)(idx & 63);
+  long long r = idx >> 6;
+  const int kk = (int)(r & 3); r >>= 2;
+  const int tap = (int)(r % 9); r /= 9;
+  const int sl = (int)(r % nslab);
+  const int g = (int)(r / nslab);
+  const int rho = L & 31;
+  const int f = g * 32 + 16 * ((rho >> 2) & 1) + 4 * (rho >> 3) + (rho & 3);
+  const int c0 = sl * 64 + ((L >> 5) + 2 * kk) * 8;
+  half_t* d = dst + idx * 8;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) d[e] = f < F ? (half_t)(float)w[((long long)f * C + c0 + e) * 9 + tap] : (half_t)0.0f;
+}
+
+#ifdef NNCV_STREAM_STAMPS
+long long* g_stamps = nullptr;
+#endif
+
+}  // namespace
+
+#ifdef NNCV_STREAM_STAMPS
+extern "C" void nncv_hip_debug_stream_stamps(void* p) { g_stamps = (long long*)p; }
+#endif
+
+size_t weight_frag32_bytes(int F, int C) { return (size_t)((F + 31) / 32) * 32 * 9 * C * 2; }
+
+void launch_weight_frag32(const void* w, int w_dt, void* dst, int F, int C, hipStream_t s) {
+  NNCV_REQUIRE(C % 64 == 0, "weight_frag32: C must be a multiple of the 128-byte slab");
+  const int Fp = (F + 31) / 32 * 32;
+  const long long total = (long long)(Fp / 32) * (C / 64) * 9 * 4 * 64;
+  const unsigned grid = (unsigned)((total + 255) / 256);
+  if (w_dt == kF16) hipLaunchKernelGGL((weight_frag32_kernel<half_t>), dim3(grid), dim3(256), 0, s, (const half_t*)w, (half_t*)dst, F, C, Fp);
+  else hipLaunchKernelGGL((weight_frag32_kernel<float>), dim3(grid), dim3(256), 0, s, (const float*)w, (half_t*)dst, F, C, Fp);
+  NNCV_HIP_CHECK(hipGetLastError());
+}
+
+bool conv3x3_stream_plan(int N, int H, int W, int out[8]) {
+  StreamGeom g;
+  if (!stream_geometry(N, H, W, &g)) return false;
+  out[0] = g.TH; out[1] = g.S; out[2] = g.top; out[3] = g.aligned; out[4] = g.top; out[5] = g.n_tiles; out[6] = (g.TH + 2) * g.NSEG; out[7] = g.NSEG;
+  return true;
+}
+
+bool conv3x3_stream_applicable(const IgemmArgs& a, int in_dt, int out_dt) {
+  static const bool off = getenv("NNCV_HIP_NO_STREAM") != nullptr;
+  // deeper layers (more than two channel slabs per tile) stay with the patch kernel unless asked for: their
+  // stages are nine K steps long and the per-stage work of this kernel shows
+  static const bool all = getenv("NNCV_HIP_STREAM_ALL") != nullptr;
+  if (off || in_dt != kF16 || out_dt != kF16 || !a.wt_frag32 || (a.C > 128 && !all)) return false;
+  const int pix = a.pix_stride ? a.pix_stride : a.C;
+  const bool act_ok = a.relu <= kActRelu || ((a.relu & 0xff) <= kActSigmoid && (a.relu & ~(0xff | kActResidualAfter)) == 0);
+  StreamGeom g;
+  return act_ok && a.aux_f0 == 0 && a.R == 3 && a.S == 3 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 1 && a.pad_w == 1 &&
+         a.OH == a.H && a.OW == a.W && a.batch == 1 && a.C % 64 == 0 && a.F % 32 == 0 && pix % 8 == 0 && a.ldo % 8 == 0 && a.ldo >= a.F &&
+         (long long)a.N * a.H * a.W * a.ldo * 2 < (1ll << 31) && (long long)a.N * a.H * a.W * pix * 2 < (1ll << 31) &&
+         a.in_bytes < kOOBs && (long long)a.F * 9 * a.C * 2 < (1ll << 31) && stream_geometry(a.N, a.H, a.W, &g);
+}
+
+template <int WF, int WK, bool ACT>
+static void launch_stream_cfg(const StreamArgs& a, int grid, double flops, double bytes, const char* tag, hipStream_t s) {
+  auto kern = conv3x3_f16_stream_kernel<WF, WK, ACT>;
+  constexpr int smem = 2 * kPatchB + 2 * 32 * WF * 4;
+  static const bool attr = [&] {
+    NNCV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+    return true;
+  }();
+  (void)attr;
+  ProfScope prof(tag, flops, bytes, s);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), smem, s, a);
+}
+
+bool launch_conv3x3_stream(const IgemmArgs& g, hipStream_t s) {
+  StreamGeom geo;
+  if (!stream_geometry(g.N, g.H, g.W, &geo)) return false;
+  // 64-filter blocks (two filter groups x two K groups) by default; 32-filter blocks (four K groups) when that is
+  // what it takes to give every CU two workgroups
+  const bool narrow = g.F % 64 != 0 || (long long)geo.n_tiles * (g.F / 64) < 384;
+  const int FB = narrow ? g.F / 32 : g.F / 64;
+  const size_t wbytes = weight_frag32_bytes(g.F, g.C);
+  // An XCD's workgroups are neighbours: a contiguous range of tile lists (tiles that share halo rows meet in one
+  // L2) with all filter blocks, or -- when the filters outgrow an L2 -- a range of filter blocks with all lists.
+  const bool by_filter = FB % kXcds == 0 && wbytes > (2u << 20);
+  // as many workgroups per filter block as two per CU allow, evened out so that all of them walk the
+  // same number of tiles (896 tiles on 512 places: 448 workgroups of two tiles, not 384 of two and 128 of one)
+  const int places = std::max(1, 512 / FB), rounds = (geo.n_tiles + places - 1) / places;
+  const int Wpf = (geo.n_tiles + rounds - 1) / rounds;
+  const int G = FB * Wpf, grid = (G + kXcds - 1) / kXcds * kXcds;
+  NNCV_REQUIRE(Wpf < 65536 && g.C / 64 < 256, "conv3x3_stream: tile step / slab count out of range");
+  StreamArgs a{};
+  const int pix = g.pix_stride ? g.pix_stride : g.C;
+  a.in = g.in; a.wf = g.wt_frag32; a.out = g.out; a.scale = g.scale; a.shift = g.shift; a.residual = g.residual;
+  a.F = g.F; a.act = g.relu; a.ldo = g.ldo;
+  a.in_bytes = g.in_bytes ? g.in_bytes : (unsigned)((size_t)g.N * g.H * g.W * pix * 2);
+  a.wf_bytes = (unsigned)wbytes;
+  a.out_bytes = (unsigned)((size_t)g.N * g.H * g.W * g.ldo * 2);
+  a.G = (unsigned)G;
+  a.div = (unsigned)(by_filter ? Wpf : FB);
+  a.mdiv = recip32(a.div);
+  a.mS32 = recip32((unsigned)geo.S);
+  a.n_tiles = (unsigned)geo.n_tiles;
+  a.tstep_nslab_flags = (unsigned)Wpf | ((unsigned)(g.C / 64) << 16) | ((by_filter ? 1u : 0u) << 24) | ((unsigned)geo.aligned << 25) | ((unsigned)geo.top << 26);
+  a.N_TH = (unsigned)g.N | ((unsigned)geo.TH << 24);
+  a.geom = (unsigned)g.H | ((unsigned)g.W << 8) | ((unsigned)geo.S << 16) | ((unsigned)geo.NSEG << 24);
+  a.pixB = (unsigned)pix * 2u;
+  a.mW16 = (unsigned)((65536 + g.W - 1) / g.W);
+#ifdef NNCV_STREAM_STAMPS
+  a.stamps = g_stamps;
+#endif
+  const double P = (double)g.N * g.H * g.W;
+  const double flops = 2.0 * P * g.C * 9.0 * g.F;
+  const double bytes = 2.0 * (P * g.C + 9.0 * g.C * g.F + P * g.F * (g.residual ? 2 : 1));
+  const bool act = g.relu > kActRelu;
+  if (narrow) {
+    if (act) launch_stream_cfg<1, 4, true>(a, grid, flops, bytes, "conv3x3_stream<f16,1,4,act>", s);
+    else launch_stream_cfg<1, 4, false>(a, grid, flops, bytes, "conv3x3_stream<f16,1,4>", s);
+  } else {
+    if (act) launch_stream_cfg<2, 2, true>(a, grid, flops, bytes, "conv3x3_stream<f16,2,2,act>", s);
+    else launch_stream_cfg<2, 2, false>(a, grid, flops, bytes, "conv3x3_stream<f16,2,2>", s);
+  }
+  NNCV_HIP_CHECK(hipGetLastError());
+  return true;
+}
+
+}  // namespace nncv_hip

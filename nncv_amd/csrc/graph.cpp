@@ -123,6 +123,10 @@ Graph::Graph(const GraphOp* ops, int n, int in_channels, const void* params, lon
         if (op.K == 3 && (op.stride == 1 || op.stride == 2) && op.pad == 1 && Cl == C && Cstored == op.F && C % (128 / (int)es) == 0) {
           nd.wfrag.reset((size_t)((op.F + 63) / 64) * 64 * 9 * C * es);
           launch_weight_frag3x3(w, dt, nd.wfrag.get(), dt, op.F, C, s);
+          if (dt == kF16 && op.stride == 1 && C % 64 == 0 && op.F % 32 == 0) {
+            nd.wfrag32.reset(weight_frag32_bytes(op.F, C));
+            launch_weight_frag32(w, dt, nd.wfrag32.get(), op.F, C, s);
+          }
         }
         break;
       }
@@ -562,7 +566,7 @@ void Graph::forward(const void* src, int N, int H, int W, float* out, void* ws, 
       case NNCV_HIP_OP_CONV: {
         IgemmArgs g{};
         const int dst = nd.add_out >= 0 ? nd.add_out : op.out;
-        g.in = at(op.in[0]); g.wt = nd.wt.get(); g.wt_frag = nd.wfrag.get(); g.out = at(dst);
+        g.in = at(op.in[0]); g.wt = nd.wt.get(); g.wt_frag = nd.wfrag.get(); g.wt_frag32 = nd.wfrag32.get(); g.out = at(dst);
         g.scale = nd.scale.as<float>(); g.shift = nd.shift.as<float>();
         g.residual = nd.add_res >= 0 ? at(nd.add_res) : (op.in[1] >= 0 ? at(op.in[1]) : nullptr);
         // padding filters (zero rows, zero scale/shift) are computed like any other: o.C >= op.F

@@ -43,7 +43,7 @@ class Graph {
   struct Node {
     GraphOp op;
     int C = 0;  // channels of in[0] as stored (the network input is padded to a whole vector)
-    DeviceBuffer wt, wfrag, scale, shift;
+    DeviceBuffer wt, wfrag, wfrag32, scale, shift;
     // Set on a GAVGPOOL that starts "pool -> 1x1 conv + bias -> 1x1 conv + bias -> SCALE of the pooled
     // tensor" whose three intermediate tensors have no other reader: the four operators run as one
     // squeeze-excitation launch and the next three nodes are skipped.

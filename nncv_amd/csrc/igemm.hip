@@ -287,6 +287,7 @@ void launch_igemm(const IgemmArgs& a_in, int in_dt, int out_dt, hipStream_t s) {
     launch_conv_pairs(a, s);
     return;
   }
+  if (conv3x3_stream_applicable(a, in_dt, out_dt) && launch_conv3x3_stream(a, s)) return;
   if (in_dt == out_dt && conv3x3_patch_applicable(a, in_dt)) {
     launch_conv3x3_patch(a, in_dt, out_dt, s);
     return;

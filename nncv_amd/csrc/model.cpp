@@ -68,6 +68,10 @@ ConvLayer::ConvLayer(const Desc& d, const void* w, const void* gamma, const void
     if (d.R == 3 && d.S == 3 && (d.stride == 1 || d.stride == 2) && d.pad == 1 && d.C % (128 / (int)es) == 0) {
       wfrag_.reset((size_t)((d.F + 63) / 64) * 64 * 9 * d.C * es);
       launch_weight_frag3x3(w, d.dt, wfrag_.get(), d.dt, d.F, d.C, s);
+      if (d.dt == kF16 && d.stride == 1 && d.C % 64 == 0 && d.F % 32 == 0) {
+        wfrag32_.reset(weight_frag32_bytes(d.F, d.C));
+        launch_weight_frag32(w, d.dt, wfrag32_.get(), d.F, d.C, s);
+      }
       if (d.dt == kF32) {
         splitk_counters_.reset(kSplitKCounters * sizeof(int));
         NNCV_HIP_CHECK(hipMemsetAsync(splitk_counters_.get(), 0, splitk_counters_.bytes(), s));
@@ -127,7 +131,7 @@ void ConvLayer::forward(const void* in, int N, int H, int W, const void* residua
   }
   NNCV_REQUIRE(d_.C % (16 / (int)es) == 0 && d_.F % 4 == 0, "conv: NHWC igemm needs C %% chunk == 0 and F %% 4 == 0");
   IgemmArgs a{};
-  a.in = in; a.wt = wt_.get(); a.wt_frag = wfrag_.get(); a.out = out;
+  a.in = in; a.wt = wt_.get(); a.wt_frag = wfrag_.get(); a.wt_frag32 = wfrag32_.get(); a.out = out;
   a.scale = scale_.as<float>(); a.shift = shift_.as<float>(); a.residual = residual;
   a.N = N; a.H = H; a.W = W; a.C = d_.C; a.F = d_.F; a.R = d_.R; a.S = d_.S; a.OH = OH; a.OW = OW;
   a.stride_h = a.stride_w = d_.stride; a.pad_h = a.pad_w = d_.pad;

@@ -55,7 +55,7 @@ class ConvLayer {
  private:
   Desc d_;
   int algo_;
-  DeviceBuffer wt_, wfrag_, U_, scale_, shift_, wt_shift_;
+  DeviceBuffer wt_, wfrag_, wfrag32_, U_, scale_, shift_, wt_shift_;
   DeviceBuffer wt_cat_, scale_cat_, shift_cat_;  // this layer's filters followed by the fused shortcut's
   DeviceBuffer aux_wfrag_;  // the fused shortcut's filters alone, fragment-major (stride-2 patch kernel)
   DeviceBuffer splitk_counters_;  // tickets of the patch kernel's K split (fp32); zero between launches

@@ -41,10 +41,9 @@ constexpr int kSlots = 128;                       // pixel slots per workgroup t
 constexpr int kPitchS = 144;                      // LDS bytes per patch cell: 128 payload + 16 pad (conflict-free 16-byte reads)
 constexpr int kSegCells = 7;                      // patch cells one load instruction fills: 63 lanes x 16 bytes = 7 x 144
 constexpr int kSegB = kSegCells * kPitchS;        // 1008 bytes
-constexpr int kLoadsPerWave = 10;                 // patch load instructions per wave and stage, always all issued
-constexpr int kSegCap = 36;                       // row segments per patch buffer
-constexpr int kPatchB = (kSegCap + 1) * kSegB + 64;  // 37360 bytes: the segments, one more that takes the loads of
-                                                     // rows past the patch, and the 16 bytes an idle lane points at
+constexpr int kLoadsPerWave = 9;                  // patch load instructions per wave and stage, always all issued
+constexpr int kSegCap = 4 * kLoadsPerWave;        // row segments per patch buffer
+constexpr int kPatchB = kSegCap * kSegB + 64;     // 36352 bytes: the segments and the 16 bytes the last lane of the last one writes
 constexpr unsigned kOOBs = 0x80000000u;           // buffer offsets at or above this are out of range
 constexpr int kRing = 9;                          // weight fragments in flight per wave (K steps ahead)
 constexpr int kXcds = 8;
@@ -94,8 +93,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   constexpr int NOWN = 4 / WK;       // pixel groups of 32 slots a wave finishes in the epilogue
   constexpr int BF = 32 * WF;        // filters per workgroup
   static_assert(kSteps % kRing == 0 || kRing % kSteps == 0, "the weight ring must tile a stage");
-  constexpr int kPieceSteps = KPG >= 2 ? 10 : 5;  // K steps of a stage that carry the next patch's load instructions
-  static_assert(kLoadsPerWave % kPieceSteps == 0 && kPieceSteps < kSteps, "patch pieces per step");
+  constexpr int kPieceSteps = KPG >= 2 ? 9 : 5;  // K steps of a stage that carry the next patch's load instructions
+  static_assert(kPieceSteps < kSteps, "patch pieces per step");
   // weight refills younger than the last patch piece at the end of a stage: what the wait for the patch may leave in flight
   constexpr int kYoung = kSteps - kPieceSteps < kRing ? kSteps - kPieceSteps : kRing;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -156,65 +155,65 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
   // ---- patch loader.  One load instruction (buffer_load ... lds: global memory straight into LDS, lane l
   //      to the instruction's LDS base + 16*l) fills one row segment: 63 lanes = chunk l % 9 of cell l / 9
-  //      of the segment's 7 cells, chunk 8 being the pad of the 144-byte cell pitch.  The buffer descriptor
-  //      of the instruction is the image row the segment belongs to, W pixels long: cells left and right of
-  //      the image, the pad chunk and whole rows above / below the image (a descriptor of no bytes) come
-  //      back as zeros from the range check, and the per-tile addressing is scalar arithmetic, once per row.
-  //      Wave w loads patch rows w, w + 4, ...; its m-th instruction is segment m % NSEG of its row m / NSEG.
-  //      Every wave issues all kLoadsPerWave instructions in every stage (those past the patch load nothing
-  //      into a spare segment): a fixed count, so the compiler's wait for a weight fragment older than a
-  //      patch request never includes the request.  The pieces are spread over the first K steps of a
-  //      stage, between its MFMAs: an instruction outside the tap loop costs its wave four idle cycles
-  //      of the matrix pipe, one inside it costs nothing. ----
+  //      of the segment's 7 cells, chunk 8 being the pad of the 144-byte cell pitch; lane 63 is the first
+  //      unit of the NEXT segment, which it loads like that segment's lane 0 does (the same bytes to the same
+  //      place).  The patch buffer is kSegCap segments in row-major order, wave w loading segments 9w .. 9w+8:
+  //      63 cells, whose tensor offsets (or an out-of-range offset for cells outside the image: the load then
+  //      returns zeros) one lane each computes once per tile; an instruction's lanes fetch their cell's
+  //      offset from there with a lane permute.  Every wave issues all nine instructions in every stage:
+  //      a fixed count, so the compiler's wait for a weight fragment older than a patch request never
+  //      includes the request.  The pieces are spread over the first K steps of a stage, between its
+  //      MFMAs: outside the tap loop an instruction costs its wave about eight idle cycles. ----
   const unsigned lcell = ((unsigned)lane * 57u) >> 9, lch = (unsigned)lane - lcell * 9u;  // lane / 9, lane % 9
-  // offset in the row of this lane's unit for a segment starting at cell 0: cell c is image column c - 1
-  const unsigned uoff = lch == 8u ? kOOBs : (lcell - 1u) * a.pixB + lch * 16u;
-  const unsigned segstep = kSegCells * a.pixB;
-  const bool dma_lane = lane < 63;
-  // the loader's cursor: first virtual row of the patch and image of the tile, byte offset of the channel slab in a
-  // pixel, LDS offset of the buffer; this wave's row counter and segment in the row; descriptor of the current
-  // row, lane offset and LDS offset of the current segment
-  unsigned pc_v0m1 = 0, pc_nt = 0, pc_slabB = 0, pc_i = 0, pc_j = 0, pc_vo = 0;
-  int pc_dst = 0, pc_lds = 0, pc_ldstep = 0;
-  bool pc_live = false;
-  __amdgpu_buffer_rsrc_t pc_rs = make_rsrc(a.in, 0u);
-  auto patch_begin = [&](int t, int slab, int dstbuf, bool live) {
+  const unsigned lchoff = lch == 8u ? kOOBs : lch * 16u;
+  const int perm0 = (int)lcell * 4;  // permute address of this lane's cell in the wave's first segment
+  // the cell this lane computes offsets for: number lane of the wave's 63 (+ the first of the next wave's)
+  const unsigned cseg = (unsigned)wave * kLoadsPerWave + (((unsigned)lane * 37u) >> 8);  // its segment: lane / 7
+  const unsigned crow = NSEG == 1 ? cseg : (cseg * (65535u / NSEG + 1u)) >> 16;            // its patch row: cseg / NSEG
+  const unsigned ccol = (cseg - crow * NSEG) * kSegCells + ((unsigned)lane - (((unsigned)lane * 37u) >> 8) * 7u) - 1u;  // image column
+  const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(a.in, a.in_bytes);
+  unsigned celloff = kOOBs;  // tensor offset of that cell for the tile being loaded
+  unsigned pc_lchslab = 0;   // lchoff + the channel slab's byte offset in a pixel
+  int pc_dst = 0;            // LDS offset of this wave's first segment in the buffer being filled
+  auto patch_tile = [&](int t, bool live) {
     const unsigned v0 = top + (unsigned)t * TH;
-    pc_v0m1 = v0 - 1u;  // wraps for the row above the first image: fails n < N
-    pc_nt = __umulhi(v0, a.mS32);
-    pc_slabB = (unsigned)slab * 128u;
-    pc_dst = dstbuf;
-    pc_live = live;
-    pc_i = 0;
-    pc_j = 0;
+    const unsigned nt = __umulhi(v0, a.mS32);
+    // patch row crow is virtual row v0 - 1 + crow; counted one image further down so that the row above the
+    // first image divides like the others (its image is then -1 and fails n < N)
+    const unsigned vS = v0 - 1u + crow + S;
+    const unsigned nS = __umulhi(vS, a.mS32);
+    const unsigned n = nS - 1u, y = vS - nS * S - top;
+    const unsigned bad = (unsigned)(y >= H) | (unsigned)(n >= N) | (unsigned)(ccol >= W) | (unsigned)(crow >= TH + 2u) |
+                         (unsigned)(aligned & (n != nt)) | (unsigned)!live;
+    celloff = (((n * H + y) * W + ccol) * a.pixB) | (bad ? kOOBs : 0u);
   };
-  auto patch_piece = [&]() {
-    if (pc_j == 0) {  // a new row
-      const unsigned r = (unsigned)wave + 4u * pc_i;
-      const unsigned v = pc_v0m1 + r;
-      const unsigned n = __umulhi(v, a.mS32);
-      const unsigned y = v - n * S - top;
-      const bool ok = pc_live & (y < H) & (n < N) & (r < TH + 2u) & (!aligned | (n == pc_nt));
-      const unsigned long long rowB = (unsigned long long)((n * H + y) * W) * a.pixB;
-      pc_rs = make_rsrc(static_cast<const unsigned char*>(a.in) + (ok ? rowB : 0ull), ok ? W * a.pixB : 0u);
-      pc_vo = uoff + pc_slabB;
-      // rows past the patch: every piece into the one spare segment
-      pc_lds = pc_dst + (int)((r < TH + 2u ? r * NSEG : (unsigned)kSegCap) * kSegB);
-      pc_ldstep = r < TH + 2u ? kSegB : 0;
-    }
-    if (dma_lane) __builtin_amdgcn_raw_ptr_buffer_load_lds(pc_rs, (lds_ptr_t)(smem + pc_lds), 16, pc_vo, 0, 0, 0);
-    // a lane left of the row wraps to a huge offset, one right of it passes W pixels: both out of range
-    pc_vo += segstep;
-    pc_lds += pc_ldstep;
-    if (++pc_j == NSEG) {
-      pc_j = 0;
-      ++pc_i;
+  auto patch_begin = [&](int slab, int dstbuf) {
+    pc_lchslab = lchoff + (unsigned)slab * 128u;
+    pc_dst = dstbuf + wave * (kLoadsPerWave * kSegB);
+  };
+  unsigned pc_vo = 0;
+  auto patch_piece_perm = [&](auto p_c) {  // the lanes' cell offsets for piece p
+    constexpr int pp = decltype(p_c)::value;
+    pc_vo = (unsigned)__builtin_amdgcn_ds_bpermute(perm0 + 28 * pp, (int)celloff);
+  };
+  auto patch_piece_load = [&](auto p_c) {
+    constexpr int pp = decltype(p_c)::value;
+    // out of range stays out of range under this sum, except for the pad chunk of a cell that is itself out of
+    // range (the two flags cancel): that unit then loads the tensor's first bytes into a pad nobody reads
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_in, (lds_ptr_t)(smem + pc_dst + pp * kSegB), 16, pc_vo + pc_lchslab, 0, 0, 0);
+  };
+  auto patch_all = [&](auto self, auto p_c) -> void {
+    constexpr int pp = decltype(p_c)::value;
+    if constexpr (pp < kLoadsPerWave) {
+      patch_piece_perm(p_c);
+      patch_piece_load(p_c);
+      self(self, std::integral_constant<int, pp + 1>());
     }
   };
 
-  patch_begin(tile, 0, 0, true);
-#pragma unroll
-  for (int m = 0; m < kLoadsPerWave; ++m) patch_piece();
+  patch_tile(tile, true);
+  patch_begin(0, 0);
+  patch_all(patch_all, std::integral_constant<int, 0>());
   __builtin_amdgcn_sched_barrier(0);
   ring_fill(std::integral_constant<int, 3>());
   ring_fill(std::integral_constant<int, 4>());
@@ -283,6 +282,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   ts[2] = clock64();
 #endif
 
+#ifdef NNCV_STREAM_STEPSTAMPS
+  int fine_idx = 0;
+#endif
   int cur = 0;      // LDS offset of the buffer the taps read
   int wo = 0;       // byte offset of the current stage's first iteration in the weight stream
   u32x4 pr[2][4];   // pixel operands of two K steps
@@ -293,67 +295,75 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       const bool last = slab + 1 == nslab;
       // The patch of the next stage goes into the other buffer.  After the last tile the same instructions
       // are issued with descriptors of no bytes (same count on every path; no memory traffic).
-      const bool more = !last || next_tile < tend;
-      patch_begin(last ? next_tile : tile, last ? 0 : slab + 1, cur ^ kPatchB, more);
+      // the cell offsets of the next tile's patch replace this tile's once its last slab has been requested
+      if (last) patch_tile(next_tile, next_tile < tend);
+      patch_begin(last ? 0 : slab + 1, cur ^ kPatchB);
       u32x4 rv[NOWN][2];
       __builtin_amdgcn_sched_barrier(0);
       int wo_next = wo + 9 * 4096;
       if (wo_next >= wwrap) wo_next = 0;
 
-      // ---- taps: 9*KPG K steps, fully unrolled; pixel operands one step ahead, weights kRing steps ahead ----
-      auto ldp = [&](auto step_c) {
+      // ---- taps: 9*KPG K steps, fully unrolled; pixel operands one step ahead, weights kRing steps ahead.
+      //      A wave issues in order and about one instruction per eight cycles: four MFMAs in a row followed by
+      //      everything else make a step last the sum of both.  So every MFMA is followed by its share of the
+      //      step's other work (the read of the next step's pixel operand, a part of a patch piece, the weight
+      //      refill), pinned there by scheduling fences, and runs under it. ----
+      auto ldp1 = [&](auto step_c, int j) {
         constexpr int st = decltype(step_c)::value;
         constexpr int t = st / KPG, k = st % KPG;
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          pr[st & 1][j] = *reinterpret_cast<const u32x4*>(smem + rowbase[t / 3][j] + (t % 3) * kPitchS + k * 32);
+        pr[st & 1][j] = *reinterpret_cast<const u32x4*>(smem + rowbase[t / 3][j] + (t % 3) * kPitchS + k * 32);
       };
-      ldp(std::integral_constant<int, 0>());
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ldp1(std::integral_constant<int, 0>(), j);
       auto steps = [&](auto self, auto step_c) -> void {
         constexpr int st = decltype(step_c)::value;
         if constexpr (st < kSteps) {
-          if constexpr (st + 1 < kSteps) ldp(std::integral_constant<int, st + 1>());
-          __builtin_amdgcn_sched_barrier(0);
-          if constexpr (st == 0) {
-            // the first step of a tile starts the sums: a zero C operand instead of 64 cleared registers
-            if (slab == 0) {
-              const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-              for (int j = 0; j < 4; ++j)
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, wring[0]), __builtin_bit_cast(half8, pr[0][j]), zero, 0, 0, 0);
-            } else {
-#pragma unroll
-              for (int j = 0; j < 4; ++j) Mma<half_t>::run(wring[0], pr[0][j], acc[j]);
-            }
-          } else {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) Mma<half_t>::run(wring[st % kRing], pr[st & 1][j], acc[j]);
-          }
-          // the next patch: kLoadsPerWave pieces over the first K steps of the stage
-          if constexpr (st < kPieceSteps) {
-#pragma unroll
-            for (int q = 0; q < kLoadsPerWave / kPieceSteps; ++q) patch_piece();
-          }
-          // the residual rows this wave finishes go out in the tile's last stage, behind the patch pieces (no
-          // residual: a buffer of no bytes, the loads return zeros without touching memory)
-          if constexpr (st == kPieceSteps) {
-            if (last) {
-#pragma unroll
-              for (int o = 0; o < NOWN; ++o) {
-                rv[o][0] = __builtin_amdgcn_raw_buffer_load_b128(rs_res, obase[o], 0, 0);
-                rv[o][1] = __builtin_amdgcn_raw_buffer_load_b128(rs_res, obase[o], 16, 0);
-              }
-            }
-          }
-          // refill this ring slot with the fragment kRing steps further down the stream
+#ifdef NNCV_STREAM_STEPSTAMPS
+          if (a.stamps && lane == 0 && fine_idx < 60) a.stamps[65536 + (blockIdx.x * 4 + wave) * 64 + fine_idx] = clock64();
+          ++fine_idx;
+#endif
+          constexpr int PPS = (kLoadsPerWave + kPieceSteps - 1) / kPieceSteps;  // patch pieces per step: 1 or 2
           constexpr int nx = st + kRing, nt = nx / KPG, nk = nx % KPG;
           static_assert(nt < 18, "the ring reaches at most into the next stage");
-          if constexpr (nt < 9) {
-            wring[st % kRing] = wload_at(wo + nt * 4096 + nk * 1024);
-          } else {
-            wring[st % kRing] = wload_at(wo_next + (nt - 9) * 4096 + nk * 1024);
+          const u32x4 wfrag = wring[st % kRing];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            if (st == 0 && slab == 0) {
+              // the first step of a tile starts the sums: a zero C operand instead of 64 cleared registers
+              const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+              acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, wfrag), __builtin_bit_cast(half8, pr[st & 1][j]), zero, 0, 0, 0);
+            } else {
+              Mma<half_t>::run(wfrag, pr[st & 1][j], acc[j]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (st + 1 < kSteps) ldp1(std::integral_constant<int, st + 1>(), j);
+            // the next patch: kLoadsPerWave pieces over the first K steps of the stage
+            if constexpr (st * PPS < kLoadsPerWave) {
+              if (j == 0) patch_piece_perm(std::integral_constant<int, st * PPS>());
+              if (j == 1) patch_piece_load(std::integral_constant<int, st * PPS>());
+              if constexpr (PPS == 2 && st * PPS + 1 < kLoadsPerWave) {
+                if (j == 2) patch_piece_perm(std::integral_constant<int, st * PPS + 1>());
+                if (j == 3) patch_piece_load(std::integral_constant<int, st * PPS + 1>());
+              }
+            }
+            // the residual rows this wave finishes go out in the tile's last stage, behind the patch pieces (no
+            // residual: a buffer of no bytes, the loads return zeros without touching memory)
+            if constexpr (st == kPieceSteps) {
+              if (j < NOWN && last) {
+                rv[j % NOWN][0] = __builtin_amdgcn_raw_buffer_load_b128(rs_res, obase[j % NOWN], 0, 0);
+                rv[j % NOWN][1] = __builtin_amdgcn_raw_buffer_load_b128(rs_res, obase[j % NOWN], 16, 0);
+              }
+            }
+            if (j == 3) {
+              // refill this ring slot with the fragment kRing steps further down the stream
+              if constexpr (nt < 9) {
+                wring[st % kRing] = wload_at(wo + nt * 4096 + nk * 1024);
+              } else {
+                wring[st % kRing] = wload_at(wo_next + (nt - 9) * 4096 + nk * 1024);
+              }
+            }
+            __builtin_amdgcn_sched_barrier(0);
           }
-          __builtin_amdgcn_sched_barrier(0);
           self(self, std::integral_constant<int, st + 1>());
         }
       };
@@ -384,6 +394,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       if (!last) continue;
 #ifdef NNCV_STREAM_STAMPS
       if (ts[3] == 0) ts[3] = clock64();
+#endif
+#ifdef NNCV_STREAM_STEPSTAMPS
+      if (a.stamps && lane == 0 && fine_idx < 60) a.stamps[65536 + (blockIdx.x * 4 + wave) * 64 + fine_idx] = clock64();
+      ++fine_idx;
 #endif
 
       // ---- end of a tile: K groups exchange partial sums through the buffer the taps just left, then
@@ -515,7 +529,7 @@ bool stream_geometry(int N, int H, int W, StreamGeom* g) {
   const int NSEG = (W + 2 + kSegCells - 1) / kSegCells;
   int thmax = 0;
   for (int th = 1; th <= H + 1; ++th)
-    if (th * W <= kSlots && (th + 2) * NSEG <= kSegCap && (th + 2 + 3) / 4 * NSEG <= kLoadsPerWave) thmax = th;
+    if (th * W <= kSlots && (th + 2) * NSEG <= kSegCap) thmax = th;
   if (thmax == 0) return false;
   const int tha0 = std::min(thmax, H);
   const int bands = (H + tha0 - 1) / tha0, tha = (H + bands - 1) / bands;

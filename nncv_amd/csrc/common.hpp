@@ -196,9 +196,10 @@ void launch_conv3x3_patch(const IgemmArgs& a, int in_dt, int out_dt, hipStream_t
 // tile plan exists for the shape (nothing launched).
 bool conv3x3_stream_applicable(const IgemmArgs& a, int in_dt, int out_dt);
 bool launch_conv3x3_stream(const IgemmArgs& a, hipStream_t s);
-// The stream kernel's tile plan for N images of H x W: out = {TH, S, top, aligned, vstart, tiles, patch cells, PW};
-// host arithmetic only (no device needed); false = no plan.
-bool conv3x3_stream_plan(int N, int H, int W, int out[8]);
+// The stream kernel's launch plan for N images of H x W with C channels and F filters: out = {TH, S, top, aligned, tiles,
+// segments per patch row, pixel groups, filter groups, K groups, filter blocks, workgroups per filter block, segment
+// capacity of a patch buffer}; host arithmetic only (no device needed); false = no plan.
+bool conv3x3_stream_plan(int N, int H, int W, int C, int F, int out[12]);
 size_t weight_frag32_bytes(int F, int C);
 void launch_weight_frag32(const void* w, int w_dt, void* dst, int F, int C, hipStream_t s);
 // Stride-2 image convolutions over pixel pairs (C = 8, fp16, 6x3 and 3x2 windows, at most 64 filters):

@@ -37,13 +37,15 @@ using namespace mt;
 
 namespace {
 
-constexpr int kSlots = 128;                       // pixel slots per workgroup tile
+constexpr int kSlots = 128;                       // pixel slots per pixel group of a workgroup tile
 constexpr int kPitchS = 144;                      // LDS bytes per patch cell: 128 payload + 16 pad (conflict-free 16-byte reads)
 constexpr int kSegCells = 7;                      // patch cells one load instruction fills: 63 lanes x 16 bytes = 7 x 144
 constexpr int kSegB = kSegCells * kPitchS;        // 1008 bytes
 constexpr int kLoadsPerWave = 9;                  // patch load instructions per wave and stage, always all issued
-constexpr int kSegCap = 4 * kLoadsPerWave;        // row segments per patch buffer
-constexpr int kPatchB = kSegCap * kSegB + 64;     // 36352 bytes: the segments and the 16 bytes the last lane of the last one writes
+// row segments per patch buffer and its bytes (the segments and the 16 bytes the last lane of the last one writes) for a
+// workgroup of nw waves: 36352 bytes for four waves, 72640 for eight
+constexpr int seg_cap(int nw) { return nw * kLoadsPerWave; }
+constexpr int patch_bytes(int nw) { return seg_cap(nw) * kSegB + 64; }
 constexpr unsigned kOOBs = 0x80000000u;           // buffer offsets at or above this are out of range
 constexpr int kRing = 9;                          // weight fragments in flight per wave (K steps ahead)
 constexpr int kXcds = 8;
@@ -84,10 +86,15 @@ static_assert(offsetof(StreamArgs, out) == 64, "sixteen preloaded dwords");
 // covers virtual rows [top + t*TH, +TH) and W columns.  The patch of a tile is its TH + 2 rows of W + 2 cells,
 // each row padded to NSEG segments of 7 cells in LDS.
 //
-// WF x WK waves: WF filter groups of 32 (the workgroup's filter block is 32*WF filters) x WK K groups.
-template <int WF, int WK, bool ACT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv3x3_f16_stream_kernel(const StreamArgs a) {
-  static_assert(WF * WK == 4, "four waves");
+// PG x WF x WK waves: PG pixel groups of up to four 32-slot rows (a tile is up to 128*PG pixel slots), WF filter
+// groups of 32 (the workgroup's filter block is 32*WF filters), WK K groups.  Four waves: two workgroups per CU;
+// eight waves: one, whose waves w and w + 4 share a SIMD -- one of each pixel group, so that a tile of seven
+// rows (four + three) loads all SIMDs alike.
+template <int PG, int WF, int WK, bool ACT>
+__global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv3x3_f16_stream_kernel(const StreamArgs a) {
+  static_assert(WF * WK == 4 && (PG == 1 || PG == 2), "four or eight waves");
+  constexpr int NW = PG * WF * WK;
+  constexpr int kPatchB = patch_bytes(NW);
   constexpr int KPG = 4 / WK;        // 32-byte K sub-steps of a tap per K group
   constexpr int kSteps = 9 * KPG;    // K steps per (tile, slab) stage and wave
   constexpr int NOWN = 4 / WK;       // pixel groups of 32 slots a wave finishes in the epilogue
@@ -105,7 +112,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wf = wave % WF, wk = wave / WF;
+  const int pg = wave / 4, wf = (wave % 4) % WF, wk = (wave % 4) / WF;
   const int lrow = lane & 31, lchunk = lane >> 5;
 
   const int tstep = (int)(a.tstep_nslab_flags & 0xffffu), nslab = (int)((a.tstep_nslab_flags >> 16) & 0xffu);
@@ -114,6 +121,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const unsigned N = a.N_TH & 0xffffffu, TH = a.N_TH >> 24;
   const unsigned H = a.geom & 0xffu, W = (a.geom >> 8) & 0xffu, S = (a.geom >> 16) & 0xffu, NSEG = a.geom >> 24;
   const int PWp = (int)NSEG * kSegCells;  // cells per patch row in LDS
+  // 32-slot rows of the tile this wave's pixel group holds: four, or what is left of the tile's
+  const int trows = (int)((TH * W + 31u) >> 5);
+  const int nrows = PG == 1 ? 4 : (trows - 4 * pg < 4 ? (trows - 4 * pg < 0 ? 0 : trows - 4 * pg) : 4);
 
   // ---- workgroup -> filter block and tile list.  Hardware deals workgroups to the 8 XCDs round-robin by
   //      linear id; `logical` makes an XCD's workgroups neighbours in the (filter block, tile) order ----
@@ -250,7 +260,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   int rowbase[3][4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const unsigned s = (unsigned)(j * 32 + lrow);
+    const unsigned s = (unsigned)(pg * kSlots + j * 32 + lrow);
     const unsigned ty = (s * a.mW16) >> 16, tx = s - ty * W;
     const int cell = ty < TH ? (int)(ty * (unsigned)PWp + tx) : 0;
 #pragma unroll
@@ -262,7 +272,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const unsigned v0 = top + (unsigned)t * TH;
 #pragma unroll
     for (int j = 0; j < NOWN; ++j) {
-      const unsigned s = (unsigned)((wk * NOWN + j) * 32 + lrow);
+      const unsigned s = (unsigned)(pg * kSlots + (wk * NOWN + j) * 32 + lrow);
       const unsigned ty = (s * a.mW16) >> 16, tx = s - ty * W;
       const unsigned v = v0 + ty;
       const unsigned n = __umulhi(v, a.mS32);
@@ -314,7 +324,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         pr[st & 1][j] = *reinterpret_cast<const u32x4*>(smem + rowbase[t / 3][j] + (t % 3) * kPitchS + k * 32);
       };
 #pragma unroll
-      for (int j = 0; j < 4; ++j) ldp1(std::integral_constant<int, 0>(), j);
+      for (int j = 0; j < 4; ++j)
+        if (PG == 1 || j < nrows) ldp1(std::integral_constant<int, 0>(), j);
       auto steps = [&](auto self, auto step_c) -> void {
         constexpr int st = decltype(step_c)::value;
         if constexpr (st < kSteps) {
@@ -328,7 +339,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           const u32x4 wfrag = wring[st % kRing];
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            if (st == 0 && slab == 0) {
+            const bool rowlive = PG == 1 || j < nrows;  // a pixel group may hold fewer rows (uniform per wave)
+            if (!rowlive) {
+            } else if (st == 0 && slab == 0) {
               // the first step of a tile starts the sums: a zero C operand instead of 64 cleared registers
               const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
               acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, wfrag), __builtin_bit_cast(half8, pr[st & 1][j]), zero, 0, 0, 0);
@@ -336,7 +349,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
               Mma<half_t>::run(wfrag, pr[st & 1][j], acc[j]);
             }
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (st + 1 < kSteps) ldp1(std::integral_constant<int, st + 1>(), j);
+            if constexpr (st + 1 < kSteps) {
+              if (rowlive) ldp1(std::integral_constant<int, st + 1>(), j);
+            }
             // the next patch: kLoadsPerWave pieces over the first K steps of the stage
             if constexpr (st * PPS < kLoadsPerWave) {
               if (j == 0) patch_piece_perm(std::integral_constant<int, st * PPS>());
@@ -415,10 +430,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const int owner = j / NOWN;
-            if ((NR == 1 || j / 2 == round) && owner != wk) {
+            if ((NR == 1 || j / 2 == round) && owner != wk && (PG == 1 || j < nrows)) {
               const int rank = wk < owner ? wk : wk - 1;  // position among the WK-1 senders
               const int jx = NR == 1 ? j : (j & 1), nj = NR == 1 ? 4 : 2;
-              unsigned char* dst = xb + (((wf * nj + jx) * (WK - 1) + rank) * 4) * 1024 + lane * 16;
+              unsigned char* dst = xb + ((((pg * WF + wf) * nj + jx) * (WK - 1) + rank) * 4) * 1024 + lane * 16;
 #pragma unroll
               for (int q = 0; q < 4; ++q)
                 *reinterpret_cast<floatx4*>(dst + q * 1024) = floatx4{acc[j][4 * q], acc[j][4 * q + 1], acc[j][4 * q + 2], acc[j][4 * q + 3]};
@@ -427,9 +442,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           __syncthreads();
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            if (j / NOWN == wk && (NR == 1 || j / 2 == round)) {
+            if (j / NOWN == wk && (NR == 1 || j / 2 == round) && (PG == 1 || j < nrows)) {
               const int jx = NR == 1 ? j : (j & 1), nj = NR == 1 ? 4 : 2;
-              const unsigned char* src = xb + (((wf * nj + jx) * (WK - 1)) * 4) * 1024 + lane * 16;
+              const unsigned char* src = xb + ((((pg * WF + wf) * nj + jx) * (WK - 1)) * 4) * 1024 + lane * 16;
 #pragma unroll
               for (int r = 0; r < WK - 1; ++r)
 #pragma unroll
@@ -453,7 +468,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        if (j / NOWN != wk) continue;
+        if (j / NOWN != wk || (PG > 1 && j >= nrows)) continue;
         const int o = j % NOWN;
         float y[FPL];
 #pragma unroll
@@ -520,16 +535,16 @@ struct StreamGeom {
 
 unsigned recip32(unsigned d) { return d == 1 ? 0u : (unsigned)(0xffffffffull / d + 1); }  // ceil(2^32 / d) for d >= 2
 
-// TH consecutive virtual rows of W columns per tile: at most kSlots pixels, and a patch of TH + 2 rows of
-// NSEG segments within kSegCap.  Aligned form: S = bands * TH >= H virtual rows per image, tiles never
+// TH consecutive virtual rows of W columns per tile: at most `slots` pixels, and a patch of TH + 2 rows of
+// NSEG segments within `segcap`.  Aligned form: S = bands * TH >= H virtual rows per image, tiles never
 // leave their image.  Gap form: S = H + 1 (one shared zero row between images), tiles of the largest TH
 // that fits.  The form with fewer tiles wins; aligned on a tie (it wastes no slot on the zero rows).
-bool stream_geometry(int N, int H, int W, StreamGeom* g) {
-  if (N < 1 || H < 1 || W < 1 || W > kSlots || H > 254 || N >= (1 << 24)) return false;
+bool stream_geometry(int N, int H, int W, int slots, int segcap, StreamGeom* g) {
+  if (N < 1 || H < 1 || W < 1 || W > slots || H > 254 || N >= (1 << 24)) return false;
   const int NSEG = (W + 2 + kSegCells - 1) / kSegCells;
   int thmax = 0;
   for (int th = 1; th <= H + 1; ++th)
-    if (th * W <= kSlots && (th + 2) * NSEG <= kSegCap) thmax = th;
+    if (th * W <= slots && (th + 2) * NSEG <= segcap) thmax = th;
   if (thmax == 0) return false;
   const int tha0 = std::min(thmax, H);
   const int bands = (H + tha0 - 1) / tha0, tha = (H + bands - 1) / bands;
@@ -577,6 +592,61 @@ __global__ void weight_frag32_kernel(const Ts* __restrict__ w, half_t* __restric
 long long* g_stamps = nullptr;
 #endif
 
+// The launch shape for a layer: pixel groups, filter groups and K groups of a workgroup, the tile geometry that goes
+// with them, and how the (filter block, tile list) pairs spread over the workgroups.
+struct StreamConfig {
+  int PG = 1, WF = 2, WK = 2;
+  StreamGeom geo;
+  int FB = 0;        // filter blocks of 32*WF
+  int Wpf = 0;       // workgroups per filter block = tile step of a workgroup
+  long long cost = 0;
+};
+
+// Candidates: four waves, two workgroups per CU -- 128 slots x 64 filters x 2 K groups, or x 32 filters x 4 K groups
+// when that is what it takes to fill the CUs; eight waves, one workgroup per CU -- 256 slots x 64 filters x 2 K groups.
+// The estimate is the matrix work of the busiest CU: its tiles x the tile's 32-slot rows x filter groups x K steps
+// (what the SIMDs of a CU share), plus a per-tile constant for the epilogue.  `only_pg` > 0 restricts the choice.
+bool stream_config(int N, int H, int W, int C, int F, bool act, int only_pg, StreamConfig* best) {
+  bool found = false;
+  for (int cand = 0; cand < (act ? 2 : 3); ++cand) {  // the eight-wave form exists with the ReLU epilogue only
+    StreamConfig c;
+    c.PG = cand == 2 ? 2 : 1;
+    c.WF = cand == 1 ? 1 : 2;
+    c.WK = 4 / c.WF;
+    // Measured, the eight-wave form loses to two independent workgroups of four (13.5 against 12.2 us on 28x28x128 at
+    // batch 32): its barriers stop both waves of every SIMD at once, where two workgroups drift apart and fill each
+    // other's waits.  It runs on request only (NNCV_HIP_STREAM_PG=2).
+    if (c.PG != (only_pg > 0 ? only_pg : 1)) continue;
+    if (F % (32 * c.WF) != 0) continue;
+    const int nw = 4 * c.PG;
+    if (!stream_geometry(N, H, W, kSlots * c.PG, seg_cap(nw), &c.geo)) continue;
+    c.FB = F / (32 * c.WF);
+    const int per_cu = c.PG == 1 ? 2 : 1;
+    // as many workgroups per filter block as the CUs hold, evened out so that all of them walk the same number of
+    // tiles (896 tiles on 512 places: 448 workgroups of two tiles, not 384 of two and 128 of one)
+    const int places = std::max(1, 256 * per_cu / c.FB), rounds = (c.geo.n_tiles + places - 1) / places;
+    c.Wpf = (c.geo.n_tiles + rounds - 1) / rounds;
+    const long long wgs = (long long)c.FB * c.Wpf;
+    const long long wg_per_cu = (wgs + 255) / 256;  // on the busiest CU
+    const int trows = (c.geo.TH * W + 31) / 32;
+    const long long ksteps = (long long)C / 64 * 36;
+    c.cost = wg_per_cu * rounds * ((long long)trows * c.WF * ksteps + 600);
+    if (!found || c.cost < best->cost) {
+      *best = c;
+      found = true;
+    }
+  }
+  return found;
+}
+
+int stream_force_pg() {
+  static const int v = [] {
+    const char* e = getenv("NNCV_HIP_STREAM_PG");
+    return e ? atoi(e) : 0;
+  }();
+  return v;
+}
+
 }  // namespace
 
 #ifdef NNCV_STREAM_STAMPS
@@ -595,56 +665,53 @@ void launch_weight_frag32(const void* w, int w_dt, void* dst, int F, int C, hipS
   NNCV_HIP_CHECK(hipGetLastError());
 }
 
-bool conv3x3_stream_plan(int N, int H, int W, int out[8]) {
-  StreamGeom g;
-  if (!stream_geometry(N, H, W, &g)) return false;
-  out[0] = g.TH; out[1] = g.S; out[2] = g.top; out[3] = g.aligned; out[4] = g.top; out[5] = g.n_tiles; out[6] = (g.TH + 2) * g.NSEG; out[7] = g.NSEG;
+bool conv3x3_stream_plan(int N, int H, int W, int C, int F, int out[12]) {
+  StreamConfig c;
+  if (!stream_config(N, H, W, C, F, false, 0, &c)) return false;
+  const StreamGeom& g = c.geo;
+  out[0] = g.TH; out[1] = g.S; out[2] = g.top; out[3] = g.aligned; out[4] = g.n_tiles; out[5] = g.NSEG;
+  out[6] = c.PG; out[7] = c.WF; out[8] = c.WK; out[9] = c.FB; out[10] = c.Wpf; out[11] = seg_cap(4 * c.PG);
   return true;
 }
 
 bool conv3x3_stream_applicable(const IgemmArgs& a, int in_dt, int out_dt) {
   static const bool off = getenv("NNCV_HIP_NO_STREAM") != nullptr;
-  // deeper layers (more than two channel slabs per tile) stay with the patch kernel unless asked for: their
-  // stages are nine K steps long and the per-stage work of this kernel shows
+  // The deepest layers (eight channel slabs per tile, few pixels) stay with the patch kernel unless asked for: 16.6 us
+  // here against 13.1 there on 7x7x512 at batch 32; up to 256 channels this kernel is 5-8 % ahead.
   static const bool all = getenv("NNCV_HIP_STREAM_ALL") != nullptr;
-  if (off || in_dt != kF16 || out_dt != kF16 || !a.wt_frag32 || (a.C > 128 && !all)) return false;
+  if (off || in_dt != kF16 || out_dt != kF16 || !a.wt_frag32 || (a.C > 256 && !all)) return false;
   const int pix = a.pix_stride ? a.pix_stride : a.C;
   const bool act_ok = a.relu <= kActRelu || ((a.relu & 0xff) <= kActSigmoid && (a.relu & ~(0xff | kActResidualAfter)) == 0);
-  StreamGeom g;
+  StreamConfig c;
   return act_ok && a.aux_f0 == 0 && a.R == 3 && a.S == 3 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 1 && a.pad_w == 1 &&
          a.OH == a.H && a.OW == a.W && a.batch == 1 && a.C % 64 == 0 && a.F % 32 == 0 && pix % 8 == 0 && a.ldo % 8 == 0 && a.ldo >= a.F &&
          (long long)a.N * a.H * a.W * a.ldo * 2 < (1ll << 31) && (long long)a.N * a.H * a.W * pix * 2 < (1ll << 31) &&
-         a.in_bytes < kOOBs && (long long)a.F * 9 * a.C * 2 < (1ll << 31) && stream_geometry(a.N, a.H, a.W, &g);
+         a.in_bytes < kOOBs && (long long)a.F * 9 * a.C * 2 < (1ll << 31) && stream_config(a.N, a.H, a.W, a.C, a.F, a.relu > kActRelu, stream_force_pg(), &c);
 }
 
-template <int WF, int WK, bool ACT>
+template <int PG, int WF, int WK, bool ACT>
 static void launch_stream_cfg(const StreamArgs& a, int grid, double flops, double bytes, const char* tag, hipStream_t s) {
-  auto kern = conv3x3_f16_stream_kernel<WF, WK, ACT>;
-  constexpr int smem = 2 * kPatchB + 2 * 32 * WF * 4;
+  auto kern = conv3x3_f16_stream_kernel<PG, WF, WK, ACT>;
+  constexpr int NW = PG * WF * WK;
+  constexpr int smem = 2 * patch_bytes(NW) + 2 * 32 * WF * 4;
   static const bool attr = [&] {
     NNCV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
     return true;
   }();
   (void)attr;
   ProfScope prof(tag, flops, bytes, s);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), smem, s, a);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), smem, s, a);
 }
 
 bool launch_conv3x3_stream(const IgemmArgs& g, hipStream_t s) {
-  StreamGeom geo;
-  if (!stream_geometry(g.N, g.H, g.W, &geo)) return false;
-  // 64-filter blocks (two filter groups x two K groups) by default; 32-filter blocks (four K groups) when that is
-  // what it takes to give every CU two workgroups
-  const bool narrow = g.F % 64 != 0 || (long long)geo.n_tiles * (g.F / 64) < 384;
-  const int FB = narrow ? g.F / 32 : g.F / 64;
+  StreamConfig cfg;
+  if (!stream_config(g.N, g.H, g.W, g.C, g.F, g.relu > kActRelu, stream_force_pg(), &cfg)) return false;
+  const StreamGeom& geo = cfg.geo;
+  const int FB = cfg.FB, Wpf = cfg.Wpf;
   const size_t wbytes = weight_frag32_bytes(g.F, g.C);
   // An XCD's workgroups are neighbours: a contiguous range of tile lists (tiles that share halo rows meet in one
   // L2) with all filter blocks, or -- when the filters outgrow an L2 -- a range of filter blocks with all lists.
   const bool by_filter = FB % kXcds == 0 && wbytes > (2u << 20);
-  // as many workgroups per filter block as two per CU allow, evened out so that all of them walk the
-  // same number of tiles (896 tiles on 512 places: 448 workgroups of two tiles, not 384 of two and 128 of one)
-  const int places = std::max(1, 512 / FB), rounds = (geo.n_tiles + places - 1) / places;
-  const int Wpf = (geo.n_tiles + rounds - 1) / rounds;
   const int G = FB * Wpf, grid = (G + kXcds - 1) / kXcds * kXcds;
   NNCV_REQUIRE(Wpf < 65536 && g.C / 64 < 256, "conv3x3_stream: tile step / slab count out of range");
   StreamArgs a{};
@@ -671,12 +738,14 @@ bool launch_conv3x3_stream(const IgemmArgs& g, hipStream_t s) {
   const double flops = 2.0 * P * g.C * 9.0 * g.F;
   const double bytes = 2.0 * (P * g.C + 9.0 * g.C * g.F + P * g.F * (g.residual ? 2 : 1));
   const bool act = g.relu > kActRelu;
-  if (narrow) {
-    if (act) launch_stream_cfg<1, 4, true>(a, grid, flops, bytes, "conv3x3_stream<f16,1,4,act>", s);
-    else launch_stream_cfg<1, 4, false>(a, grid, flops, bytes, "conv3x3_stream<f16,1,4>", s);
+  if (cfg.PG == 2) {
+    launch_stream_cfg<2, 2, 2, false>(a, grid, flops, bytes, "conv3x3_stream<f16,2x2x2>", s);
+  } else if (cfg.WF == 1) {
+    if (act) launch_stream_cfg<1, 1, 4, true>(a, grid, flops, bytes, "conv3x3_stream<f16,1x1x4,act>", s);
+    else launch_stream_cfg<1, 1, 4, false>(a, grid, flops, bytes, "conv3x3_stream<f16,1x1x4>", s);
   } else {
-    if (act) launch_stream_cfg<2, 2, true>(a, grid, flops, bytes, "conv3x3_stream<f16,2,2,act>", s);
-    else launch_stream_cfg<2, 2, false>(a, grid, flops, bytes, "conv3x3_stream<f16,2,2>", s);
+    if (act) launch_stream_cfg<1, 2, 2, true>(a, grid, flops, bytes, "conv3x3_stream<f16,1x2x2,act>", s);
+    else launch_stream_cfg<1, 2, 2, false>(a, grid, flops, bytes, "conv3x3_stream<f16,1x2x2>", s);
   }
   NNCV_HIP_CHECK(hipGetLastError());
   return true;

@@ -109,6 +109,14 @@ int nncv_hip_conv_algo(const nncv_hip_conv* c);
  * in is [N,C,H,W] UNPADDED, out [N,F,OH,OW]; residual may be NULL. NHWC is the native layout. */
 int nncv_hip_conv_forward(nncv_hip_conv* c, const void* in, int N, int H, int W, int layout, const void* residual,
                           void* out, void* stream);
+/* The same as nncv_hip_conv_forward with layout = 1 (NHWC), for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  The
+ * workspace the layer's kernels need (the partial sums and ticket counters of the K split of fp32 3x3 layers) is a
+ * device array of the library, 4 MiB + 1 KiB on every GPU it runs on, held until the process ends; the call allocates
+ * and frees nothing.  A layer/shape whose workspace is larger fails with an error that says so.  All calls on one GPU
+ * share the array: calls that overlap in time on one GPU race (calls on one stream, or ordered by events, do not). */
+int nncv_hip_conv_forward_noalloc(nncv_hip_conv* c, const void* in, int N, int H, int W, const void* residual, void* out,
+                                  void* stream);
 /* Measurement helper: `reps` NHWC launches of the layer back to back on `stream` between one pair
  * of HIP events (after 5 untimed ones); *avg_us = elapsed / reps. Includes the gap between
  * consecutive dispatches, so it reads slightly above a profiler's per-kernel time. */

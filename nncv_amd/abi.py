@@ -35,7 +35,7 @@ EXPORTS = [
     "nncv_hip_profile_enable", "nncv_hip_profile_report",
     "nncv_hip_resnet18_create", "nncv_hip_resnet18_destroy", "nncv_hip_resnet18_forward",
     "nncv_hip_resnet18_forward_tap",
-    "nncv_hip_conv_create", "nncv_hip_conv_destroy", "nncv_hip_conv_algo", "nncv_hip_conv_forward", "nncv_hip_conv_time", "nncv_hip_conv3x3_patch_plan",
+    "nncv_hip_conv_create", "nncv_hip_conv_destroy", "nncv_hip_conv_algo", "nncv_hip_conv_forward", "nncv_hip_conv_forward_noalloc", "nncv_hip_conv_time", "nncv_hip_conv3x3_patch_plan",
     "nncv_hip_plan_arena", "nncv_hip_preprocess_u8", "nncv_hip_argmax", "nncv_hip_resnet18_classify_u8",
     "nncv_hip_matmul_f32", "nncv_hip_wino43_filter", "nncv_hip_wino43_input", "nncv_hip_wino43_gemm",
     "nncv_hip_wino43_output", "nncv_hip_maxpool3x3s2", "nncv_hip_global_avgpool",
@@ -109,6 +109,7 @@ def lib():
         L.nncv_hip_conv_destroy.restype = None
         L.nncv_hip_conv_algo.argtypes = [vp]
         L.nncv_hip_conv_forward.argtypes = [vp, vp, i, i, i, i, vp, vp, vp]
+        L.nncv_hip_conv_forward_noalloc.argtypes = [vp, vp, i, i, i, vp, vp, vp]
         L.nncv_hip_conv_time.argtypes = [vp, vp, i, i, i, vp, vp, i, vp, P(ctypes.c_float)]
         L.nncv_hip_matmul_f32.argtypes = [vp, vp, vp, i, i, i, vp]
         L.nncv_hip_plan_arena.argtypes = [i, P(i), P(i), P(ctypes.c_uint64), ctypes.c_uint64, P(ctypes.c_uint64)]

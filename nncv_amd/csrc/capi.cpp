@@ -37,6 +37,7 @@ void Context::init(int device) {
   NNCV_HIP_CHECK(hipEventCreateWithFlags(&tail_event_, hipEventDisableTiming));
   device_ = device;
   ready_ = true;
+  (void)noalloc_scratch();  // the scratch array's address on this device, resolved with the device current
 }
 
 void Context::order_after_previous(hipStream_t s) {
@@ -689,6 +690,25 @@ int nncv_hip_conv_forward(nncv_hip_conv* c, const void* in, int N, int H, int W,
       L.forward_strided(in, strides_of(kNCHW, L.desc().C, H, W), N, H, W, residual, out, strides_of(kNCHW, L.desc().F, OH, OW),
                         false, ws, sy.s);
     }
+    sy.finish();
+  });
+}
+
+int nncv_hip_conv_forward_noalloc(nncv_hip_conv* c, const void* in, int N, int H, int W, const void* residual, void* out,
+                                  void* stream) {
+  return guarded([&] {
+    NNCV_REQUIRE(c && c->c && in && out, "null argument");
+    const ConvLayer& L = *c->c;
+    const size_t wsb = L.workspace_bytes(N, H, W, false);
+    NNCV_REQUIRE(wsb <= kNoAllocWorkspaceBytes,
+                 "nncv_hip_conv_forward_noalloc: this layer and shape need " + std::to_string(wsb) + " bytes of workspace, the "
+                 "scratch array holds " + std::to_string(kNoAllocWorkspaceBytes) + "; use nncv_hip_conv_forward");
+    static_assert(ConvLayer::kSplitKCounterInts * sizeof(int) <= kNoAllocCounterBytes, "ticket counters outgrow their slot");
+    Sync sy(stream);
+    char* scratch = static_cast<char*>(noalloc_scratch());
+    // the array keeps the previous call's contents: the tickets must start at zero (the workspace is written before it is read)
+    launch_clear_words(scratch, ConvLayer::kSplitKCounterInts, sy.s);
+    L.forward(in, N, H, W, residual, out, scratch + kNoAllocCounterBytes, sy.s, reinterpret_cast<int*>(scratch));
     sy.finish();
   });
 }

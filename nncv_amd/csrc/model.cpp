@@ -18,7 +18,7 @@ static int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
 // scratch of the patch kernel's K split: at most 256 workgroups' 64x64 fp32 partial tiles
 constexpr size_t kSplitKWsBytes = 256 * 4096 * sizeof(float);
-constexpr int kSplitKCounters = 256;
+constexpr int kSplitKCounters = ConvLayer::kSplitKCounterInts;
 
 ConvLayer::ConvLayer(const Desc& d, const void* w, const void* gamma, const void* beta, const void* mean, const void* var,
                      hipStream_t s)
@@ -106,7 +106,8 @@ size_t ConvLayer::workspace_bytes(int N, int H, int W, bool strided) const {
   return b;
 }
 
-void ConvLayer::forward(const void* in, int N, int H, int W, const void* residual, void* out, void* ws, hipStream_t s) const {
+void ConvLayer::forward(const void* in, int N, int H, int W, const void* residual, void* out, void* ws, hipStream_t s,
+                        int* counters) const {
   const int OH = out_h(H), OW = out_w(W);
   NNCV_REQUIRE(N > 0 && OH > 0 && OW > 0, "conv: empty tensor");
   const size_t es = dtype_size(d_.dt);
@@ -138,7 +139,7 @@ void ConvLayer::forward(const void* in, int N, int H, int W, const void* residua
   a.relu = d_.relu; a.ldo = d_.F; a.batch = 1;
   if (ws && splitk_counters_.get()) {
     a.splitk_ws = ws; a.splitk_ws_bytes = kSplitKWsBytes;
-    a.splitk_counters = splitk_counters_.as<int>(); a.splitk_counters_n = kSplitKCounters;
+    a.splitk_counters = counters ? counters : splitk_counters_.as<int>(); a.splitk_counters_n = kSplitKCounters;
   }
   launch_igemm(a, d_.dt, d_.dt, s);
 }

@@ -36,8 +36,11 @@ class ConvLayer {
   int out_w(int W) const { return (W + 2 * d_.pad - d_.S) / d_.stride + 1; }
   size_t workspace_bytes(int N, int H, int W, bool strided = false) const;
   // in/out/residual: NHWC device tensors of type dt (stem: `in` is NCHW [N,3,H,W]).
-  // `ws` must hold workspace_bytes().
-  void forward(const void* in, int N, int H, int W, const void* residual, void* out, void* ws, hipStream_t s) const;
+  // `ws` must hold workspace_bytes().  `counters`: kSplitKCounterInts zeroed ints to use as the K split's tickets
+  // instead of the layer's own (null = the layer's own).
+  void forward(const void* in, int N, int H, int W, const void* residual, void* out, void* ws, hipStream_t s,
+               int* counters = nullptr) const;
+  static constexpr int kSplitKCounterInts = 256;
   // generic-layout form used by the operator-level ABI: strides for in / out (residual shares out's)
   void forward_strided(const void* in, Strides4 in_st, int N, int H, int W, const void* residual, void* out, Strides4 out_st,
                        bool accumulate, void* ws, hipStream_t s) const;

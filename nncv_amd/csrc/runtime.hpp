@@ -86,6 +86,14 @@ class Arena {
 
 inline size_t align256(size_t b) { return (b + 255) & ~size_t(255); }
 
+// The device array behind nncv_hip_conv_forward_noalloc (noalloc.hip): 1 KiB of ticket counters, then the
+// workspace.  noalloc_scratch() is its address on the current device (resolved once per device).
+constexpr size_t kNoAllocCounterBytes = 1024;
+constexpr size_t kNoAllocWorkspaceBytes = size_t(4) << 20;
+constexpr size_t kNoAllocScratchBytes = kNoAllocCounterBytes + kNoAllocWorkspaceBytes;
+void* noalloc_scratch();
+void launch_clear_words(void* p, int n_words, hipStream_t s);
+
 // Process-wide state.  All public entry points serialise on `mu`.
 class Context {
  public:

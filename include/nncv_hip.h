@@ -154,6 +154,9 @@ unsigned long long nncv_hip_plan_arena(int n, const int* first_op, const int* la
                                        unsigned long long align, unsigned long long* offsets);
 
 int nncv_hip_matmul_f32(const float* A, const float* B, float* C, int M, int N, int K, void* stream);
+/* Measurement helper, like nncv_hip_conv_time: `reps` launches of C += A.B back to back on `stream` between one pair
+ * of HIP events (after 5 untimed ones); *avg_us = elapsed / reps.  C keeps accumulating. */
+int nncv_hip_matmul_time(const float* A, const float* B, float* C, int M, int N, int K, int reps, void* stream, float* avg_us);
 
 /* Winograd F(4x4,3x3) stages on DEVICE buffers (layouts: U[36][F][C], V[36][tiles][C], M[36][tiles][F],
  * tiles = N*ceil(OH/4)*ceil(OW/4)); exposed so each stage can be checked and profiled alone. */

@@ -37,7 +37,7 @@ EXPORTS = [
     "nncv_hip_resnet18_forward_tap",
     "nncv_hip_conv_create", "nncv_hip_conv_destroy", "nncv_hip_conv_algo", "nncv_hip_conv_forward", "nncv_hip_conv_forward_noalloc", "nncv_hip_conv_time", "nncv_hip_conv3x3_patch_plan",
     "nncv_hip_plan_arena", "nncv_hip_preprocess_u8", "nncv_hip_argmax", "nncv_hip_resnet18_classify_u8",
-    "nncv_hip_matmul_f32", "nncv_hip_wino43_filter", "nncv_hip_wino43_input", "nncv_hip_wino43_gemm",
+    "nncv_hip_matmul_f32", "nncv_hip_matmul_time", "nncv_hip_wino43_filter", "nncv_hip_wino43_input", "nncv_hip_wino43_gemm",
     "nncv_hip_wino43_output", "nncv_hip_maxpool3x3s2", "nncv_hip_global_avgpool",
     "nncv_hip_graph_create", "nncv_hip_graph_destroy", "nncv_hip_graph_output_shape", "nncv_hip_graph_forward",
     "nncv_hip_graph_plan", "nncv_hip_mobilenetv3_small_ops", "nncv_hip_dwconv", "nncv_hip_scale_channels", "nncv_hip_eltwise",
@@ -112,6 +112,7 @@ def lib():
         L.nncv_hip_conv_forward_noalloc.argtypes = [vp, vp, i, i, i, vp, vp, vp]
         L.nncv_hip_conv_time.argtypes = [vp, vp, i, i, i, vp, vp, i, vp, P(ctypes.c_float)]
         L.nncv_hip_matmul_f32.argtypes = [vp, vp, vp, i, i, i, vp]
+        L.nncv_hip_matmul_time.argtypes = [vp, vp, vp, i, i, i, i, vp, ctypes.POINTER(ctypes.c_float)]
         L.nncv_hip_plan_arena.argtypes = [i, P(i), P(i), P(ctypes.c_uint64), ctypes.c_uint64, P(ctypes.c_uint64)]
         L.nncv_hip_plan_arena.restype = ctypes.c_uint64
         L.nncv_hip_preprocess_u8.argtypes = [vp, i, i, i, i, i, vp, vp]

@@ -757,6 +757,28 @@ unsigned long long nncv_hip_plan_arena(int n, const int* first_op, const int* la
   return rc == 0 ? total : ~0ull;
 }
 
+int nncv_hip_matmul_time(const float* A, const float* B, float* C, int M, int N, int K, int reps, void* stream, float* avg_us) {
+  return guarded([&] {
+    NNCV_REQUIRE(A && B && C && avg_us && reps > 0, "null argument");
+    Context::get().init(-1);
+    Sync sy(stream);
+    hipEvent_t e0, e1;
+    NNCV_HIP_CHECK(hipEventCreate(&e0));
+    NNCV_HIP_CHECK(hipEventCreate(&e1));
+    for (int i = 0; i < 5; ++i) launch_gemm_nn_f32(A, B, C, M, N, K, sy.s);
+    NNCV_HIP_CHECK(hipEventRecord(e0, sy.s));
+    for (int i = 0; i < reps; ++i) launch_gemm_nn_f32(A, B, C, M, N, K, sy.s);
+    NNCV_HIP_CHECK(hipEventRecord(e1, sy.s));
+    NNCV_HIP_CHECK(hipEventSynchronize(e1));
+    float ms = 0.0f;
+    NNCV_HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    *avg_us = ms * 1000.0f / (float)reps;
+    sy.finish();
+  });
+}
+
 int nncv_hip_matmul_f32(const float* A, const float* B, float* C, int M, int N, int K, void* stream) {
   return guarded([&] {
     NNCV_REQUIRE(A && B && C, "null argument");

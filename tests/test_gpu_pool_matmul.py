@@ -41,7 +41,11 @@ def test_global_avgpool(dt, N, C, H, W):
     assert np.abs(host(out) - want).max() <= tol * max(1.0, np.abs(want).max())
 
 
-@pytest.mark.parametrize("M,N,K", [(1024, 1024, 1024), (130, 68, 36), (64, 64, 16), (257, 512, 1000), (1, 4, 4)])
+# linalg.matmul puts no condition on M, N, K: odd sizes (rows that are not 16-byte multiples) take the element-wise
+# loader; the sizes also walk the launch shapes: 128x128 tiles, 64x64 tiles with 1, 2 and 4 K groups
+@pytest.mark.parametrize("M,N,K", [(1024, 1024, 1024), (130, 68, 36), (64, 64, 16), (257, 512, 1000), (1, 4, 4),
+                                   (33, 17, 5), (1, 1, 1), (65, 130, 259), (1000, 1001, 127), (2048, 2048, 64), (300, 200, 130),
+                                   (1500, 1300, 200), (97, 1, 1031)])
 def test_matmul_device(M, N, K):
     a = synth.uniform(320, (M, K), -1, 1)
     b = synth.uniform(321, (K, N), -1, 1)
@@ -67,3 +71,27 @@ def test_cfg1_matmul_through_reference_abi():
     c2 = np.zeros((1024, 1024), np.float32)
     abi.matmul(at, b, c2)
     assert np.array_equal(c, c2)
+
+
+def test_matmul_through_reference_abi_any_shape():
+    """The reference's compiled linalg.matmul takes any M, N, K; so does the symbol here (no abort on rows that are
+    not multiples of 16 bytes)."""
+    for (M, N, K) in ((33, 17, 5), (7, 9, 3)):
+        a = synth.uniform(330, (M, K), -1, 1)
+        b = synth.uniform(331, (K, N), -1, 1)
+        c = synth.uniform(332, (M, N), -1, 1)
+        want = oracle.matmul(a, b, c)
+        abi.matmul(a, b, c)
+        assert max_rel(c, want) < FP32_MAX_REL
+
+
+def test_matmul_k_groups_are_deterministic():
+    """The K groups of a workgroup meet in a fixed order: two runs give the same bits."""
+    a, b = synth.cfg1_matmul()
+    ad, bd = dev(a), dev(b)
+    outs = []
+    for _ in range(2):
+        c = dev(np.zeros((1024, 1024), np.float32))
+        abi.check(abi.lib().nncv_hip_matmul_f32(ad.data_ptr(), bd.data_ptr(), c.data_ptr(), 1024, 1024, 1024, None))
+        outs.append(host(c))
+    assert np.array_equal(outs[0], outs[1])

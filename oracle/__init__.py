@@ -447,6 +447,7 @@ def hwp_lib():
             raise RuntimeError("%s is missing: run `make -C oracle`" % p)
         L = ctypes.CDLL(p)
         L.hwp_conv2d_nchw_fchw.argtypes = [_f32p, _f32p, _f32p] + [ctypes.c_int] * 9
+        L.hwp_conv2d_ref_schedule.argtypes = [_f32p, _f32p, _f32p] + [ctypes.c_int] * 9
         L.hwp_set_num_threads.argtypes = [ctypes.c_int]
         L.hwp_set_num_threads.restype = None
         _HWP = L
@@ -460,22 +461,26 @@ def hwp_threads(n=None):
     return int(hwp_lib().hwp_num_threads())
 
 
-def hwp_conv2d(x, w, stride=1, pad=0):
-    """conv_2d_nchw_fchw over a zero halo of `pad`, fp32 accumulation, OpenMP x AVX2."""
+def hwp_conv2d(x, w, stride=1, pad=0, schedule="omp"):
+    """conv_2d_nchw_fchw over a zero halo of `pad`, fp32 accumulation.  schedule "omp": this repository's own OpenMP x
+    AVX2 routine; "ref": the reference's tile order, sequential (ModernTile.cpp:184-199, :330-331)."""
     x, w = _c(x), _c(w)
     N, C, H, W = x.shape
     F, C2, R, S = w.shape
     assert C == C2
     OH, OW = (H + 2 * pad - R) // stride + 1, (W + 2 * pad - S) // stride + 1
     y = np.empty((N, F, OH, OW), np.float32)
-    rc = hwp_lib().hwp_conv2d_nchw_fchw(x, w, y, N, C, H, W, F, R, S, stride, pad)
+    fn = hwp_lib().hwp_conv2d_nchw_fchw if schedule == "omp" else hwp_lib().hwp_conv2d_ref_schedule
+    rc = fn(x, w, y, N, C, H, W, F, R, S, stride, pad)
     assert rc == 0
     return y
 
 
-def hwp_resnet18_forward(x, params):
-    """ResNet-18 of tests/Nets/Res18.mlir with the convolutions on the AVX2/OpenMP routine above and
-    every other op on the scalar oracle's; same parameter blob order as resnet18_forward."""
+def hwp_resnet18_forward(x, params, schedule="omp"):
+    """ResNet-18 of tests/Nets/Res18.mlir with the convolutions on one of the AVX2 routines above (`schedule` as in
+    hwp_conv2d) and every other op on the scalar oracle's; same parameter blob order as resnet18_forward."""
+    import functools
+    hwp_conv2d = functools.partial(globals()["hwp_conv2d"], schedule=schedule)
     from nncv_amd import resnet18_spec as spec
     x, params = _c(x), _c(params)
     tensors, off = {}, 0

@@ -166,22 +166,25 @@ def test_winograd_equals_direct_ragged(H, W):
     assert V.shape == (36, 2 * ((H + 3) // 4) * ((W + 3) // 4), 5)
 
 
+@pytest.mark.parametrize("schedule", ["omp", "ref"])
 @pytest.mark.parametrize("R,stride,pad", [(3, 1, 1), (3, 2, 1), (1, 2, 0), (7, 2, 3), (3, 1, 0)])
-def test_hostwparallel_conv_matches_scalar_oracle(R, stride, pad):
-    """The AVX2/OpenMP convolution timed as the CPU baseline computes the same convolution as the
-    scalar oracle (fp32 vs fp64 accumulation: agreement to fp32 rounding), ragged sizes included."""
+def test_hostwparallel_conv_matches_scalar_oracle(R, stride, pad, schedule):
+    """Both AVX2 convolutions timed as CPU baselines (the OpenMP one and the reference's sequential tile order) compute
+    the same convolution as the scalar oracle (fp32 vs fp64 accumulation: agreement to fp32 rounding), ragged sizes and
+    filter counts that are not multiples of 8 included."""
     x = synth.normal(910, (2, 12, 19, 23))
     w = synth.normal(911, (10, 12, R, R), std=0.2)
-    got = oracle.hwp_conv2d(x, w, stride, pad)
+    got = oracle.hwp_conv2d(x, w, stride, pad, schedule=schedule)
     want = oracle.conv2d_nchw_fchw(oracle.pad_nchw(x, pad), w, stride=stride)
     assert got.shape == want.shape
     assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max()
 
 
-def test_hostwparallel_resnet18_matches_scalar_oracle():
+@pytest.mark.parametrize("schedule", ["omp", "ref"])
+def test_hostwparallel_resnet18_matches_scalar_oracle(schedule):
     blob = synth.resnet18_params()
     x = synth.uniform(912, (1, 3, 64, 96), 0.0, 1.0)
-    got = oracle.hwp_resnet18_forward(x, blob)
+    got = oracle.hwp_resnet18_forward(x, blob, schedule=schedule)
     want = oracle.resnet18_forward(x, blob)
     assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
     assert got.argmax(1) == want.argmax(1)

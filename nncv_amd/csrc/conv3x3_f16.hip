@@ -19,9 +19,17 @@
 //    rows.  Either every image takes a whole number of tiles (aligned form), or the images are one zero
 //    row apart and tiles run across image borders (gap form: that shared row is the halo of both images);
 //    14x14 and 7x7 images fill 126 of 128 slots that way instead of 98.
-//  * Patch cells are 128 bytes apart and their eight 16-byte chunks are stored XOR-swizzled with bits 1..3
-//    of the cell number: the direct-to-LDS load needs whole kilobytes per wave instruction, and the
-//    swizzle keeps the 16-byte reads of 16 neighbouring cells on distinct banks.
+//  * Patch cells (the 64 channels of one pixel, 128 bytes) are 144 bytes apart in LDS, which keeps the 16-byte
+//    reads of 32 neighbouring cells off each other's banks.  A load instruction fills a row segment of seven
+//    cells: 63 lanes x 16 bytes = 7 x 144 (lane 63 writes what lane 0 of the next segment overwrites).
+//    Which pixel a lane fetches is worked out once per tile, one segment per lane, and dealt to the nine
+//    load instructions of a wave with ds_bpermute; a lane whose cell is padding, halo outside the image or
+//    past the tile asks for an offset beyond the buffer and gets zeros.  Every wave issues all nine loads
+//    in every stage, so the compiler's count of outstanding loads is exact and the weight ring is never
+//    over-waited.
+//  * Inside a stage each MFMA is followed by its share of the other work (next K step's LDS reads, a weight
+//    refill, a piece of the next patch) and pinned there, so the matrix pipe is issued to at a steady rate.
+//    The two workgroups of a CU take turns at the higher wave priority, tile by tile.
 //  * The filters of a wave are stored permuted (row 8q+4h+e of the MFMA holds filter 16h+4q+e), so a
 //    lane ends up with 16 consecutive output channels of a pixel: results go from the accumulators to
 //    memory with two 16-byte stores, without a transposing pass through LDS.  K groups (the waves that
@@ -76,9 +84,6 @@ struct StreamArgs {
   const void* residual;   // like out, or null
   unsigned out_bytes, mW16;  // mW16 = ceil(2^16 / W)
   int F, act, ldo;
-#ifdef NNCV_STREAM_STAMPS
-  long long* stamps;
-#endif
 };
 static_assert(offsetof(StreamArgs, out) == 64, "sixteen preloaded dwords");
 
@@ -105,10 +110,6 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
   // weight refills younger than the last patch piece at the end of a stage: what the wait for the patch may leave in flight
   constexpr int kYoung = kSteps - kPieceSteps < kRing ? kSteps - kPieceSteps : kRing;
   extern __shared__ __align__(16) unsigned char smem[];
-#ifdef NNCV_STREAM_STAMPS
-  long long ts[8] = {clock64(), 0, 0, 0, 0, 0, 0, 0};
-  const long long wall0 = wall_clock64();
-#endif
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -136,9 +137,6 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
   int tile = (int)(by_filter ? rd : qd);
   const int tend = (int)a.n_tiles;
   if (tile >= tend) return;
-#ifdef NNCV_STREAM_STAMPS
-  ts[6] = clock64();
-#endif
 
   const __amdgpu_buffer_rsrc_t rs_wf = make_rsrc(a.wf, a.wf_bytes);
 
@@ -212,18 +210,19 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
     // range (the two flags cancel): that unit then loads the tensor's first bytes into a pad nobody reads
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_in, (lds_ptr_t)(smem + pc_dst + pp * kSegB), 16, pc_vo + pc_lchslab, 0, 0, 0);
   };
-  auto patch_all = [&](auto self, auto p_c) -> void {
-    constexpr int pp = decltype(p_c)::value;
-    if constexpr (pp < kLoadsPerWave) {
-      patch_piece_perm(p_c);
-      patch_piece_load(p_c);
-      self(self, std::integral_constant<int, pp + 1>());
-    }
+  // the first patch of a workgroup: nothing to hide the permutes' latency under, so all nine go out before the loads
+  auto patch_all = [&]() {
+    unsigned pv[kLoadsPerWave];
+#pragma unroll
+    for (int pp = 0; pp < kLoadsPerWave; ++pp) pv[pp] = (unsigned)__builtin_amdgcn_ds_bpermute(perm0 + 28 * pp, (int)celloff);
+#pragma unroll
+    for (int pp = 0; pp < kLoadsPerWave; ++pp)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_in, (lds_ptr_t)(smem + pc_dst + pp * kSegB), 16, pv[pp] + pc_lchslab, 0, 0, 0);
   };
 
   patch_tile(tile, true);
   patch_begin(0, 0);
-  patch_all(patch_all, std::integral_constant<int, 0>());
+  patch_all();
   __builtin_amdgcn_sched_barrier(0);
   ring_fill(std::integral_constant<int, 3>());
   ring_fill(std::integral_constant<int, 4>());
@@ -232,9 +231,6 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
   ring_fill(std::integral_constant<int, 7>());
   ring_fill(std::integral_constant<int, 8>());
   __builtin_amdgcn_sched_barrier(0);
-#ifdef NNCV_STREAM_STAMPS
-  ts[1] = clock64();
-#endif
 
   // ---- everything below needs the rest of the arguments ----
   const __amdgpu_buffer_rsrc_t rs_out = make_rsrc(a.out, a.out_bytes);
@@ -288,13 +284,7 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
   // the first patch is older than the six fragments and the two scale / shift loads requested after it
   __builtin_amdgcn_s_waitcnt(vmcnt_only(8));
   __syncthreads();
-#ifdef NNCV_STREAM_STAMPS
-  ts[2] = clock64();
-#endif
 
-#ifdef NNCV_STREAM_STEPSTAMPS
-  int fine_idx = 0;
-#endif
   int stage_no = 0;
   int cur = 0;      // LDS offset of the buffer the taps read
   int wo = 0;       // byte offset of the current stage's first iteration in the weight stream
@@ -339,10 +329,6 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
       auto steps = [&](auto self, auto step_c) -> void {
         constexpr int st = decltype(step_c)::value;
         if constexpr (st < kSteps) {
-#ifdef NNCV_STREAM_STEPSTAMPS
-          if (a.stamps && lane == 0 && fine_idx < 60) a.stamps[65536 + (blockIdx.x * 4 + wave) * 64 + fine_idx] = clock64();
-          ++fine_idx;
-#endif
           constexpr int PPS = (kLoadsPerWave + kPieceSteps - 1) / kPieceSteps;  // patch pieces per step: 1 or 2
           constexpr int nx = st + kRing, nt = nx / KPG, nk = nx % KPG;
           static_assert(nt < 18, "the ring reaches at most into the next stage");
@@ -417,13 +403,6 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
 #pragma unroll
         for (int j = 0; j < 4; ++j) rowbase[r][j] += delta;
       if (!last) continue;
-#ifdef NNCV_STREAM_STAMPS
-      if (ts[3] == 0) ts[3] = clock64();
-#endif
-#ifdef NNCV_STREAM_STEPSTAMPS
-      if (a.stamps && lane == 0 && fine_idx < 60) a.stamps[65536 + (blockIdx.x * 4 + wave) * 64 + fine_idx] = clock64();
-      ++fine_idx;
-#endif
 
       // ---- end of a tile: K groups exchange partial sums through the buffer the taps just left, then
       //      scale/shift, residual, activation, one rounding, two 16-byte stores per pixel ----
@@ -467,9 +446,6 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
           }
         }
       }
-#ifdef NNCV_STREAM_STAMPS
-      if (ts[4] == 0) ts[4] = clock64();
-#endif
       floatx4 sc4[4], sh4[4];
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
@@ -524,17 +500,6 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
     tile = next_tile;
     tile_outputs(tile);
   }
-#ifdef NNCV_STREAM_STAMPS
-  ts[5] = clock64();
-  if (a.stamps && tid == 0) {
-    long long* d = a.stamps + 16 * (long long)blockIdx.x;
-    for (int i = 0; i < 6; ++i) d[i] = ts[i];
-    d[6] = ts[6] - ts[0];
-    d[7] = 0;
-    d[8] = wall0;
-    d[9] = wall_clock64();
-  }
-#endif
 }
 
 // ---- host side: tile plan ---------------------------------------------------------------------------
@@ -598,9 +563,6 @@ __global__ void weight_frag32_kernel(const Ts* __restrict__ w, half_t* __restric
   for (int e = 0; e < 8; ++e) d[e] = f < F ? (half_t)(float)w[((long long)f * C + c0 + e) * 9 + tap] : (half_t)0.0f;
 }
 
-#ifdef NNCV_STREAM_STAMPS
-long long* g_stamps = nullptr;
-#endif
 
 // The launch shape for a layer: pixel groups, filter groups and K groups of a workgroup, the tile geometry that goes
 // with them, and how the (filter block, tile list) pairs spread over the workgroups.
@@ -659,9 +621,6 @@ int stream_force_pg() {
 
 }  // namespace
 
-#ifdef NNCV_STREAM_STAMPS
-extern "C" void nncv_hip_debug_stream_stamps(void* p) { g_stamps = (long long*)p; }
-#endif
 
 size_t weight_frag32_bytes(int F, int C) { return (size_t)((F + 31) / 32) * 32 * 9 * C * 2; }
 
@@ -741,9 +700,6 @@ bool launch_conv3x3_stream(const IgemmArgs& g, hipStream_t s) {
   a.geom = (unsigned)g.H | ((unsigned)g.W << 8) | ((unsigned)geo.S << 16) | ((unsigned)geo.NSEG << 24);
   a.pixB = (unsigned)pix * 2u;
   a.mW16 = (unsigned)((65536 + g.W - 1) / g.W);
-#ifdef NNCV_STREAM_STAMPS
-  a.stamps = g_stamps;
-#endif
   const double P = (double)g.N * g.H * g.W;
   const double flops = 2.0 * P * g.C * 9.0 * g.F;
   const double bytes = 2.0 * (P * g.C + 9.0 * g.C * g.F + P * g.F * (g.residual ? 2 : 1));

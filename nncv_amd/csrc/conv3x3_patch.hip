@@ -73,6 +73,7 @@ struct PatchArgs {
   const float* aux_scale;
   const float* aux_shift;
   int aux_F, aux_relu, aux_fb0;
+  int aux_inline;  // the workgroup of filter block b also computes block b of the auxiliary filters (aux_F == F): no extra blocks
   unsigned aux_wf_bytes;
   // K split over workgroups (the SK instances): grid.z = ksplit workgroups share an output tile, each
   // walks `spk` channel slabs; their fp32 partial tiles meet in `partial` and the last one to
@@ -573,6 +574,40 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
       prime(prime, std::integral_constant<int, 0>());
     }
   }
+  // ---- inline form of the auxiliary 1x1 stride-2 filters: this workgroup's own block of them, computed after its
+  //      3x3 block.  Its operands (the centre pixels of the slots, every slab at once, and all its weight
+  //      fragments) are requested here and arrive under the epilogue of the 3x3 block. ----
+  constexpr int AP = 64 * WS / (NT / 8);       // loader passes over the slots: NT/8 pixels each
+  constexpr int kAuxSlabs = WS == 1 ? 4 : 1;   // slabs the inline form holds in registers
+  u32x4 aregs[kAuxSlabs][AP];
+  u32x4 awreg[kAuxSlabs][NF];
+  EpiScale<OutT> aess;
+  if constexpr (ST == 2) {
+    if (a.aux_inline) {
+      const __amdgpu_buffer_rsrc_t rs_awf = make_rsrc(a.aux_wf, a.aux_wf_bytes);
+#pragma unroll
+      for (int i = 0; i < AP; ++i) {
+        const int sl = i * (NT / 8) + p8;
+        int nl = 0, rem = sl, tx;
+        if (a.TN > 1) nl = fast_div(sl, a.TH * TW, a.inv_thw, &rem);
+        const int ty = fast_div(rem, TW, a.inv_w, &tx);
+        const bool ok = (sl < nslots) & ((n0 + nl) < a.N) & ((y0 + ty) < OH) & ((x0 + tx) < OW);
+        const unsigned off = __umul24((unsigned)(((n0 + nl) * a.H + 2 * (y0 + ty)) * a.W + 2 * (x0 + tx)), ces) + pc;
+#pragma unroll
+        for (int sb = 0; sb < kAuxSlabs; ++sb)
+          aregs[sb][i] = __builtin_amdgcn_raw_buffer_load_b128(rs_in, ok && sb < nslab_all ? off + sb * 128 : kOOBp, 0, 0);
+      }
+      const int awbase = NI == 2 ? (fblk * nslab_all * 8 + wk * KPG * 2) * 1024 : ((fblk >> 1) * nslab_all * 8 + wk * KPG * 2 + (fblk & 1)) * 1024;
+#pragma unroll
+      for (int sb = 0; sb < kAuxSlabs; ++sb)
+#pragma unroll
+        for (int k = 0; k < KPG; ++k)
+#pragma unroll
+          for (int i = 0; i < NI; ++i)
+            awreg[sb][k * NI + i] = __builtin_amdgcn_raw_buffer_load_b128(rs_awf, wlane, sb < nslab_all ? awbase + sb * 8192 + wfrag(k, i) : 0, 0);
+      aess.load(lane, f0blk, a.aux_F, a.aux_scale, a.aux_shift);
+    }
+  }
   if constexpr (kLateScale) ess.load(lane, f0blk, a.F, a.scale, a.shift);
   __syncthreads();  // every wave is done with the patch: LDS becomes the output tiles
 
@@ -584,6 +619,42 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   } else {
     tile_reduce_store<OutT, WK, NI, ACT>(acc, smem + ws * WK * kTileBytes, wk, lane, obase, f0blk, a.F, ess,
                                          static_cast<const OutT*>(a.residual), static_cast<OutT*>(a.out), a.relu);
+  }
+  if constexpr (ST == 2 && !SK) {
+    if (a.aux_inline) {
+      __syncthreads();  // the output tiles have been read: LDS becomes the slots' centre pixels, [slot][slab][64 ch] + 16 pad
+      const int apitch = nslab_all * 128 + 16;
+#pragma unroll
+      for (int i = 0; i < AP; ++i)
+#pragma unroll
+        for (int sb = 0; sb < kAuxSlabs; ++sb)
+          if (sb < nslab_all) *reinterpret_cast<u32x4*>(smem + (i * (NT / 8) + p8) * apitch + sb * 128 + pc) = aregs[sb][i];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+      __syncthreads();
+#pragma unroll
+      for (int sb = 0; sb < kAuxSlabs; ++sb)
+        if (sb < nslab_all) {  // uniform
+#pragma unroll
+          for (int k = 0; k < KPG; ++k) {
+            u32x4 p[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+              p[j] = *reinterpret_cast<const u32x4*>(smem + (ws * 64 + j * 32 + lrow) * apitch + sb * 128 + (lchunk + 2 * wk * KPG) * 16 + k * 32);
+#pragma unroll
+            for (int i = 0; i < NI; ++i)
+#pragma unroll
+              for (int j = 0; j < 2; ++j) Mma<T>::run(awreg[sb][k * NI + i], p[j], acc[i][j]);
+          }
+        }
+      __syncthreads();  // every wave is done with the pixels: LDS becomes the output tiles again
+      tile_reduce_store<OutT, WK, NI, false>(acc, smem + ws * WK * kTileBytes, wk, lane, obase, f0blk, a.aux_F, aess,
+                                             static_cast<const OutT*>(nullptr), static_cast<OutT*>(a.aux_out), a.aux_relu);
+    }
   }
 }
 
@@ -735,9 +806,11 @@ static void launch_patch_cfg(const PatchArgs& a, double flops, double bytes, con
   }();
   (void)attr;
   ProfScope prof(tag, flops, bytes, s);
-  const int fblocks = (a.F + 32 * NI - 1) / (32 * NI) + (a.aux_F + 32 * NI - 1) / (32 * NI);
   PatchArgs b = a;
   b.aux_fb0 = (a.F + 32 * NI - 1) / (32 * NI);
+  // inline form of the auxiliary filters: same count as the 3x3 filters, rows of the same length, every slab held at once
+  b.aux_inline = ST == 2 && !SK && a.aux_inline && a.aux_F == a.F && a.ldo == a.aux_F && a.C * (int)sizeof(T) / 128 <= (WS == 1 ? 4 : 1);
+  const int fblocks = b.aux_fb0 + (b.aux_inline ? 0 : (a.aux_F + 32 * NI - 1) / (32 * NI));
   if (b.xcd_by_filter && fblocks % kXcdsP != 0) b.xcd_by_filter = 0;
   dim3 grid((a.tiles + kXcdsP - 1) / kXcdsP * kXcdsP, fblocks, SK ? a.ksplit : 1);
   hipLaunchKernelGGL(kern, grid, dim3(Cfg::NT), Cfg::smem, s, b.in, b.tiles, b.tiles_y, b.TN, b.TH, b.N, b.H, b.W, b.C, b.rw_log,
@@ -754,6 +827,8 @@ void launch_conv3x3_patch(const IgemmArgs& g, int in_dt, int out_dt, hipStream_t
     a.aux_scale = g.scale ? g.scale + g.aux_f0 : nullptr; a.aux_shift = g.shift ? g.shift + g.aux_f0 : nullptr;
     a.aux_wf_bytes = (unsigned)((size_t)((a.aux_F + 63) / 64) * 64 * g.C * dtype_size(in_dt));
   }
+  static const bool no_inline = getenv("NNCV_HIP_NO_AUX_INLINE") != nullptr;
+  a.aux_inline = a.aux_F > 0 && !no_inline;
   int ws = 0;
   const int st = g.stride_h;
   a.OH = g.OH; a.OW = g.OW;

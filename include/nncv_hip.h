@@ -122,6 +122,13 @@ int nncv_hip_conv_forward_noalloc(nncv_hip_conv* c, const void* in, int N, int H
  * consecutive dispatches, so it reads slightly above a profiler's per-kernel time. */
 int nncv_hip_conv_time(nncv_hip_conv* c, const void* in, int N, int H, int W, const void* residual, void* out, int reps,
                        void* stream, float* avg_us);
+/* The handle-less entry points (_mlir_ciface_forward and its fp16 / MobileNetV3 forms) keep the device copy of a
+ * parameter blob between calls, keyed by the blob's host address, length and type, and notice new contents at the same
+ * address through a fingerprint of 4096 evenly spaced samples (hashing all 47 MB on every call would cost more than the
+ * forward pass).  A caller that rewrites parameters in place calls this afterwards: the device copies made from
+ * `params` (all of them when `params` is NULL) are dropped and rebuilt on the next call.  Returns 0.  No counterpart
+ * in the reference, whose compiled forward re-reads the blob on every call (examples/Res18/main.cpp:95-99). */
+int nncv_hip_params_invalidate(const void* params);
 /* Diagnostic, host arithmetic only (works without a GPU): the tile plan of the 3x3 LDS-patch kernel for
  * N x OH x OW output pixels at `stride` (1 | 2), F filters and `slabs` 128-byte channel slabs.
  * plan[8] = {WS (64-slot groups per workgroup), TN images, TH rows, TW columns per tile, NTX column tiles per
@@ -129,6 +136,13 @@ int nncv_hip_conv_time(nncv_hip_conv* c, const void* in, int N, int H, int W, co
  * no plan exists. No counterpart in the reference: it lets the CPU test suite check the planner's invariants
  * (a plan that overflows LDS or the loader would fault on the device). */
 int nncv_hip_conv3x3_patch_plan(int stride, int N, int OH, int OW, int F, int slabs, int* plan);
+/* Diagnostic, host arithmetic only: the launch plan of the fp16 3x3 stride-1 stream kernel for N x H x W pixels, C
+ * channels and F filters.  plan[12] = {TH virtual rows per tile, S virtual rows per image, top (1: the images are one
+ * zero row apart), aligned (1: tiles never leave their image), tiles, NSEG seven-cell segments per patch row, PG pixel
+ * groups, WF filter groups, WK K groups of a workgroup, filter blocks, workgroups per filter block (= the tile step of a
+ * workgroup), row segments one patch buffer holds}.  Returns 0, or 1 when the kernel does not take the shape.
+ * No counterpart in the reference: it lets the CPU test suite check that a plan never outgrows the kernel's LDS. */
+int nncv_hip_conv3x3_stream_plan(int N, int H, int W, int C, int F, int* plan);
 
 /* C += A.B, fp32 row-major, DEVICE pointers (K and N multiples of 4). */
 /* The reference driver's image preparation and top-1 scan on the device

@@ -187,6 +187,8 @@ std::vector<CachedModel>& model_cache() {
   return c;
 }
 
+void drop_graphs_of(const void* m);
+
 // cheap change detector for a parameter blob that lives at the same address: 4096 strided samples
 uint64_t fingerprint(const void* p, long long n, size_t es) {
   NNCV_REQUIRE(p && n > 0, "params: empty memref");
@@ -212,13 +214,18 @@ ResNet18& cached_model(const void* host, long long n, int dt, hipStream_t s) {
   auto& cache = model_cache();
   for (auto& e : cache)
     if (e.host_ptr == host && e.n == n && e.dt == dt) {
-      if (e.fingerprint != fp) {  // same address, new contents: rebuild
+      if (e.fingerprint != fp) {  // same address, new contents: rebuild (captured passes of the old object die with it)
+        drop_graphs_of(e.model.get());
+        e.model.reset();
         e.model = build_model(host, n, dt, kAlgoAuto, s);
         e.fingerprint = fp;
       }
       return *e.model;
     }
-  if (cache.size() >= 4) cache.erase(cache.begin());
+  if (cache.size() >= 4) {
+    drop_graphs_of(cache.front().model.get());
+    cache.erase(cache.begin());
+  }
   cache.push_back(CachedModel{host, n, dt, fp, build_model(host, n, dt, kAlgoAuto, s)});
   return *cache.back().model;
 }
@@ -343,12 +350,17 @@ Graph& cached_mobilenetv3(const void* host, long long n, int dt, hipStream_t s) 
   for (auto& e : cache)
     if (e.host_ptr == host && e.n == n && e.dt == dt) {
       if (e.fingerprint != fp) {
+        drop_graphs_of(e.graph.get());
+        e.graph.reset();
         e.graph = make();
         e.fingerprint = fp;
       }
       return *e.graph;
     }
-  if (cache.size() >= 4) cache.erase(cache.begin());
+  if (cache.size() >= 4) {
+    drop_graphs_of(cache.front().graph.get());
+    cache.erase(cache.begin());
+  }
   cache.push_back(CachedGraph{host, n, dt, fp, make()});
   return *cache.back().graph;
 }
@@ -512,6 +524,33 @@ void nncv_hip_profile_enable(int on) {
 int nncv_hip_conv3x3_patch_plan(int stride, int N, int OH, int OW, int F, int slabs, int* plan) {
   if (!plan) return 1;
   return conv3x3_patch_plan(stride, N, OH, OW, F, slabs, plan) ? 0 : 1;
+}
+
+int nncv_hip_params_invalidate(const void* params) {
+  return guarded([&] {
+    std::lock_guard<std::recursive_mutex> lk(Context::get().mu);
+    auto& mc = model_cache();
+    for (size_t i = 0; i < mc.size();)
+      if (!params || mc[i].host_ptr == params) {
+        drop_graphs_of(mc[i].model.get());
+        mc.erase(mc.begin() + i);
+      } else {
+        ++i;
+      }
+    auto& gc = graph_model_cache();
+    for (size_t i = 0; i < gc.size();)
+      if (!params || gc[i].host_ptr == params) {
+        drop_graphs_of(gc[i].graph.get());
+        gc.erase(gc.begin() + i);
+      } else {
+        ++i;
+      }
+  });
+}
+
+int nncv_hip_conv3x3_stream_plan(int N, int H, int W, int C, int F, int* plan) {
+  if (!plan) return 1;
+  return conv3x3_stream_plan(N, H, W, C, F, plan) ? 0 : 1;
 }
 
 size_t nncv_hip_profile_report(char* buf, size_t cap) {

@@ -580,11 +580,16 @@ struct StreamConfig {
 // (what the SIMDs of a CU share), plus a per-tile constant for the epilogue.  `only_pg` > 0 restricts the choice.
 bool stream_config(int N, int H, int W, int C, int F, bool act, int only_pg, StreamConfig* best) {
   bool found = false;
-  for (int cand = 0; cand < (act ? 2 : 3); ++cand) {  // the eight-wave form exists with the ReLU epilogue only
+  static const int force_wf = [] {
+    const char* e = getenv("NNCV_HIP_STREAM_WF");
+    return e ? atoi(e) : 0;
+  }();
+  for (int cand = 0; cand < (act ? 2 : 4); ++cand) {  // the eight-wave form and the 128-filter one exist with the ReLU epilogue only
     StreamConfig c;
     c.PG = cand == 2 ? 2 : 1;
-    c.WF = cand == 1 ? 1 : 2;
+    c.WF = cand == 1 ? 1 : cand == 3 ? 4 : 2;
     c.WK = 4 / c.WF;
+    if (force_wf > 0 && c.WF != force_wf && !act) continue;
     // Measured, the eight-wave form loses to two independent workgroups of four (13.5 against 12.2 us on 28x28x128 at
     // batch 32): its barriers stop both waves of every SIMD at once, where two workgroups drift apart and fill each
     // other's waits.  It runs on request only (NNCV_HIP_STREAM_PG=2).
@@ -603,6 +608,12 @@ bool stream_config(int N, int H, int W, int C, int F, bool act, int only_pg, Str
     const int trows = (c.geo.TH * W + 31) / 32;
     const long long ksteps = (long long)C / 64 * 36;
     c.cost = wg_per_cu * rounds * ((long long)trows * c.WF * ksteps + 600);
+    // 128 filters per workgroup, no K groups: no exchange of partial sums at the end of a tile.  Measured against the
+    // 64-filter form on 28x28x128: 18.1 / 66.4 us against 18.8 / 68.5 at batch 64 / 256 (448 / 512 workgroups).  With
+    // about one workgroup per CU (224 at batch 32; 214 on 14x14x256 at batch 64) it is ahead on some runs (10.4 against
+    // 10.5, 16.6 against 17.2) and far behind on others (13.9), depending on where the workgroups land, and with 108
+    // (14x14x256 at batch 32) it loses outright (15.0 against 10.2): it is taken from 400 workgroups up.
+    if (c.WF == 4) c.cost = wgs >= 400 ? 0 : (1ll << 60);
     if (!found || c.cost < best->cost) {
       *best = c;
       found = true;
@@ -706,6 +717,8 @@ bool launch_conv3x3_stream(const IgemmArgs& g, hipStream_t s) {
   const bool act = g.relu > kActRelu;
   if (cfg.PG == 2) {
     launch_stream_cfg<2, 2, 2, false>(a, grid, flops, bytes, "conv3x3_stream<f16,2x2x2>", s);
+  } else if (cfg.WF == 4) {
+    launch_stream_cfg<1, 4, 1, false>(a, grid, flops, bytes, "conv3x3_stream<f16,1x4x1>", s);
   } else if (cfg.WF == 1) {
     if (act) launch_stream_cfg<1, 1, 4, true>(a, grid, flops, bytes, "conv3x3_stream<f16,1x1x4,act>", s);
     else launch_stream_cfg<1, 1, 4, false>(a, grid, flops, bytes, "conv3x3_stream<f16,1x1x4>", s);

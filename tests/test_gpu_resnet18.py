@@ -60,6 +60,20 @@ def test_cfg3_fp32_256_through_reference_abi(blob, tmp_path):
     params[-1000:] += 1.0  # fc.bias
     shifted = abi.forward(x, params)
     assert np.allclose(shifted, got + 1.0, atol=1e-5)
+    # a change between the fingerprint's samples goes unnoticed until the caller says so (nncv_hip_params_invalidate):
+    # that is the documented contract of the cache
+    n = params.size
+    step = max(1, n // 4096)
+    i = n - 1000 + 7  # fc.bias[7]
+    assert i % step != 0 and i != n - 1, "pick an element the fingerprint does not sample"
+    params[i] += 2.0
+    stale = abi.forward(x, params)
+    assert np.array_equal(stale, shifted)
+    assert abi.lib().nncv_hip_params_invalidate(params.ctypes.data) == 0
+    fresh = abi.forward(x, params)
+    want2 = shifted.copy()
+    want2[:, 7] += 2.0
+    assert np.allclose(fresh, want2, atol=1e-5)
 
 
 def test_fp16_small_batch(blob):

@@ -1,0 +1,83 @@
+"""Host-side checks of the fp16 3x3 stream kernel's launch planner (host arithmetic, no GPU needed).
+
+A plan whose patch needs more row segments than a buffer holds, more pixel slots than the waves own, or whose
+reciprocal divisions leave their exact range would make the kernel write outside its LDS allocation or address the
+wrong pixels, so the invariants are checked here for many shapes, together with the plans of the ResNet-18 layers."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from nncv_amd import abi
+
+KEYS = ("TH", "S", "top", "aligned", "tiles", "NSEG", "PG", "WF", "WK", "FB", "Wpf", "segcap")
+
+
+@pytest.fixture(scope="module")
+def plan():
+    L = ctypes.CDLL(abi.LIB_PATH)
+    L.nncv_hip_conv3x3_stream_plan.argtypes = [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_int)]
+    L.nncv_hip_conv3x3_stream_plan.restype = ctypes.c_int
+
+    def call(N, H, W, C, F):
+        out = (ctypes.c_int * 12)()
+        if L.nncv_hip_conv3x3_stream_plan(N, H, W, C, F, out) != 0:
+            return None
+        return dict(zip(KEYS, out))
+    return call
+
+
+def check(p, N, H, W, C, F):
+    slots = 128 * p["PG"]
+    assert p["PG"] in (1, 2) and p["WF"] * p["WK"] == 4 and p["segcap"] == 36 * p["PG"]
+    assert F % (32 * p["WF"]) == 0 and p["FB"] * 32 * p["WF"] == F
+    assert 1 <= p["TH"] and p["TH"] * W <= slots                         # every pixel of a tile has an MFMA slot
+    assert p["NSEG"] * 7 >= W + 2                                        # a patch row holds the row and its two halo cells
+    assert (p["TH"] + 2) * p["NSEG"] <= p["segcap"]                      # the patch fits one LDS buffer
+    assert 2 * (p["segcap"] * 1008 + 64) + 2 * 32 * p["WF"] * 4 <= (80 if p["PG"] == 1 else 160) * 1024  # two workgroups per CU (one of eight waves)
+    assert 2 <= p["S"] <= 255
+    if p["aligned"]:
+        assert p["top"] == 0 and p["S"] % p["TH"] == 0 and p["S"] >= H   # a whole number of tiles per image
+        assert p["tiles"] == N * (p["S"] // p["TH"])
+    else:
+        assert p["top"] == 1 and p["S"] == H + 1                         # one shared zero row between images
+        rows = N * (H + 1) - 1
+        assert (p["tiles"] - 1) * p["TH"] < rows <= p["tiles"] * p["TH"]  # the tiles cover virtual rows 1 .. rows
+    assert (N * p["S"] + p["TH"] + 2) * p["S"] < 2 ** 31                 # the reciprocal multiplications stay exact
+    assert 1 <= p["Wpf"] <= p["tiles"] and p["Wpf"] < 65536
+    # every tile is walked: a workgroup starts at tile i < Wpf and steps by Wpf
+    assert (p["tiles"] + p["Wpf"] - 1) // p["Wpf"] >= 1
+
+
+def test_invariants_on_random_shapes(plan):
+    rng = np.random.default_rng(20251126)
+    found = 0
+    for _ in range(20000):
+        N = int(rng.choice([1, 1, 2, 3, 4, 5, 8, 16, 32, 64, 256, 1000]))
+        H, W = int(rng.integers(1, 200)), int(rng.integers(1, 200))
+        C = 64 * int(rng.integers(1, 9))
+        F = 32 * int(rng.integers(1, 17))
+        p = plan(N, H, W, C, F)
+        if p is None:
+            # only what cannot fit is refused: a row wider than the slots or the buffer, more rows than the 8-bit fields
+            # hold, one-row images (a single virtual row per image has no reciprocal), dividends beyond the exact range
+            assert W > 128 or H > 254 or H == 1 or 3 * ((W + 2 + 6) // 7) > 36 or (N * (H + 1) + 200) * (H + 1) >= 2 ** 31, (N, H, W, C, F)
+            continue
+        found += 1
+        check(p, N, H, W, C, F)
+    assert found > 5000
+
+
+@pytest.mark.parametrize("N,H,W,C,F,expect", [
+    (32, 56, 56, 64, 64, dict(TH=2, aligned=1, tiles=896, WF=2, WK=2, Wpf=448)),      # layer1: 896 tiles, two per workgroup
+    (32, 28, 28, 128, 128, dict(TH=4, aligned=1, tiles=224, WF=2, WK=2, FB=2)),       # layer2, the roofline kernel's shape
+    (32, 14, 14, 256, 256, dict(TH=9, aligned=0, S=15, WF=2, FB=4)),                  # layer3: images one zero row apart
+    (64, 28, 28, 128, 128, dict(TH=4, tiles=448, WF=4, WK=1, FB=1)),                  # batch 64: 128 filters per workgroup, no K groups
+    (1, 28, 28, 128, 128, dict(WF=1, WK=4)),                                          # batch 1: 32-filter blocks fill more CUs
+])
+def test_resnet18_plans(plan, N, H, W, C, F, expect):
+    p = plan(N, H, W, C, F)
+    assert p is not None
+    check(p, N, H, W, C, F)
+    for k, v in expect.items():
+        assert p[k] == v, (k, p)

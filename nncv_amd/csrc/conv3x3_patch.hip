@@ -809,7 +809,9 @@ static void launch_patch_cfg(const PatchArgs& a, double flops, double bytes, con
   PatchArgs b = a;
   b.aux_fb0 = (a.F + 32 * NI - 1) / (32 * NI);
   // inline form of the auxiliary filters: same count as the 3x3 filters, rows of the same length, every slab held at once
-  b.aux_inline = ST == 2 && !SK && a.aux_inline && a.aux_F == a.F && a.ldo == a.aux_F && a.C * (int)sizeof(T) / 128 <= (WS == 1 ? 4 : 1);
+  // ... and only where the 3x3 blocks alone fill the CUs: on a small launch the separate blocks are extra parallelism
+  b.aux_inline = ST == 2 && !SK && a.aux_inline && a.aux_F == a.F && a.ldo == a.aux_F && a.C * (int)sizeof(T) / 128 <= (WS == 1 ? 4 : 1) &&
+                 (long long)a.tiles * b.aux_fb0 >= 200;
   const int fblocks = b.aux_fb0 + (b.aux_inline ? 0 : (a.aux_F + 32 * NI - 1) / (32 * NI));
   if (b.xcd_by_filter && fblocks % kXcdsP != 0) b.xcd_by_filter = 0;
   dim3 grid((a.tiles + kXcdsP - 1) / kXcdsP * kXcdsP, fblocks, SK ? a.ksplit : 1);

@@ -663,10 +663,17 @@ bool conv3x3_stream_applicable(const IgemmArgs& a, int in_dt, int out_dt) {
   const int pix = a.pix_stride ? a.pix_stride : a.C;
   const bool act_ok = a.relu <= kActRelu || ((a.relu & 0xff) <= kActSigmoid && (a.relu & ~(0xff | kActResidualAfter)) == 0);
   StreamConfig c;
-  return act_ok && a.aux_f0 == 0 && a.R == 3 && a.S == 3 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 1 && a.pad_w == 1 &&
+  const bool shape_ok = act_ok && a.aux_f0 == 0 && a.R == 3 && a.S == 3 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 1 && a.pad_w == 1 &&
          a.OH == a.H && a.OW == a.W && a.batch == 1 && a.C % 64 == 0 && a.F % 32 == 0 && pix % 8 == 0 && a.ldo % 8 == 0 && a.ldo >= a.F &&
          (long long)a.N * a.H * a.W * a.ldo * 2 < (1ll << 31) && (long long)a.N * a.H * a.W * pix * 2 < (1ll << 31) &&
          a.in_bytes < kOOBs && (long long)a.F * 9 * a.C * 2 < (1ll << 31) && stream_config(a.N, a.H, a.W, a.C, a.F, a.relu > kActRelu, stream_force_pg(), &c);
+  if (!shape_ok) return false;
+  // Small launches and poorly filled tiles stay with the patch kernel (measured, stream / patch us): 1x28x28x128 5.7 /
+  // 4.9, 4x28x28x128 5.9 / 5.0, 8x14x14x256 7.9 / 6.3 -- 112 workgroups of 32 filters or fewer -- against 8x28x28x128
+  // 5.9 / 6.3, 16x14x14x256 7.9 / 8.6, 4x56x56x64 4.9 / 5.4 (216-224 workgroups); rows of 80 pixels fill 80 of a
+  // tile's 128 slots: 16x80x80x64 18.2 / 15.7, where the patch kernel cuts the rows into column tiles.
+  const long long fine_wgs = (long long)c.geo.n_tiles * (a.F / 32);
+  return all || (fine_wgs >= 160 && c.geo.TH * a.W >= 96);
 }
 
 template <int PG, int WF, int WK, bool ACT>

@@ -96,25 +96,35 @@ def test_fp16_layers_take_the_kernels_they_are_measured_on(blob):
     ones through the patch kernel's stride-2 form with the 1x1 shortcut riding along (no separate shortcut launch), so a
     silent fall-back to the implicit-GEMM kernels shows up here and not only in the timings."""
     hb = synth.round_fp16(blob)
-    x = synth.round_fp16(synth.uniform(4003, (4, 3, 224, 224), 0.0, 1.0))
     m = Model(hb, abi.F16, abi.ALGO_IGEMM)
-    xd = dev(x, abi.F16)
-    m(xd)
-    torch.cuda.synchronize()
-    abi.profile_enable(True)
-    try:
-        abi.profile_report()
-        got = host(m(xd))
-        rep = abi.profile_report()
-    finally:
-        abi.profile_enable(False)
-    print({k: v["launches"] for k, v in rep.items()}, flush=True)
-    count = lambda prefix: sum(v["launches"] for k, v in rep.items() if k.startswith(prefix))
+
+    def tags(xd):
+        m(xd)
+        torch.cuda.synchronize()
+        abi.profile_enable(True)
+        try:
+            abi.profile_report()
+            got = host(m(xd))
+            rep = abi.profile_report()
+        finally:
+            abi.profile_enable(False)
+        print({k: v["launches"] for k, v in rep.items()}, flush=True)
+        return got, rep, (lambda prefix: sum(v["launches"] for k, v in rep.items() if k.startswith(prefix)))
+
+    # batch 32, the measured configuration (input values do not matter for the route)
+    _, rep, count = tags(dev(synth.round_fp16(synth.uniform(4004, (32, 3, 224, 224), 0.0, 1.0)), abi.F16))
     assert count("conv3x3_patch") + count("conv3x3_stream") == 13
     assert count("conv3x3_stream") == 10  # layer1 (4), layer2 (3) and layer3 (3)
     assert count("conv3x3s2_patch") == 3
     assert count("igemm") == 0
     assert sum(v["launches"] for v in rep.values()) == 18  # + stem/pool and pool/FC
+    # batch 4 against the oracle: the small launches of layer2 / layer3 stay with the patch kernel
+    x = synth.round_fp16(synth.uniform(4003, (4, 3, 224, 224), 0.0, 1.0))
+    got, rep, count = tags(dev(x, abi.F16))
+    assert count("conv3x3_patch") + count("conv3x3_stream") == 13
+    assert count("conv3x3_stream") == 4  # layer1
+    assert count("conv3x3s2_patch") == 3 and count("igemm") == 0
+    assert sum(v["launches"] for v in rep.values()) == 18
     assert rel_l2(got, oracle.resnet18_forward(x, hb)) < FP16_REL_L2
 
 

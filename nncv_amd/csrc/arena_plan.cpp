@@ -1,10 +1,20 @@
 #include "arena_plan.hpp"
 
 #include <algorithm>
+#include <cstdlib>
 #include <limits>
 #include <numeric>
 
 namespace nncv_hip {
+
+int arena_linger() {
+  static const int v = [] {
+    const char* e = getenv("NNCV_HIP_ARENA_LINGER");
+    const int n = e ? atoi(e) : 3;
+    return n < 0 ? 0 : n;
+  }();
+  return v;
+}
 
 size_t plan_offsets(std::vector<TensorLife>& t, size_t align) {
   const size_t mask = align > 1 ? align - 1 : 0;

@@ -23,4 +23,12 @@ struct TensorLife {
 // sizes are rounded up to `align` bytes (a power of two; 1 = none).
 size_t plan_offsets(std::vector<TensorLife>& tensors, size_t align);
 
+// Operator steps a tensor's memory is kept after its last reader before the planners of the forward passes hand it to
+// another tensor (they add this to every last_op).  Measured on ResNet-18 at batch 32 (rocprofv3, median per launch): a
+// launch whose output lies where the previous launch's INPUT lay runs 2-4.4 us longer (16.4 against 12.0 us for the first
+// stride-1 convolution after a down-sampling one, 14.0 against 11.8 one stage deeper), one launch further back it is
+// still 2.3 us (13.4 against 11.1), from three launches on nothing; the whole pass gains 9 us of 256 for 20 % more
+// workspace.  NNCV_HIP_ARENA_LINGER overrides (0 = hand memory on at once).
+int arena_linger();
+
 }  // namespace nncv_hip

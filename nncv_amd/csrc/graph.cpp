@@ -431,6 +431,9 @@ const Graph::Plan& Graph::plan_of(int N, int H, int W) const {
     if (view_of_[t] >= 0) life[t] = TensorLife{life[t].first_op, life[t].first_op, 0, 0};
   for (int i = 0; i < n; ++i)  // the output of a convolution that was merged with its ADD is never stored
     if (nodes_[i].add_out >= 0) life[nodes_[i].op.out] = TensorLife{i + 1, i + 1, 0, 0};
+  // memory is handed on a few launches after its last reader, not at once (arena_plan.hpp)
+  for (int t = 0; t < n_tensors_; ++t)
+    if (life[t].bytes > 0) life[t].last_op = std::min(n + 1, life[t].last_op + arena_linger());
   p.total = plan_offsets(life, 256);
   p.offset.resize(n_tensors_);
   p.root_bytes.resize(n_tensors_);

@@ -339,6 +339,7 @@ static Plan make_plan(const ConvLayer& stem, const std::vector<const ConvLayer*>
   t[ix[nb]].last_op = 26;
   const int i_pooled = add(26, 27, (size_t)N * 512 * es);
   const int i_cws = add(0, 27, cws);
+  for (auto& e : t) e.last_op = std::min(27, e.last_op + arena_linger());
   p.total = plan_offsets(t, 256) + 4096;
   p.stem_out = t[i_stem].offset; p.pooled = t[i_pooled].offset; p.cws = t[i_cws].offset;
   for (int k = 0; k <= nb; ++k) p.x[k] = t[ix[k]].offset;

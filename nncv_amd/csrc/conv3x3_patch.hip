@@ -872,7 +872,14 @@ void launch_conv3x3_patch(const IgemmArgs& g, int in_dt, int out_dt, hipStream_t
     const int nslab = a.C * (int)dtype_size(in_dt) / 128;
     const long long wgs = (long long)a.tiles * (a.F / 32 + (a.aux_F + 31) / 32);
     const int want = (int)std::min<long long>(std::min(nslab, kMaxSplit), sk_env > 0 ? sk_env : 256 / wgs);
-    if (want >= 2 && wgs <= g.splitk_counters_n) {
+    // Only walks of eight slabs and more are split: the reduction through memory costs about as much as four slabs of
+    // taps (one fp32 layer [1,64,56,56] -> 64, two slabs: 8.3 us whole against 12.4 split in two; the fp32 network at
+    // [1,3,256,256]: 0.282 ms splitting from two slabs, 0.265 from four, 0.263 from eight, 0.289 from sixteen, 0.360 never).
+    static const int min_slabs = [] {
+      const char* e = getenv("NNCV_HIP_SPLITK_MINSLAB");
+      return e ? atoi(e) : 8;
+    }();
+    if (want >= 2 && nslab >= min_slabs && wgs <= g.splitk_counters_n) {
       a.spk = (nslab + want - 1) / want;
       a.ksplit = (nslab + a.spk - 1) / a.spk;
       if ((size_t)wgs * a.ksplit * 4096 * sizeof(float) > g.splitk_ws_bytes) a.ksplit = 1;

@@ -144,7 +144,6 @@ int nncv_hip_conv3x3_patch_plan(int stride, int N, int OH, int OW, int F, int sl
  * No counterpart in the reference: it lets the CPU test suite check that a plan never outgrows the kernel's LDS. */
 int nncv_hip_conv3x3_stream_plan(int N, int H, int W, int C, int F, int* plan);
 
-/* C += A.B, fp32 row-major, DEVICE pointers (K and N multiples of 4). */
 /* The reference driver's image preparation and top-1 scan on the device
  * (examples/Res18/main.cpp:38-77 and :103-111).
  * preprocess: hwc_u8 is a DEVICE [N,H,W,channels] 8-bit image (channels 3 or 4, the first three
@@ -167,6 +166,8 @@ int nncv_hip_resnet18_classify_u8(nncv_hip_model* m, const void* hwc_u8, int N, 
 unsigned long long nncv_hip_plan_arena(int n, const int* first_op, const int* last_op, const unsigned long long* bytes,
                                        unsigned long long align, unsigned long long* offsets);
 
+/* C += A.B, fp32 row-major, DEVICE pointers, any M, N, K >= 1 (the device form of _mlir_ciface_matmul;
+ * tests/MatMulOptimization/MatMulDeafult.mlir:11-21). */
 int nncv_hip_matmul_f32(const float* A, const float* B, float* C, int M, int N, int K, void* stream);
 /* Measurement helper, like nncv_hip_conv_time: `reps` launches of C += A.B back to back on `stream` between one pair
  * of HIP events (after 5 untimed ones); *avg_us = elapsed / reps.  C keeps accumulating. */

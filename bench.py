@@ -74,6 +74,9 @@ def main():
     ap.add_argument("--no-batch1", action="store_true", help="skip the batch-1 measurement and the per-layer sweep (for per-kernel profiles)")
     ap.add_argument("--no-sweep", action="store_true", help="skip the per-layer 3x3 sweep at batch 64 (BASELINE config 5)")
     ap.add_argument("--profile-steps", type=int, default=5)
+    ap.add_argument("--in-flight", type=int, default=2,
+                    help="forward passes kept in flight: step k runs on model handle and HIP stream k mod this number "
+                         "(each handle owns its workspace); 1 = one pass after the other")
     ap.add_argument("--workload", default="resnet18", choices=["resnet18", "mobilenetv3", "yolov5s"],
                     help="resnet18 = the headline configuration; mobilenetv3 / yolov5s = the networks of tests/Nets/MobileNetV3.mlir "
                          "and Yolov5s.mlir through the operator-list executor (same step definition, their own JSON line; "
@@ -125,34 +128,52 @@ def main():
     xd = torch.from_numpy(x).cuda()
     logits = torch.empty((N, 1000), dtype=torch.float32, device="cuda")
     stream = torch.cuda.current_stream().cuda_stream
+    # Passes in flight: handle i and stream i serve steps i, i + K, i + 2K ...  A handle owns its workspace, so passes of
+    # different handles overlap on the GPU (one pass's launch gaps, prologues and tails fill with the other's work); every
+    # pass is still a whole forward over one batch of N images, into its own logits buffer.
+    K = max(1, args.in_flight)
+    models, keep_streams, outs, stream_objs = [model], [stream], [logits], []
+    for _ in range(1, K):
+        h = L.nncv_hip_resnet18_create(blob.ctypes.data, blob.size, abi.F16, algo)
+        if not h:
+            raise RuntimeError(L.nncv_hip_last_error().decode())
+        models.append(h)
+        stream_objs.append(torch.cuda.Stream())  # kept alive to the end of main
+        keep_streams.append(stream_objs[-1].cuda_stream)
+        outs.append(torch.empty((N, 1000), dtype=torch.float32, device="cuda"))
 
     def step(xt, out, n):
         abi.check(L.nncv_hip_resnet18_forward(model, xt.data_ptr(), n, H, H, out.data_ptr(), stream))
 
-    def timed(xt, out, n, warmup, steps):
+    def timed(xt, out_list, n, warmup, steps, k_in_flight):
+        def go(i):
+            j = i % k_in_flight
+            abi.check(L.nncv_hip_resnet18_forward(models[j], xt.data_ptr(), n, H, H, out_list[j].data_ptr(), keep_streams[j]))
         # clock warm-up: untimed steps until CLOCK_WARMUP_MS of wall time have passed, then the W asked for
         t_w = time.perf_counter()
         while (time.perf_counter() - t_w) * 1e3 < CLOCK_WARMUP_MS:
-            for _ in range(20):
-                step(xt, out, n)
+            for i in range(20):
+                go(i)
             torch.cuda.synchronize()
-        for _ in range(warmup):
-            step(xt, out, n)
+        for i in range(warmup):
+            go(i)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(steps):
-            step(xt, out, n)
-        torch.cuda.synchronize()
+        for i in range(steps):
+            go(i)
+        torch.cuda.synchronize()  # every stream
         return (time.perf_counter() - t0) / steps
 
-    sec = timed(xd, logits, N, args.warmup, args.steps)
+    sec = timed(xd, outs, N, args.warmup, args.steps, K)
+    sec_serial = sec if K == 1 else timed(xd, outs, N, args.warmup, args.steps, 1)
     ips = N / sec
     flops_step = spec.flops_per_image(H) * N
 
     # batch 1 (the other half of the headline metric)
     x1 = xd[:1].contiguous()
-    l1 = torch.empty((1, 1000), dtype=torch.float32, device="cuda")
-    sec1 = None if args.no_batch1 else timed(x1, l1, 1, args.warmup, max(args.steps, 50))
+    l1 = [torch.empty((1, 1000), dtype=torch.float32, device="cuda") for _ in range(K)]
+    sec1 = None if args.no_batch1 else timed(x1, l1, 1, args.warmup, max(args.steps, 50), K)
+    sec1_serial = None if args.no_batch1 else (sec1 if K == 1 else timed(x1, l1, 1, args.warmup, max(args.steps, 50), 1))
 
     # event-timed per-kernel pass (separate from the timed region above: the events serialise launches)
     abi.profile_enable(True)
@@ -223,11 +244,20 @@ def main():
         "data": "synthetic",
         "config": {"workload": "BASELINE config 4: ResNet-18 forward, fp16, input [%d,3,224,224], seeded U[0,1] input, "
                                "random-init Kaiming/BN-folded weights from a model.bin-order blob" % N,
-                   "batch": N, "image": H, "algo3x3": args.algo, "input_resident_in_hbm": True},
+                   "batch": N, "image": H, "algo3x3": args.algo, "input_resident_in_hbm": True,
+                   "passes_in_flight": K,
+                   "passes_in_flight_note": "step k runs on model handle and HIP stream k mod %d, each handle with its own "
+                                            "workspace and logits buffer; every step is one whole forward pass over one batch "
+                                            "of %d images; `one_pass_at_a_time` is the same loop on one handle and one stream" % (K, N)},
         "tflops_effective": round(flops_step / sec / 1e12, 3),
         "frac_of_fp16_mfma_peak": round(flops_step / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 5),
         "conv3x3s1_gflop_per_step": round(conv3x3_flops / 1e9, 2),
-        "batch1": None if sec1 is None else {"images_per_s": round(1.0 / sec1, 2), "ms_per_image": round(sec1 * 1e3, 4)},
+        "one_pass_at_a_time": {"images_per_s": round(N / sec_serial, 2), "ms_per_step": round(sec_serial * 1e3, 4),
+                               "tflops_effective": round(flops_step / sec_serial / 1e12, 3)},
+        "batch1": None if sec1 is None else {"images_per_s": round(1.0 / sec1, 2), "ms_per_image": round(sec1 * 1e3, 4),
+                                             "passes_in_flight": K,
+                                             "one_pass_at_a_time": {"images_per_s": round(1.0 / sec1_serial, 2),
+                                                                    "ms_per_image": round(sec1_serial * 1e3, 4)}},
         "model_create_ms": round(t_create * 1e3, 2),
         "roofline": roofline,
         "kernels": kernels,
@@ -246,7 +276,8 @@ def main():
         torch.cuda.synchronize()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(blob32, x)
-    L.nncv_hip_resnet18_destroy(model)
+    for h in models:
+        L.nncv_hip_resnet18_destroy(h)
     print(json.dumps(out))
 
 
@@ -440,36 +471,47 @@ def bench_graph(args, L):
         from nncv_amd import mobilenetv3_spec as mspec
         blob32, ops = synth.mobilenetv3_params(), abi.mobilenetv3_small_ops()[0]
         name, fixture = "MobileNetV3-small", "tests/Nets/MobileNetV3.mlir"
-    g = abi.graph_create(ops, 3, blob32.astype(np.float16))
+    K = max(1, args.in_flight)  # passes in flight: graph handle i and stream i serve steps i, i + K ... (see main)
+    gs = [abi.graph_create(ops, 3, blob32.astype(np.float16)) for _ in range(K)]
+    g = gs[0]
     oc, oh, ow = abi.graph_output_shape(g, H, H)
     per_image = oc * oh * ow
     x = synth.uniform(4000, (N, 3, H, H), 0.0, 1.0).astype(np.float16)
     xd = torch.from_numpy(x).cuda()
-    result = torch.empty((N, per_image), dtype=torch.float32, device="cuda")
+    results = [torch.empty((N, per_image), dtype=torch.float32, device="cuda") for _ in range(K)]
+    result = results[0]
     stream = torch.cuda.current_stream().cuda_stream
+    stream_objs = [torch.cuda.Stream() for _ in range(1, K)]
+    streams = [stream] + [t.cuda_stream for t in stream_objs]
 
     def step(xt, out, n):
         abi.check(L.nncv_hip_graph_forward(g, xt.data_ptr(), n, H, H, out.data_ptr(), n * per_image, stream))
 
-    def timed(xt, out, n, warmup, steps):
+    def timed(xt, out_list, n, warmup, steps, k_in_flight):
+        def go(i):
+            j = i % k_in_flight
+            abi.check(L.nncv_hip_graph_forward(gs[j], xt.data_ptr(), n, H, H, out_list[j].data_ptr(), n * per_image, streams[j]))
         # clock warm-up: untimed steps until CLOCK_WARMUP_MS of wall time have passed, then the W asked for
         t_w = time.perf_counter()
         while (time.perf_counter() - t_w) * 1e3 < CLOCK_WARMUP_MS:
-            for _ in range(20):
-                step(xt, out, n)
+            for i in range(20):
+                go(i)
             torch.cuda.synchronize()
-        for _ in range(warmup):
-            step(xt, out, n)
+        for i in range(warmup):
+            go(i)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(steps):
-            step(xt, out, n)
+        for i in range(steps):
+            go(i)
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps
 
-    sec = timed(xd, result, N, args.warmup, args.steps)
-    x1, r1 = xd[:1].contiguous(), torch.empty((1, per_image), dtype=torch.float32, device="cuda")
-    sec1 = None if args.no_batch1 else timed(x1, r1, 1, args.warmup, max(args.steps, 50))
+    sec = timed(xd, results, N, args.warmup, args.steps, K)
+    sec_serial = sec if K == 1 else timed(xd, results, N, args.warmup, args.steps, 1)
+    x1 = xd[:1].contiguous()
+    r1 = [torch.empty((1, per_image), dtype=torch.float32, device="cuda") for _ in range(K)]
+    sec1 = None if args.no_batch1 else timed(x1, r1, 1, args.warmup, max(args.steps, 50), K)
+    sec1_serial = None if args.no_batch1 else (sec1 if K == 1 else timed(x1, r1, 1, args.warmup, max(args.steps, 50), 1))
     abi.profile_enable(True)
     abi.profile_report()
     for _ in range(args.profile_steps):
@@ -505,9 +547,13 @@ def bench_graph(args, L):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 (fp32 accumulate)", "data": "synthetic",
         "config": {"workload": "%s forward (the network of %s), fp16, input [%d,3,%d,%d], seeded U[0,1] input, random-init weights "
                                "from a model.bin-order blob" % (name, fixture, N, H, H),
-                   "batch": N, "image": H, "input_resident_in_hbm": True},
+                   "batch": N, "image": H, "input_resident_in_hbm": True, "passes_in_flight": K},
         "tflops_effective": round(flops_step / sec / 1e12, 3),
-        "batch1": None if sec1 is None else {"images_per_s": round(1.0 / sec1, 2), "ms_per_image": round(sec1 * 1e3, 4)},
+        "one_pass_at_a_time": {"images_per_s": round(N / sec_serial, 2), "ms_per_step": round(sec_serial * 1e3, 4)},
+        "batch1": None if sec1 is None else {"images_per_s": round(1.0 / sec1, 2), "ms_per_image": round(sec1 * 1e3, 4),
+                                             "passes_in_flight": K,
+                                             "one_pass_at_a_time": {"images_per_s": round(1.0 / sec1_serial, 2),
+                                                                    "ms_per_image": round(sec1_serial * 1e3, 4)}},
         "roofline": roofline, "kernels": kernels, "device": L.nncv_hip_device_arch().decode(),
     }
     if not args.no_cpu_baseline:
@@ -533,7 +579,8 @@ def bench_graph(args, L):
                 break
         out["cpu_baseline"] = {"value": round(done / dt, 3), "unit": "images/s", "cores": cores, "kind": "port",
                                "sample": "%d images (batches of %d) in %.1f s; fp32, %s" % (done, nb, dt, what)}
-    L.nncv_hip_graph_destroy(g)
+    for h in gs:
+        L.nncv_hip_graph_destroy(h)
     print(json.dumps(out))
 
 

@@ -88,7 +88,11 @@ typedef struct nncv_hip_model nncv_hip_model;
  * and transforms the filters once. */
 nncv_hip_model* nncv_hip_resnet18_create(const void* params, int64_t n_elems, int dtype, int algo3x3);
 void nncv_hip_resnet18_destroy(nncv_hip_model* m);
-/* src: DEVICE NCHW [N,3,H,W] of the model's dtype; logits: DEVICE [N,1000] fp32. */
+/* src: DEVICE NCHW [N,3,H,W] of the model's dtype; logits: DEVICE [N,1000] fp32.  `stream`: the caller's HIP stream
+ * (the call only enqueues), or NULL for the library's own stream (the call then returns when the pass is done).
+ * A handle owns its workspace: passes of different handles on different streams run concurrently (two passes in
+ * flight fill each other's launch gaps -- the way to the highest throughput); calls on one handle are ordered one
+ * after the other, also across streams. */
 int nncv_hip_resnet18_forward(nncv_hip_model* m, const void* src, int N, int H, int W, float* logits, void* stream);
 
 /* Same, and also copies the NHWC activation after `stage` (0: after the max-pool, 1..4: after

@@ -9,6 +9,8 @@
    reference's example, kept as tests/golden/cat_256x256.jpg) and prints its top-1 index, which must
    be the oracle's on the pixels the same decoder produces.  Skipped where that build is absent.
  * _mlir_ciface_forward from two threads at once: each result equals the one a serial call gives.
+ * the device entry point on two streams: one handle (ordered by the library) and two handles (concurrent, each
+   with its own workspace) -- both bit-equal to passes run alone.
 """
 import os
 import shutil
@@ -130,3 +132,34 @@ def test_device_calls_on_two_streams_do_not_overlap_in_the_shared_workspace(blob
     assert np.array_equal(oa.cpu().numpy(), want_a)
     assert np.array_equal(ob.cpu().numpy(), want_b)
     m.close()
+
+
+@pytest.mark.parametrize("dt", [abi.F16, abi.F32])
+def test_two_handles_on_two_streams_run_concurrently_and_stay_exact(blob, dt):
+    """Every network handle owns its workspace: passes of two handles enqueued alternately on two caller streams, with
+    nothing ordering them, overlap on the GPU and must still each give the bits of a pass run alone -- fp16 at the
+    measured batch and fp32 at batch 1, where the deep layers split K over workgroups (tickets and partial sums are
+    per handle too)."""
+    import torch
+    from gpu_util import Model, dev, host
+    b = synth.round_fp16(blob) if dt == abi.F16 else blob
+    N = 16 if dt == abi.F16 else 1
+    ma, mb = Model(b, dt, abi.ALGO_AUTO), Model(b, dt, abi.ALGO_AUTO)
+    L = abi.lib()
+    mk = (lambda seed: synth.round_fp16(synth.uniform(seed, (N, 3, 224, 224), 0.0, 1.0))) if dt == abi.F16 else \
+         (lambda seed: synth.uniform(seed, (N, 3, 224, 224), 0.0, 1.0))
+    xa, xb = dev(mk(9400), dt), dev(mk(9401), dt)
+    want_a, want_b = host(ma(xa)), host(mb(xb))
+    assert not np.array_equal(want_a, want_b)
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    oa = torch.zeros((N, 1000), dtype=torch.float32, device="cuda")
+    ob = torch.zeros((N, 1000), dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    for it in range(8):
+        abi.check(L.nncv_hip_resnet18_forward(ma.h, xa.data_ptr(), N, 224, 224, oa.data_ptr(), s1.cuda_stream))
+        abi.check(L.nncv_hip_resnet18_forward(mb.h, xb.data_ptr(), N, 224, 224, ob.data_ptr(), s2.cuda_stream))
+    torch.cuda.synchronize()
+    assert np.array_equal(oa.cpu().numpy(), want_a)
+    assert np.array_equal(ob.cpu().numpy(), want_b)
+    ma.close()
+    mb.close()

@@ -277,14 +277,14 @@ ResNet18& cached_model(const void* host, long long n, int dt, hipStream_t s) {
 
 // ---- HIP-graph replay of the forward pass --------------------------------------------------
 // A forward pass is 18-73 kernel launches on one stream with fixed arguments for a given (model,
-// input pointer, output pointer, shape, workspace).  Where the pass is launch-bound -- small inputs, where
-// the host cannot enqueue kernels as fast as the GPU retires them -- the second call with the same
-// combination captures the launches into a graph and every later call replays it: one submission
-// instead of 18-73 (MobileNetV3 at batch 1: 0.308 ms against 0.323).  A replay costs about 4 us of its
-// own between consecutive passes, which plain launches do not (their successors are already queued), so
-// larger passes are enqueued plainly: ResNet-18 at batch 32 0.260 ms against 0.264 replayed, batch 4-16
-// 3-5 us less, YOLOv5s and MobileNetV3 at batch 16 / 32 0.3-1 % less.  The pass contains no memset nodes.
-// NNCV_HIP_GRAPH=0 turns replay off, =1 forces it for every size; the event profiler bypasses it.
+// input pointer, output pointer, shape, workspace).  The second call with the same combination captures
+// the launches into a graph and every later call replays it: one submission instead of 18-73.  That is
+// what batch-1 latency is made of (MobileNetV3 at batch 1: 0.308 ms against 0.323), and it is what lets
+// the host keep two passes in flight on two streams (ResNet-18 at batch 32: 0.184 ms per pass replayed
+// against 0.196 with plain launches; MobileNetV3 at batch 32: 0.269 against 0.326).  With one pass at a
+// time and a large batch a replay costs about 4 us that queued plain launches do not (0.264 against
+// 0.260 ms): NNCV_HIP_GRAPH=size replays only launch-bound passes (up to two / four 224x224 images),
+// NNCV_HIP_GRAPH=0 none.  The pass contains no memset nodes; the event profiler bypasses replay.
 struct GraphEntry {
   const void* m;  // the ResNet18 or Graph object the launches belong to
   const void* src;
@@ -320,9 +320,9 @@ void drop_graphs_of(const void* m) {
 // `run` enqueues the whole pass on `s`; `owner` identifies the model it belongs to.
 void replay(const void* owner, const std::function<void()>& run, const void* src, int N, int H, int W, const float* logits, void* ws,
             hipStream_t s, bool launch_bound) {
-  static const int mode = [] {  // -1 by size, 0 never, 1 always
+  static const int mode = [] {  // -1 by size, 0 never, 1 always (the default)
     const char* e = getenv("NNCV_HIP_GRAPH");
-    return !e ? -1 : (atoi(e) != 0 ? 1 : 0);
+    return !e ? 1 : (!strcmp(e, "size") ? -1 : (atoi(e) != 0 ? 1 : 0));
   }();
   const bool use = mode == 1 || (mode == -1 && launch_bound);
   if (!use || profiler_enabled()) {

@@ -510,3 +510,36 @@ def test_three_chained_5x5_max_pools_run_as_one_launch(dt, shape, concat):
     for it in range(3):
         assert np.array_equal(host(g(xd)), first), it
     g.close()
+
+
+def test_two_graph_handles_on_two_streams_stay_exact():
+    """Operator-list handles own their workspace like the ResNet-18 ones: two handles of the same network fed
+    alternately on two caller streams, nothing ordering them, each reproduce the bits of a pass run alone; one handle
+    on two streams is ordered by the library."""
+    ops, blob = small_net()
+    blob = r16(blob)
+    xa, xb = r16(synth.normal(7601, (4, 3, 40, 24))), r16(synth.normal(7602, (4, 3, 40, 24)))
+    ga, gb = Graph(ops, 3, blob, abi.F16), Graph(ops, 3, blob, abi.F16)
+    xda, xdb = dev(xa, abi.F16), dev(xb, abi.F16)
+    want_a, want_b = host(ga(xda)), host(gb(xdb))
+    assert rel_l2(want_a, oracle.run_graph(ops, xa, blob, 3)) < FP16_REL_L2
+    n = want_a.size
+    oa, ob = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    L = abi.lib()
+    torch.cuda.synchronize()
+    for it in range(6):
+        abi.check(L.nncv_hip_graph_forward(ga.h, xda.data_ptr(), 4, 40, 24, oa.data_ptr(), n, s1.cuda_stream))
+        abi.check(L.nncv_hip_graph_forward(gb.h, xdb.data_ptr(), 4, 40, 24, ob.data_ptr(), n, s2.cuda_stream))
+    torch.cuda.synchronize()
+    assert np.array_equal(oa.cpu().numpy().reshape(want_a.shape), want_a)
+    assert np.array_equal(ob.cpu().numpy().reshape(want_b.shape), want_b)
+    # one handle, two streams, two inputs: the second call waits for the first
+    for it in range(4):
+        abi.check(L.nncv_hip_graph_forward(ga.h, xda.data_ptr(), 4, 40, 24, oa.data_ptr(), n, s1.cuda_stream))
+        abi.check(L.nncv_hip_graph_forward(ga.h, xdb.data_ptr(), 4, 40, 24, ob.data_ptr(), n, s2.cuda_stream))
+    torch.cuda.synchronize()
+    assert np.array_equal(oa.cpu().numpy().reshape(want_a.shape), want_a)
+    assert np.array_equal(ob.cpu().numpy().reshape(want_b.shape), host(ga(xdb)))
+    ga.close()
+    gb.close()

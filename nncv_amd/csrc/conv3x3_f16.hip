@@ -1,5 +1,6 @@
 // fp16 3x3 stride-1 pad-1 convolution + BN/residual/activation for gfx950: the stream form of the LDS-patch
-// kernel (conv3x3_patch.hip keeps every other case: fp32, stride 2, odd channel counts, wide rows).
+// kernel (conv3x3_patch.hip keeps every other case: fp32, stride 2, odd channel counts, wide rows, more than 256
+// channels, and launches too small to fill the CUs, where its shorter prologue wins).
 // Replaces what ModernTile.cpp:184-199 + ModernVec.cpp:54-62 emit for linalg.conv_2d_nchw_fchw
 // (tests/Nets/Res18.mlir:157 ...) together with the BN / add / ReLU generics behind it (:127-142, :193-203).
 //

@@ -54,7 +54,9 @@ constexpr int kActResidualAfter = 0x100;
 constexpr float kSixth = 0.16666667163372039794921875f;
 
 // `arith.cmpf ugt` + select: NaN is kept, everything not greater than zero becomes +0.
-__device__ __forceinline__ float relu_ugt(float x) { return (x <= 0.0f) ? 0.0f : x; }
+// One instruction on gfx950: v_maximum3_f32(x, 0, 0) is the IEEE-754-2019 maximum, which propagates NaN and orders
+// -0 below +0, i.e. the same values as the compare + select.
+__device__ __forceinline__ float relu_ugt(float x) { return __builtin_elementwise_maximum(x, 0.0f); }
 
 // 1 / (1 + exp(-x)) on the hardware's exp2 and reciprocal units (v_exp_f32, v_rcp_f32: about 1 ulp
 // each, so the result is within a few ulp of the correctly rounded one -- far inside the 1e-4 / 1e-2

@@ -205,3 +205,55 @@ def test_driver_preprocess_and_top1_restatements():
     z = np.random.default_rng(2).normal(size=(4, 50)).astype(np.float32)
     assert np.array_equal(oracle.top1_scan(z), z.argmax(1))  # no ties, all above -100
     assert oracle.top1_scan(np.full((1, 5), -200.0, np.float32))[0] == 0
+
+
+def test_preprocess_u8_against_exact_arithmetic_and_properties():
+    """oracle.preprocess_u8 pinned without retyping its float formula: against exact rational arithmetic on the
+    driver's constants (examples/Res18/main.cpp:38-77) for every 8-bit value and channel, by the round trip back to
+    the 8-bit value, by monotonicity, and by one-hot images for the HWC -> CHW placement (a fourth channel is ignored)."""
+    from fractions import Fraction
+    mean = [Fraction(float(np.float32(v))) for v in (0.485, 0.456, 0.406)]  # the float literals the driver compiles in
+    std = [Fraction(float(np.float32(v))) for v in (0.229, 0.224, 0.225)]
+    img = np.zeros((1, 256, 1, 3), np.uint8)
+    img[0, :, 0, :] = np.arange(256, dtype=np.uint8)[:, None]
+    got = oracle.preprocess_u8(img)  # [1,3,256,1]
+    assert got.shape == (1, 3, 256, 1) and got.dtype == np.float32
+    for c in range(3):
+        col = got[0, c, :, 0]
+        assert np.all(np.diff(col) > 0)  # strictly increasing in the pixel value
+        for u in range(256):
+            exact = (Fraction(u, 255) - mean[c]) / std[c]
+            # three fp32 roundings on the way, the subtraction cancelling up to half of the operand: a few ulp of 0.5 / std
+            assert abs(Fraction(float(col[u])) - exact) <= Fraction(1, 10 ** 6), (c, u)
+            back = (Fraction(float(col[u])) * std[c] + mean[c]) * 255
+            assert round(back) == u
+    # ImageNet constants: a mid-grey pixel lands near zero in every channel, black and white at -mean/std and (1-mean)/std
+    assert np.all(np.abs(got[0, :, 124, 0]) < 0.4)
+    assert np.allclose(got[0, :, 0, 0], [-0.485 / 0.229, -0.456 / 0.224, -0.406 / 0.225], rtol=1e-6)
+    assert np.allclose(got[0, :, 255, 0], [0.515 / 0.229, 0.544 / 0.224, 0.594 / 0.225], rtol=1e-6)
+    # placement: a single bright sample at (y, x, c) changes exactly output [c, y, x]; alpha is ignored
+    base = oracle.preprocess_u8(np.zeros((2, 3, 4, 4), np.uint8))
+    for (n, y, x, c) in ((0, 0, 0, 0), (1, 2, 3, 1), (0, 1, 2, 2)):
+        im = np.zeros((2, 3, 4, 4), np.uint8)
+        im[n, y, x, c] = 200
+        d = oracle.preprocess_u8(im) != base
+        assert d.sum() == 1 and d[n, c, y, x]
+    im = np.zeros((2, 3, 4, 4), np.uint8)
+    im[..., 3] = 255
+    assert np.array_equal(oracle.preprocess_u8(im), base)
+
+
+def test_top1_scan_semantics():
+    """The driver's scan (examples/Res18/main.cpp:103-111): strict `>` from -100 and index 0, left to right: the first of
+    equal maxima wins, rows that never exceed -100 give 0, NaN never wins; without ties it is numpy's argmax."""
+    z = np.random.default_rng(2).normal(size=(64, 1000)).astype(np.float32)
+    assert np.array_equal(oracle.top1_scan(z), z.argmax(1))
+    f = lambda row: int(oracle.top1_scan(np.array([row], np.float32))[0])
+    assert f([1, 3, 3, 2]) == 1
+    assert f([-200, -150, -100, -101]) == 0          # -100 itself does not exceed the initial maximum
+    assert f([-200, -99.5, -300]) == 1
+    assert f([np.nan, 1.0, 0.5]) == 1
+    assert f([np.nan, -200, -300]) == 0
+    assert f([2.0, np.nan, 5.0, np.nan]) == 2
+    assert f([np.inf, np.inf]) == 0 and f([-np.inf, -np.inf]) == 0
+

@@ -125,6 +125,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     tab[tid] = a.scale ? a.scale[tid] : 1.0f;
     tab[64 + tid] = a.shift ? a.shift[tid] : 0.0f;
   }
+  // The 64 x 224 filter matrix (28 KB) ends up in the registers of EVERY wave.  It comes from memory once per workgroup,
+  // through the (still unused) convolution tile in LDS, instead of once per wave: a quarter of the vector-memory traffic
+  // of the prologue (58 MB over the 512 workgroups of a launch otherwise).  Filter rows are 464 bytes apart there
+  // (448 + 16: the 32 lanes of a fragment read distinct banks).
+  constexpr int kWPitch = 448 + 16;
+  static_assert(64 * kWPitch <= kConvBytes, "the filters fit the convolution tile");
+  {
+    u32x4 stage[7];
+#pragma unroll
+    for (int k = 0; k < 7; ++k) stage[k] = reinterpret_cast<const u32x4*>(a.wt)[tid + 256 * k];  // 1792 chunks of 16 bytes
+#pragma unroll
+    for (int k = 0; k < 7; ++k) {
+      const int c = tid + 256 * k, f = c / 28, w = c - f * 28;
+      *reinterpret_cast<u32x4*>(conv_t + f * kWPitch + w * 16) = stage[k];
+    }
+  }
+  __syncthreads();
   u32x4 wreg[7][2][2];  // [filter row][K half][filter half]
 #pragma unroll
   for (int r = 0; r < 7; ++r)
@@ -132,7 +149,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int h = 0; h < 2; ++h)
 #pragma unroll
       for (int i = 0; i < 2; ++i)
-        wreg[r][h][i] = *reinterpret_cast<const u32x4*>(a.wt + ((i * 32 + lrow) * 7 + r) * 32 + h * 16 + lchunk * 8);
+        wreg[r][h][i] = *reinterpret_cast<const u32x4*>(conv_t + (i * 32 + lrow) * kWPitch + (r * 32 + h * 16 + lchunk * 8) * 2);
 
   // ---- this lane's two convolution pixels (slots) ----
   int cy[2], cx[2], abase[2];

@@ -14,6 +14,10 @@ Besides the headline images/s the line carries
                 the published dense fp16 MFMA peak;
   kernels       an event-timed breakdown for every kernel tag (ms per step, share);
   batch1        images/s of the same network at batch 1;
+  config.passes_in_flight, one_pass_at_a_time
+                `value` keeps several forward passes in flight, each on its own model handle and stream (the
+                count is the best of 2, 3 and 4 in a short trial, the streams are chosen by measuring which of
+                them overlap); the same loop on one handle and one stream is reported next to it;
   host_abi      images/s through the reference's own entry point, _mlir_ciface_forward_f16, with host
                 buffers in and out (what examples/Res18/main.cpp:95-99 times): PCIe transfers included;
   configs       BASELINE configs 1-3: the 1024^3 fp32 matmul, the single fp32 3x3 convolution (direct and
@@ -38,6 +42,51 @@ import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
+# Hardware queues of this process (the HIP runtime's own setting, read when it initialises; its default is 4, of which
+# three serve streams other than the default one).  Streams beyond the queues share them and their work runs one after
+# the other, so passes on four streams overlap like passes on two.  Eight leave every stream used here a queue of its own.
+os.environ.setdefault("GPU_MAX_HW_QUEUES", "8")
+IN_FLIGHT_CANDIDATES = (2, 3, 4)
+
+
+def concurrent_streams(torch, run_pass, want, candidates=8):
+    """`want` streams from torch's pool whose work overlaps, and what the probe found.
+
+    Two streams overlap only when the runtime gave them different hardware queues AND those queues sit on different
+    pipes of the command processor (four pipes; queue q of a process is served by pipe q mod 4): passes on two streams
+    that share a queue run one after the other, on two queues of one pipe they gain 14 %.  Which queue a stream gets
+    depends on every stream the process created before it, so the streams are chosen by measurement: run_pass(h, s)
+    enqueues one short pass of handle h on stream s; a candidate is taken when a pass on it next to a pass on each
+    stream already taken costs less than 1.5 passes."""
+    objs = [torch.cuda.Stream() for _ in range(candidates)]
+
+    def ms(a, b, n):
+        for _ in range(n):
+            run_pass(0, a.cuda_stream)
+            if b is not None:
+                run_pass(1, b.cuda_stream)
+        torch.cuda.synchronize()
+
+    t_w = time.perf_counter()
+    while (time.perf_counter() - t_w) * 1e3 < CLOCK_WARMUP_MS:
+        ms(objs[0], None, 20)
+
+    def cost(a, b):
+        ms(a, b, 5)
+        t0 = time.perf_counter()
+        ms(a, b, 30)
+        return (time.perf_counter() - t0) / 30
+
+    alone = cost(objs[0], None)
+    taken = [objs[0]]
+    for c in objs[1:]:
+        if len(taken) >= want:
+            break
+        if all(cost(m, c) < 1.5 * alone for m in taken):
+            taken.append(c)
+    found = len(taken)
+    taken += [c for c in objs if c not in taken][:max(0, want - found)]
+    return taken, {"candidates": candidates, "overlapping": found}
 
 MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 matrix peak
 MFMA_F32_PEAK_TFLOPS = 157.3    # MI355X fp32 matrix peak
@@ -74,9 +123,13 @@ def main():
     ap.add_argument("--no-batch1", action="store_true", help="skip the batch-1 measurement and the per-layer sweep (for per-kernel profiles)")
     ap.add_argument("--no-sweep", action="store_true", help="skip the per-layer 3x3 sweep at batch 64 (BASELINE config 5)")
     ap.add_argument("--profile-steps", type=int, default=5)
-    ap.add_argument("--in-flight", type=int, default=2,
+    ap.add_argument("--in-flight", type=int, default=0,
                     help="forward passes kept in flight: step k runs on model handle and HIP stream k mod this number "
-                         "(each handle owns its workspace); 1 = one pass after the other")
+                         "(each handle owns its workspace); 1 = one pass after the other; 0 = the best of 2, 3 and 4 in a "
+                         "short trial (how many passes overlap depends on the hardware queues the runtime was given)")
+    ap.add_argument("--in-flight-batch1", type=int, default=0,
+                    help="the same for the batch-1 measurement (a batch-1 pass is a chain of 18 short launches that leaves "
+                         "most of the chip idle)")
     ap.add_argument("--workload", default="resnet18", choices=["resnet18", "mobilenetv3", "yolov5s"],
                     help="resnet18 = the headline configuration; mobilenetv3 / yolov5s = the networks of tests/Nets/MobileNetV3.mlir "
                          "and Yolov5s.mlir through the operator-list executor (same step definition, their own JSON line; "
@@ -131,16 +184,23 @@ def main():
     # Passes in flight: handle i and stream i serve steps i, i + K, i + 2K ...  A handle owns its workspace, so passes of
     # different handles overlap on the GPU (one pass's launch gaps, prologues and tails fill with the other's work); every
     # pass is still a whole forward over one batch of N images, into its own logits buffer.
-    K = max(1, args.in_flight)
-    models, keep_streams, outs, stream_objs = [model], [stream], [logits], []
-    for _ in range(1, K):
+    asked1 = 1 if args.no_batch1 else args.in_flight_batch1
+    KMAX = max(args.in_flight, asked1, max(IN_FLIGHT_CANDIDATES) if 0 in (args.in_flight, asked1) else 1)
+    models, outs = [model], [logits]
+    for _ in range(1, KMAX):
         h = L.nncv_hip_resnet18_create(blob.ctypes.data, blob.size, abi.F16, algo)
         if not h:
             raise RuntimeError(L.nncv_hip_last_error().decode())
         models.append(h)
-        stream_objs.append(torch.cuda.Stream())  # kept alive to the end of main
-        keep_streams.append(stream_objs[-1].cuda_stream)
         outs.append(torch.empty((N, 1000), dtype=torch.float32, device="cuda"))
+
+    x1 = xd[:1].contiguous()
+    l1 = [torch.empty((1, 1000), dtype=torch.float32, device="cuda") for _ in range(KMAX)]
+    pool_objs, stream_probe = [], None  # the stream objects stay alive to the end of main
+    if KMAX > 1:
+        pool_objs, stream_probe = concurrent_streams(
+            torch, lambda h, s: abi.check(L.nncv_hip_resnet18_forward(models[h], x1.data_ptr(), 1, H, H, l1[h].data_ptr(), s)), KMAX)
+    pool_streams = [t.cuda_stream for t in pool_objs]
 
     def step(xt, out, n):
         abi.check(L.nncv_hip_resnet18_forward(model, xt.data_ptr(), n, H, H, out.data_ptr(), stream))
@@ -148,7 +208,10 @@ def main():
     def timed(xt, out_list, n, warmup, steps, k_in_flight):
         def go(i):
             j = i % k_in_flight
-            abi.check(L.nncv_hip_resnet18_forward(models[j], xt.data_ptr(), n, H, H, out_list[j].data_ptr(), keep_streams[j]))
+            # with several passes in flight every handle gets a stream of its own from torch's pool; one pass at a time
+            # stays on the default stream, like every other measurement of this script
+            sj = stream if k_in_flight == 1 else pool_streams[j]
+            abi.check(L.nncv_hip_resnet18_forward(models[j], xt.data_ptr(), n, H, H, out_list[j].data_ptr(), sj))
         # clock warm-up: untimed steps until CLOCK_WARMUP_MS of wall time have passed, then the W asked for
         t_w = time.perf_counter()
         while (time.perf_counter() - t_w) * 1e3 < CLOCK_WARMUP_MS:
@@ -164,16 +227,23 @@ def main():
         torch.cuda.synchronize()  # every stream
         return (time.perf_counter() - t0) / steps
 
+    def pick_in_flight(asked, xt, out_list, n):
+        """(passes in flight, {candidate: ms per pass in the trial})"""
+        if asked > 0:
+            return asked, None
+        trial = {k: timed(xt, out_list, n, 20, max(30, args.steps // 2), k) for k in IN_FLIGHT_CANDIDATES}
+        return min(trial, key=trial.get), {str(k): round(v * 1e3, 4) for k, v in trial.items()}
+
+    K, k_trial = pick_in_flight(args.in_flight, xd, outs, N)
     sec = timed(xd, outs, N, args.warmup, args.steps, K)
     sec_serial = sec if K == 1 else timed(xd, outs, N, args.warmup, args.steps, 1)
     ips = N / sec
     flops_step = spec.flops_per_image(H) * N
 
     # batch 1 (the other half of the headline metric)
-    x1 = xd[:1].contiguous()
-    l1 = [torch.empty((1, 1000), dtype=torch.float32, device="cuda") for _ in range(K)]
-    sec1 = None if args.no_batch1 else timed(x1, l1, 1, args.warmup, max(args.steps, 50), K)
-    sec1_serial = None if args.no_batch1 else (sec1 if K == 1 else timed(x1, l1, 1, args.warmup, max(args.steps, 50), 1))
+    K1, k1_trial = (1, None) if args.no_batch1 else pick_in_flight(args.in_flight_batch1, x1, l1, 1)
+    sec1 = None if args.no_batch1 else timed(x1, l1, 1, args.warmup, max(args.steps, 50), K1)
+    sec1_serial = None if args.no_batch1 else (sec1 if K1 == 1 else timed(x1, l1, 1, args.warmup, max(args.steps, 50), 1))
 
     # event-timed per-kernel pass (separate from the timed region above: the events serialise launches)
     abi.profile_enable(True)
@@ -245,7 +315,7 @@ def main():
         "config": {"workload": "BASELINE config 4: ResNet-18 forward, fp16, input [%d,3,224,224], seeded U[0,1] input, "
                                "random-init Kaiming/BN-folded weights from a model.bin-order blob" % N,
                    "batch": N, "image": H, "algo3x3": args.algo, "input_resident_in_hbm": True,
-                   "passes_in_flight": K,
+                   "passes_in_flight": K, "passes_in_flight_trial_ms": k_trial, "stream_probe": stream_probe,
                    "passes_in_flight_note": "step k runs on model handle and HIP stream k mod %d, each handle with its own "
                                             "workspace and logits buffer; every step is one whole forward pass over one batch "
                                             "of %d images; `one_pass_at_a_time` is the same loop on one handle and one stream" % (K, N)},
@@ -255,7 +325,7 @@ def main():
         "one_pass_at_a_time": {"images_per_s": round(N / sec_serial, 2), "ms_per_step": round(sec_serial * 1e3, 4),
                                "tflops_effective": round(flops_step / sec_serial / 1e12, 3)},
         "batch1": None if sec1 is None else {"images_per_s": round(1.0 / sec1, 2), "ms_per_image": round(sec1 * 1e3, 4),
-                                             "passes_in_flight": K,
+                                             "passes_in_flight": K1, "passes_in_flight_trial_ms": k1_trial,
                                              "one_pass_at_a_time": {"images_per_s": round(1.0 / sec1_serial, 2),
                                                                     "ms_per_image": round(sec1_serial * 1e3, 4)}},
         "model_create_ms": round(t_create * 1e3, 2),
@@ -471,18 +541,25 @@ def bench_graph(args, L):
         from nncv_amd import mobilenetv3_spec as mspec
         blob32, ops = synth.mobilenetv3_params(), abi.mobilenetv3_small_ops()[0]
         name, fixture = "MobileNetV3-small", "tests/Nets/MobileNetV3.mlir"
-    K = max(1, args.in_flight)  # passes in flight: graph handle i and stream i serve steps i, i + K ... (see main)
-    gs = [abi.graph_create(ops, 3, blob32.astype(np.float16)) for _ in range(K)]
+    # passes in flight: graph handle i and stream i serve steps i, i + K ... (see main)
+    asked1 = 1 if args.no_batch1 else args.in_flight_batch1
+    KMAX = max(args.in_flight, asked1, max(IN_FLIGHT_CANDIDATES) if 0 in (args.in_flight, asked1) else 1)
+    gs = [abi.graph_create(ops, 3, blob32.astype(np.float16)) for _ in range(KMAX)]
     g = gs[0]
     oc, oh, ow = abi.graph_output_shape(g, H, H)
     per_image = oc * oh * ow
     x = synth.uniform(4000, (N, 3, H, H), 0.0, 1.0).astype(np.float16)
     xd = torch.from_numpy(x).cuda()
-    results = [torch.empty((N, per_image), dtype=torch.float32, device="cuda") for _ in range(K)]
+    results = [torch.empty((N, per_image), dtype=torch.float32, device="cuda") for _ in range(KMAX)]
     result = results[0]
     stream = torch.cuda.current_stream().cuda_stream
-    stream_objs = [torch.cuda.Stream() for _ in range(1, K)]
-    streams = [stream] + [t.cuda_stream for t in stream_objs]
+    x1 = xd[:1].contiguous()
+    r1 = [torch.empty((1, per_image), dtype=torch.float32, device="cuda") for _ in range(KMAX)]
+    pool_objs, stream_probe = [], None
+    if KMAX > 1:
+        pool_objs, stream_probe = concurrent_streams(
+            torch, lambda h, s: abi.check(L.nncv_hip_graph_forward(gs[h], x1.data_ptr(), 1, H, H, r1[h].data_ptr(), per_image, s)), KMAX)
+    pool_streams = [t.cuda_stream for t in pool_objs]
 
     def step(xt, out, n):
         abi.check(L.nncv_hip_graph_forward(g, xt.data_ptr(), n, H, H, out.data_ptr(), n * per_image, stream))
@@ -490,7 +567,8 @@ def bench_graph(args, L):
     def timed(xt, out_list, n, warmup, steps, k_in_flight):
         def go(i):
             j = i % k_in_flight
-            abi.check(L.nncv_hip_graph_forward(gs[j], xt.data_ptr(), n, H, H, out_list[j].data_ptr(), n * per_image, streams[j]))
+            sj = stream if k_in_flight == 1 else pool_streams[j]  # see main: pool streams when passes overlap
+            abi.check(L.nncv_hip_graph_forward(gs[j], xt.data_ptr(), n, H, H, out_list[j].data_ptr(), n * per_image, sj))
         # clock warm-up: untimed steps until CLOCK_WARMUP_MS of wall time have passed, then the W asked for
         t_w = time.perf_counter()
         while (time.perf_counter() - t_w) * 1e3 < CLOCK_WARMUP_MS:
@@ -506,12 +584,18 @@ def bench_graph(args, L):
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps
 
+    def pick_in_flight(asked, xt, out_list, n):
+        if asked > 0:
+            return asked, None
+        trial = {k: timed(xt, out_list, n, 20, max(30, args.steps // 2), k) for k in IN_FLIGHT_CANDIDATES}
+        return min(trial, key=trial.get), {str(k): round(v * 1e3, 4) for k, v in trial.items()}
+
+    K, k_trial = pick_in_flight(args.in_flight, xd, results, N)
     sec = timed(xd, results, N, args.warmup, args.steps, K)
     sec_serial = sec if K == 1 else timed(xd, results, N, args.warmup, args.steps, 1)
-    x1 = xd[:1].contiguous()
-    r1 = [torch.empty((1, per_image), dtype=torch.float32, device="cuda") for _ in range(K)]
-    sec1 = None if args.no_batch1 else timed(x1, r1, 1, args.warmup, max(args.steps, 50), K)
-    sec1_serial = None if args.no_batch1 else (sec1 if K == 1 else timed(x1, r1, 1, args.warmup, max(args.steps, 50), 1))
+    K1, k1_trial = (1, None) if args.no_batch1 else pick_in_flight(args.in_flight_batch1, x1, r1, 1)
+    sec1 = None if args.no_batch1 else timed(x1, r1, 1, args.warmup, max(args.steps, 50), K1)
+    sec1_serial = None if args.no_batch1 else (sec1 if K1 == 1 else timed(x1, r1, 1, args.warmup, max(args.steps, 50), 1))
     abi.profile_enable(True)
     abi.profile_report()
     for _ in range(args.profile_steps):
@@ -547,11 +631,12 @@ def bench_graph(args, L):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 (fp32 accumulate)", "data": "synthetic",
         "config": {"workload": "%s forward (the network of %s), fp16, input [%d,3,%d,%d], seeded U[0,1] input, random-init weights "
                                "from a model.bin-order blob" % (name, fixture, N, H, H),
-                   "batch": N, "image": H, "input_resident_in_hbm": True, "passes_in_flight": K},
+                   "batch": N, "image": H, "input_resident_in_hbm": True, "passes_in_flight": K,
+                   "passes_in_flight_trial_ms": k_trial, "stream_probe": stream_probe},
         "tflops_effective": round(flops_step / sec / 1e12, 3),
         "one_pass_at_a_time": {"images_per_s": round(N / sec_serial, 2), "ms_per_step": round(sec_serial * 1e3, 4)},
         "batch1": None if sec1 is None else {"images_per_s": round(1.0 / sec1, 2), "ms_per_image": round(sec1 * 1e3, 4),
-                                             "passes_in_flight": K,
+                                             "passes_in_flight": K1, "passes_in_flight_trial_ms": k1_trial,
                                              "one_pass_at_a_time": {"images_per_s": round(1.0 / sec1_serial, 2),
                                                                     "ms_per_image": round(sec1_serial * 1e3, 4)}},
         "roofline": roofline, "kernels": kernels, "device": L.nncv_hip_device_arch().decode(),

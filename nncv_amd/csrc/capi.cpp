@@ -334,7 +334,9 @@ void replay(const void* owner, const std::function<void()>& run, const void* src
   for (auto& e : cache)
     if (e.m == owner && e.src == src && e.logits == logits && e.N == N && e.H == H && e.W == W && e.ws == ws && e.s == s) hit = &e;
   if (!hit) {  // first sighting: run eagerly (this also performs every one-time kernel attribute set-up)
-    if (cache.size() >= 16) {
+    if (cache.size() >= 32) {
+      // the oldest entry goes; its last replay may still be running on another stream
+      (void)hipDeviceSynchronize();
       drop_graph(cache.front());
       cache.erase(cache.begin());
     }

@@ -127,6 +127,9 @@ def main():
                     help="forward passes kept in flight: step k runs on model handle and HIP stream k mod this number "
                          "(each handle owns its workspace); 1 = one pass after the other; 0 = the best of 2, 3 and 4 in a "
                          "short trial (how many passes overlap depends on the hardware queues the runtime was given)")
+    ap.add_argument("--no-overlap-hint", action="store_true",
+                    help="do not tell the library how many passes are in flight (nncv_hip_set_overlap_hint): it then plans "
+                         "every launch as if it had the chip to itself")
     ap.add_argument("--in-flight-batch1", type=int, default=0,
                     help="the same for the batch-1 measurement (a batch-1 pass is a chain of 18 short launches that leaves "
                          "most of the chip idle)")
@@ -212,6 +215,8 @@ def main():
             # stays on the default stream, like every other measurement of this script
             sj = stream if k_in_flight == 1 else pool_streams[j]
             abi.check(L.nncv_hip_resnet18_forward(models[j], xt.data_ptr(), n, H, H, out_list[j].data_ptr(), sj))
+        # the library plans its launches for the number of passes the caller keeps in flight
+        abi.check(L.nncv_hip_set_overlap_hint(1 if args.no_overlap_hint else k_in_flight))
         # clock warm-up: untimed steps until CLOCK_WARMUP_MS of wall time have passed, then the W asked for
         t_w = time.perf_counter()
         while (time.perf_counter() - t_w) * 1e3 < CLOCK_WARMUP_MS:
@@ -225,7 +230,9 @@ def main():
         for i in range(steps):
             go(i)
         torch.cuda.synchronize()  # every stream
-        return (time.perf_counter() - t0) / steps
+        dt = time.perf_counter() - t0
+        abi.check(L.nncv_hip_set_overlap_hint(1))
+        return dt / steps
 
     def pick_in_flight(asked, xt, out_list, n):
         """(passes in flight, {candidate: ms per pass in the trial})"""
@@ -569,6 +576,8 @@ def bench_graph(args, L):
             j = i % k_in_flight
             sj = stream if k_in_flight == 1 else pool_streams[j]  # see main: pool streams when passes overlap
             abi.check(L.nncv_hip_graph_forward(gs[j], xt.data_ptr(), n, H, H, out_list[j].data_ptr(), n * per_image, sj))
+        # the library plans its launches for the number of passes the caller keeps in flight
+        abi.check(L.nncv_hip_set_overlap_hint(1 if args.no_overlap_hint else k_in_flight))
         # clock warm-up: untimed steps until CLOCK_WARMUP_MS of wall time have passed, then the W asked for
         t_w = time.perf_counter()
         while (time.perf_counter() - t_w) * 1e3 < CLOCK_WARMUP_MS:
@@ -582,7 +591,9 @@ def bench_graph(args, L):
         for i in range(steps):
             go(i)
         torch.cuda.synchronize()
-        return (time.perf_counter() - t0) / steps
+        dt = time.perf_counter() - t0
+        abi.check(L.nncv_hip_set_overlap_hint(1))
+        return dt / steps
 
     def pick_in_flight(asked, xt, out_list, n):
         if asked > 0:

@@ -133,6 +133,15 @@ int nncv_hip_conv_time(nncv_hip_conv* c, const void* in, int N, int H, int W, co
  * `params` (all of them when `params` is NULL) are dropped and rebuilt on the next call.  Returns 0.  No counterpart
  * in the reference, whose compiled forward re-reads the blob on every call (examples/Res18/main.cpp:95-99). */
 int nncv_hip_params_invalidate(const void* params);
+/* Tells the library how many forward passes the caller keeps in flight at once (different network handles on
+ * different streams; 1 = one pass after the other, the initial value unless NNCV_HIP_OVERLAP says otherwise).  From 3
+ * up the planners choose the launch shapes that measured faster when launches of several passes share the chip (fewer,
+ * larger workgroups in the fp16 3x3 kernel; no lingering of tensors in the workspace; average pool and FC as two small
+ * launches): ResNet-18 fp16 at batch 32 with four passes in flight 0.159 against 0.168 ms per pass, but 0.275 against
+ * 0.256 ms with one pass at a time.  Results are the same tensors either way.  A change waits for the device and drops
+ * the captured graphs of every handle, so call it between phases, not per pass.  Returns 0.  No counterpart in the
+ * reference, whose compiled forward is one synchronous CPU call (examples/Res18/main.cpp:95-99). */
+int nncv_hip_set_overlap_hint(int passes);
 /* Diagnostic, host arithmetic only (works without a GPU): the tile plan of the 3x3 LDS-patch kernel for
  * N x OH x OW output pixels at `stride` (1 | 2), F filters and `slabs` 128-byte channel slabs.
  * plan[8] = {WS (64-slot groups per workgroup), TN images, TH rows, TW columns per tile, NTX column tiles per

@@ -35,7 +35,7 @@ EXPORTS = [
     "nncv_hip_profile_enable", "nncv_hip_profile_report",
     "nncv_hip_resnet18_create", "nncv_hip_resnet18_destroy", "nncv_hip_resnet18_forward",
     "nncv_hip_resnet18_forward_tap",
-    "nncv_hip_conv_create", "nncv_hip_conv_destroy", "nncv_hip_conv_algo", "nncv_hip_conv_forward", "nncv_hip_conv_forward_noalloc", "nncv_hip_conv_time", "nncv_hip_conv3x3_patch_plan", "nncv_hip_conv3x3_stream_plan", "nncv_hip_params_invalidate",
+    "nncv_hip_conv_create", "nncv_hip_conv_destroy", "nncv_hip_conv_algo", "nncv_hip_conv_forward", "nncv_hip_conv_forward_noalloc", "nncv_hip_conv_time", "nncv_hip_conv3x3_patch_plan", "nncv_hip_conv3x3_stream_plan", "nncv_hip_params_invalidate", "nncv_hip_set_overlap_hint",
     "nncv_hip_plan_arena", "nncv_hip_preprocess_u8", "nncv_hip_argmax", "nncv_hip_resnet18_classify_u8",
     "nncv_hip_matmul_f32", "nncv_hip_matmul_time", "nncv_hip_wino43_filter", "nncv_hip_wino43_input", "nncv_hip_wino43_gemm",
     "nncv_hip_wino43_output", "nncv_hip_maxpool3x3s2", "nncv_hip_global_avgpool",
@@ -92,6 +92,7 @@ def lib():
         L._mlir_ciface_batch_nchw_conv.restype = None
         L.nncv_hip_init.argtypes = [i]
         L.nncv_hip_params_invalidate.argtypes = [vp]
+        L.nncv_hip_set_overlap_hint.argtypes = [i]
         L.nncv_hip_last_error.restype = ctypes.c_char_p
         L.nncv_hip_device_arch.restype = ctypes.c_char_p
         L.nncv_hip_profile_enable.argtypes = [i]

@@ -1,20 +1,39 @@
 #include "arena_plan.hpp"
 
 #include <algorithm>
+#include <atomic>
 #include <cstdlib>
 #include <limits>
 #include <numeric>
 
 namespace nncv_hip {
 
-int arena_linger() {
-  static const int v = [] {
-    const char* e = getenv("NNCV_HIP_ARENA_LINGER");
-    const int n = e ? atoi(e) : 3;
-    return n < 0 ? 0 : n;
-  }();
+namespace {
+std::atomic<int>& overlap_state() {
+  static std::atomic<int> v{[] {
+    const char* e = getenv("NNCV_HIP_OVERLAP");
+    const int n = e ? atoi(e) : 1;
+    return n < 1 ? 1 : n;
+  }()};
   return v;
 }
+}  // namespace
+
+int overlap_hint() { return overlap_state().load(std::memory_order_relaxed); }
+void set_overlap_hint(int passes) { overlap_state().store(passes < 1 ? 1 : passes, std::memory_order_relaxed); }
+
+namespace {
+int linger_env() {
+  static const int forced = [] {
+    const char* e = getenv("NNCV_HIP_ARENA_LINGER");
+    return e ? std::max(0, atoi(e)) : -1;
+  }();
+  return forced;
+}
+}  // namespace
+
+int arena_linger() { return linger_env() >= 0 ? linger_env() : 3; }
+bool arena_linger_forced() { return linger_env() >= 0; }
 
 size_t plan_offsets(std::vector<TensorLife>& t, size_t align) {
   const size_t mask = align > 1 ? align - 1 : 0;

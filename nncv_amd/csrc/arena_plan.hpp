@@ -28,7 +28,22 @@ size_t plan_offsets(std::vector<TensorLife>& tensors, size_t align);
 // launch whose output lies where the previous launch's INPUT lay runs 2-4.4 us longer (16.4 against 12.0 us for the first
 // stride-1 convolution after a down-sampling one, 14.0 against 11.8 one stage deeper), one launch further back it is
 // still 2.3 us (13.4 against 11.1), from three launches on nothing; the whole pass gains 9 us of 256 for 20 % more
-// workspace.  NNCV_HIP_ARENA_LINGER overrides (0 = hand memory on at once).
+// workspace.  NNCV_HIP_ARENA_LINGER overrides (0 = hand memory on at once); arena_linger_forced() says that it did.
 int arena_linger();
+bool arena_linger_forced();
+
+// How many forward passes the caller says it keeps in flight on different streams (nncv_hip_set_overlap_hint; 1 unless
+// told otherwise, NNCV_HIP_OVERLAP sets the initial value).  From three up the planners pick the forms that measured
+// faster when launches of different passes share the chip -- what counts then is how long a launch's workgroups hold
+// their LDS and register slots, not how soon the launch ends: the 128-filter form of the 3x3 stream kernel wherever
+// the filter count allows it (half the workgroups of the 64-filter form, no exchange between K groups) and the patch
+// kernel's 256-slot form where it does not; in ResNet-18 from batch 16 up also no lingering in the arena (the penalty
+// it avoids belongs to launches that have the chip to themselves; four smaller working sets share the caches better:
+// 0.165 against 0.168 ms -- MobileNetV3's small tensors measured the other way, 0.169 against 0.162, and keep
+// lingering) and average pool and FC as two small launches instead of the fused head's 1024 workgroups that each pool
+// their image again.  ResNet-18 at batch 32 with four passes in flight: 0.160 against 0.174 ms per pass; one pass at a
+// time the same choices cost 7 % (0.275 against 0.256).
+int overlap_hint();
+void set_overlap_hint(int passes);
 
 }  // namespace nncv_hip

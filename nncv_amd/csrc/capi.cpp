@@ -581,6 +581,19 @@ int nncv_hip_conv3x3_patch_plan(int stride, int N, int OH, int OW, int F, int sl
   return conv3x3_patch_plan(stride, N, OH, OW, F, slabs, plan) ? 0 : 1;
 }
 
+int nncv_hip_set_overlap_hint(int passes) {
+  return guarded([&] {
+    const int want = passes < 1 ? 1 : passes;
+    if (want == overlap_hint()) return;
+    // captured passes hold the launch shapes and workspace offsets of the old setting
+    (void)hipDeviceSynchronize();
+    auto& gc = graph_cache();
+    for (auto& e : gc) drop_graph(e);
+    gc.clear();
+    set_overlap_hint(want);
+  });
+}
+
 int nncv_hip_params_invalidate(const void* params) {
   return guarded([&] {
     std::lock_guard<std::recursive_mutex> lk(Context::get().mu);

@@ -37,6 +37,7 @@
 //    split the channel slab) exchange half of their partial sums through LDS once per tile.
 #include <algorithm>
 
+#include "arena_plan.hpp"
 #include "mfma_tile.hpp"
 #include "runtime.hpp"
 
@@ -614,7 +615,9 @@ bool stream_config(int N, int H, int W, int C, int F, bool act, int only_pg, Str
     // about one workgroup per CU (224 at batch 32; 214 on 14x14x256 at batch 64) it is ahead on some runs (10.4 against
     // 10.5, 16.6 against 17.2) and far behind on others (13.9), depending on where the workgroups land, and with 108
     // (14x14x256 at batch 32) it loses outright (15.0 against 10.2): it is taken from 400 workgroups up.
-    if (c.WF == 4) c.cost = wgs >= 400 ? 0 : (1ll << 60);
+    // When the caller keeps three or more passes in flight it is taken wherever it fits: half the workgroups hold the
+    // CUs' slots for about the same time (four passes in flight, ResNet-18 at batch 32: 0.163 against 0.168 ms per pass).
+    if (c.WF == 4) c.cost = (wgs >= 400 || overlap_hint() >= 3) ? 0 : (1ll << 60);
     if (!found || c.cost < best->cost) {
       *best = c;
       found = true;
@@ -674,6 +677,10 @@ bool conv3x3_stream_applicable(const IgemmArgs& a, int in_dt, int out_dt) {
   // 5.9 / 6.3, 16x14x14x256 7.9 / 8.6, 4x56x56x64 4.9 / 5.4 (216-224 workgroups); rows of 80 pixels fill 80 of a
   // tile's 128 slots: 16x80x80x64 18.2 / 15.7, where the patch kernel cuts the rows into column tiles.
   const long long fine_wgs = (long long)c.geo.n_tiles * (a.F / 32);
+  // With three or more passes in flight (overlap_hint) a ReLU layer whose filter count rules out the 128-filter form goes
+  // to the patch kernel, whose 256-slot workgroups hold fewer slots for the same work than the 64-filter form here
+  // (ResNet-18's layer1 at batch 32, four passes in flight: 0.161 against 0.165 ms per pass).
+  if (!all && overlap_hint() >= 3 && a.relu <= kActRelu && c.WF != 4) return false;
   return all || (fine_wgs >= 160 && c.geo.TH * a.W >= 96);
 }
 

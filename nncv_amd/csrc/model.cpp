@@ -339,7 +339,8 @@ static Plan make_plan(const ConvLayer& stem, const std::vector<const ConvLayer*>
   t[ix[nb]].last_op = 26;
   const int i_pooled = add(26, 27, (size_t)N * 512 * es);
   const int i_cws = add(0, 27, cws);
-  for (auto& e : t) e.last_op = std::min(27, e.last_op + arena_linger());
+  const int linger = (overlap_hint() >= 3 && N >= 16 && !arena_linger_forced()) ? 0 : arena_linger();  // see overlap_hint
+  for (auto& e : t) e.last_op = std::min(27, e.last_op + linger);
   p.total = plan_offsets(t, 256) + 4096;
   p.stem_out = t[i_stem].offset; p.pooled = t[i_pooled].offset; p.cws = t[i_cws].offset;
   for (int k = 0; k <= nb; ++k) p.x[k] = t[ix[k]].offset;
@@ -401,7 +402,9 @@ void ResNet18::forward(const void* src, int N, int H, int W, void* logits, void*
   }
   char* body_out = base + p.x[8];
   // head: global average pool (sum, one divide), FC with bias (Res18.mlir:609-628)
-  static const bool split_head = getenv("NNCV_HIP_NO_HEAD_FUSION") != nullptr;
+  static const bool never_fused = getenv("NNCV_HIP_NO_HEAD_FUSION") != nullptr;
+  // see overlap_hint (arena_plan.hpp); at small batches the fused head is a few dozen workgroups and one launch less
+  const bool split_head = never_fused || (overlap_hint() >= 3 && N >= 16);
   if (!split_head) {
     launch_avgpool_fc(body_out, fc_w_.get(), fc_b_.as<float>(), static_cast<float*>(logits), dt_, N, h * w, 512, 1000, s);
     return;

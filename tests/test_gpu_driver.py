@@ -163,3 +163,65 @@ def test_two_handles_on_two_streams_run_concurrently_and_stay_exact(blob, dt):
     assert np.array_equal(ob.cpu().numpy(), want_b)
     ma.close()
     mb.close()
+
+
+def test_overlap_hint_changes_the_launch_shapes_not_the_results(blob):
+    """nncv_hip_set_overlap_hint(4): the planners switch to the forms meant for several passes in flight (128-filter stream
+    form on layer2 / layer3, layer1 on the patch kernel, average pool and FC as separate launches), the logits stay within
+    the fp16 bar of the oracle with its top-1, four handles on four streams each reproduce the bits of a pass run alone,
+    and hint 1 brings the usual shapes back."""
+    import torch
+    import oracle
+    from gpu_util import Model, dev, host, rel_l2, FP16_REL_L2
+    L = abi.lib()
+    hb = synth.round_fp16(blob)
+    N = 16
+    xs = [synth.round_fp16(synth.uniform(9500 + i, (N, 3, 224, 224), 0.0, 1.0)) for i in range(4)]
+
+    def tags(m, xd):
+        m(xd)
+        torch.cuda.synchronize()
+        abi.profile_enable(True)
+        try:
+            abi.profile_report()
+            got = host(m(xd))
+            rep = abi.profile_report()
+        finally:
+            abi.profile_enable(False)
+        return got, {k: v["launches"] for k, v in rep.items()}
+
+    try:
+        abi.check(L.nncv_hip_set_overlap_hint(4))
+        ms = [Model(hb, abi.F16, abi.ALGO_AUTO) for _ in range(4)]
+        xd = [dev(x, abi.F16) for x in xs]
+        alone, rep = tags(ms[0], xd[0])
+        print("hint 4:", rep, flush=True)
+        count = lambda r, prefix: sum(v for k, v in r.items() if k.startswith(prefix))
+        assert rep.get("conv3x3_stream<f16,1x4x1>", 0) == 6            # layer2 and layer3
+        assert count(rep, "conv3x3_patch") == 7 and count(rep, "conv3x3_stream") == 6  # layer1 joins layer4 on the patch kernel
+        assert count(rep, "conv3x3s2_patch") == 3 and count(rep, "igemm") == 1  # the FC of the split head
+        assert "avgpool_fc" not in rep and rep.get("global_avgpool", 0) == 1
+        want = oracle.resnet18_forward(xs[0][:4], hb)
+        assert rel_l2(alone[:4], want) < FP16_REL_L2 and (alone[:4].argmax(1) == want.argmax(1)).all()
+        # four passes in flight, repeatedly: every handle must reproduce the pass it gives alone
+        wants = [alone] + [host(ms[i](xd[i])) for i in range(1, 4)]
+        st = [torch.cuda.Stream() for _ in range(4)]
+        outs = [torch.zeros((N, 1000), dtype=torch.float32, device="cuda") for _ in range(4)]
+        torch.cuda.synchronize()
+        for it in range(6):
+            for i in range(4):
+                abi.check(L.nncv_hip_resnet18_forward(ms[i].h, xd[i].data_ptr(), N, 224, 224, outs[i].data_ptr(), st[i].cuda_stream))
+        torch.cuda.synchronize()
+        for i in range(4):
+            assert np.array_equal(outs[i].cpu().numpy(), wants[i]), i
+        # back to one pass at a time: the usual shapes, and (different K order in layer2 / layer3) the same logits
+        # to within rounding of the fp16 activations
+        abi.check(L.nncv_hip_set_overlap_hint(1))
+        again, rep1 = tags(ms[0], xd[0])
+        print("hint 1:", rep1, flush=True)
+        assert count(rep1, "conv3x3_stream") == 10 and rep1.get("avgpool_fc", 0) == 1
+        assert rel_l2(again, alone) < 5e-3
+        for m in ms:
+            m.close()
+    finally:
+        abi.check(L.nncv_hip_set_overlap_hint(1))

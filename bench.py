@@ -313,6 +313,10 @@ def main():
         roofline.update({"achieved": round(achieved, 3), "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 5),
                          "avg_launch_us": round(d["ms"] / d["launches"] * 1e3, 3), "launches": d["launches"],
                          "timing": "one HIP event pair per launch (includes ~4 us of event latency)"})
+    roofline["launch_shapes"] = ("those of one pass at a time (overlap hint 1), which the summaries under profiles/ hold; with "
+                                 "three or more passes in flight layer2 / layer3 run the same kernel's 128-filter form and "
+                                 "layer1 the patch kernel (see config.passes_in_flight), where a launch of one pass has no "
+                                 "duration of its own")
     conv3x3_flops = 13 * 2 * 56 * 56 * 64 * 64 * 9 * N  # the 13 stride-1 3x3 layers all cost the same per image
     out = {
         "metric": "resnet18_fp16_bs%d_images_per_s" % N, "value": round(ips, 2), "unit": "images/s",

@@ -36,8 +36,32 @@ def bn_params(seed, F):
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "x".join(str(v) for v in c[:5]) + "_act%d" % c[7])
 def test_stream_kernel_matches_the_oracle(case):
+    check_case(case, 9600 + CASES.index(case) * 10)
+
+
+# With three or more passes in flight (nncv_hip_set_overlap_hint) the 128-filter form is taken wherever the filter count
+# allows it, also on launches of a few dozen workgroups, and ReLU layers it does not fit go to the patch kernel.
+OVERLAP_CASES = [
+    (8, 28, 28, 128, 128, True, True, abi.ACT_RELU, "conv3x3_stream<f16,1x4x1>"),      # 56 workgroups, two slabs
+    (12, 14, 14, 256, 256, True, True, abi.ACT_RELU, "conv3x3_stream<f16,1x4x1>"),     # 40 workgroups across image borders, four slabs
+    (5, 97, 31, 64, 128, True, False, abi.ACT_RELU, "conv3x3_stream<f16,1x4x1>"),      # short last tile of an image
+    (20, 56, 56, 64, 64, True, False, abi.ACT_RELU, "conv3x3_patch<f16,4,1>"),         # 64 filters: the patch kernel's 256-slot form
+    (6, 40, 40, 128, 128, True, True, abi.ACT_HARDSWISH, "conv3x3_stream<f16,1x2x2,act>"),  # other activations keep their form
+]
+
+
+@pytest.mark.parametrize("case", OVERLAP_CASES, ids=lambda c: "x".join(str(v) for v in c[:5]) + "_act%d" % c[7])
+def test_launch_shapes_under_the_overlap_hint_match_the_oracle(case):
+    L = abi.lib()
+    try:
+        abi.check(L.nncv_hip_set_overlap_hint(4))
+        check_case(case, 9900 + OVERLAP_CASES.index(case) * 10)
+    finally:
+        abi.check(L.nncv_hip_set_overlap_hint(1))
+
+
+def check_case(case, seed):
     N, H, W, C, F, use_bn, use_res, act, tag = case
-    seed = 9600 + CASES.index(case) * 10
     print("stream case", case, flush=True)
     x = synth.round_fp16(synth.normal(seed, (N, C, H, W)))
     w = synth.round_fp16(synth.normal(seed + 1, (F, C, 3, 3), std=float(np.sqrt(2.0 / (C * 9)))))

@@ -42,9 +42,9 @@ import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
-# Hardware queues of this process (the HIP runtime's own setting, read when it initialises; its default is 4, of which
-# three serve streams other than the default one).  Streams beyond the queues share them and their work runs one after
-# the other, so passes on four streams overlap like passes on two.  Eight leave every stream used here a queue of its own.
+# Hardware queues of this process (the HIP runtime's own setting, read when it initialises; default 4).  Streams that
+# share a queue run their work one after the other; where the environment does not fix the number, eight queues make that
+# rarer.  Which streams actually overlap is measured below (concurrent_streams), whatever the number is.
 os.environ.setdefault("GPU_MAX_HW_QUEUES", "8")
 IN_FLIGHT_CANDIDATES = (2, 3, 4)
 

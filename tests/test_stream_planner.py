@@ -81,3 +81,32 @@ def test_resnet18_plans(plan, N, H, W, C, F, expect):
     check(p, N, H, W, C, F)
     for k, v in expect.items():
         assert p[k] == v, (k, p)
+
+
+def test_invariants_hold_under_the_overlap_hint(plan):
+    """nncv_hip_set_overlap_hint(4) makes the planner take the 128-filter form wherever the filter count allows it: the
+    same invariants must hold for those plans, and the hint must not leak into later tests."""
+    L = ctypes.CDLL(abi.LIB_PATH)
+    L.nncv_hip_set_overlap_hint.argtypes = [ctypes.c_int]
+    assert L.nncv_hip_set_overlap_hint(4) == 0
+    try:
+        rng = np.random.default_rng(20251127)
+        wide = 0
+        for _ in range(8000):
+            N = int(rng.choice([1, 2, 3, 8, 16, 32, 64]))
+            H, W = int(rng.integers(2, 130)), int(rng.integers(1, 129))
+            C = 64 * int(rng.integers(1, 5))
+            F = 32 * int(rng.integers(1, 13))
+            p = plan(N, H, W, C, F)
+            if p is None:
+                continue
+            check(p, N, H, W, C, F)
+            if F % 128 == 0:
+                assert (p["WF"], p["WK"]) == (4, 1), (N, H, W, C, F, p)
+                wide += 1
+        assert wide > 500
+        p = plan(32, 14, 14, 256, 256)
+        assert p["WF"] == 4 and p["FB"] == 2 and p["FB"] * p["Wpf"] == 108
+    finally:
+        assert L.nncv_hip_set_overlap_hint(1) == 0
+    assert plan(32, 14, 14, 256, 256)["WF"] == 2

@@ -191,7 +191,7 @@ def main():
     KMAX = max(args.in_flight, asked1, max(IN_FLIGHT_CANDIDATES) if 0 in (args.in_flight, asked1) else 1)
     models, outs = [model], [logits]
     for _ in range(1, KMAX):
-        h = L.nncv_hip_resnet18_create(blob.ctypes.data, blob.size, abi.F16, algo)
+        h = L.nncv_hip_resnet18_clone(model)  # its own workspace on the same device weights
         if not h:
             raise RuntimeError(L.nncv_hip_last_error().decode())
         models.append(h)

@@ -88,6 +88,13 @@ typedef struct nncv_hip_model nncv_hip_model;
  * and transforms the filters once. */
 nncv_hip_model* nncv_hip_resnet18_create(const void* params, int64_t n_elems, int dtype, int algo3x3);
 void nncv_hip_resnet18_destroy(nncv_hip_model* m);
+/* A second handle on the SAME device weights (fp16 models only; an fp32 model keeps the tickets of its K-split launches
+ * with its layers, which two passes at once would share): its own workspace, so its passes overlap with those of
+ * `m` and of other clones on other streams like those of separately created models do, without a second copy of the
+ * 23 MB of filters in memory and in the caches (four passes in flight: 0.160 against 0.163 ms per pass).  The weights
+ * live until the last handle on them is destroyed.  NULL on error.  No counterpart in the reference, whose compiled
+ * forward is stateless (examples/Res18/main.cpp:95-99). */
+nncv_hip_model* nncv_hip_resnet18_clone(nncv_hip_model* m);
 /* src: DEVICE NCHW [N,3,H,W] of the model's dtype; logits: DEVICE [N,1000] fp32.  `stream`: the caller's HIP stream
  * (the call only enqueues), or NULL for the library's own stream (the call then returns when the pass is done).
  * A handle owns its workspace: passes of different handles on different streams run concurrently (two passes in

@@ -5,6 +5,7 @@ There is no fallback: if the library is missing or cannot be loaded this module 
 """
 import ctypes
 import os
+import sys
 
 import numpy as np
 
@@ -33,7 +34,7 @@ EXPORTS = [
     "_mlir_ciface_forward", "_mlir_ciface_forward_f16", "_mlir_ciface_matmul", "_mlir_ciface_batch_nchw_conv",
     "nncv_hip_init", "nncv_hip_last_error", "nncv_hip_device_arch",
     "nncv_hip_profile_enable", "nncv_hip_profile_report",
-    "nncv_hip_resnet18_create", "nncv_hip_resnet18_destroy", "nncv_hip_resnet18_forward",
+    "nncv_hip_resnet18_create", "nncv_hip_resnet18_clone", "nncv_hip_resnet18_destroy", "nncv_hip_resnet18_forward",
     "nncv_hip_resnet18_forward_tap",
     "nncv_hip_conv_create", "nncv_hip_conv_destroy", "nncv_hip_conv_algo", "nncv_hip_conv_forward", "nncv_hip_conv_forward_noalloc", "nncv_hip_conv_time", "nncv_hip_conv3x3_patch_plan", "nncv_hip_conv3x3_stream_plan", "nncv_hip_params_invalidate", "nncv_hip_set_overlap_hint",
     "nncv_hip_plan_arena", "nncv_hip_preprocess_u8", "nncv_hip_argmax", "nncv_hip_resnet18_classify_u8",
@@ -79,6 +80,13 @@ def lib():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise RuntimeError("%s is missing: run `python -m nncv_amd.build` (needs hipcc)" % LIB_PATH)
+        # A process must hold ONE HIP runtime.  PyTorch ships its own copy of it: imported AFTER this library was loaded
+        # (which brings in the system's copy), torch finds "no HIP GPUs"; imported before, both use torch's copy.
+        if "torch" not in sys.modules:
+            try:
+                import torch  # noqa: F401
+            except ImportError:
+                pass
         L = ctypes.CDLL(LIB_PATH)
         vp, i, i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64
         P = ctypes.POINTER
@@ -101,6 +109,8 @@ def lib():
         L.nncv_hip_profile_report.restype = ctypes.c_size_t
         L.nncv_hip_resnet18_create.argtypes = [vp, i64, i, i]
         L.nncv_hip_resnet18_create.restype = vp
+        L.nncv_hip_resnet18_clone.argtypes = [vp]
+        L.nncv_hip_resnet18_clone.restype = vp
         L.nncv_hip_resnet18_destroy.argtypes = [vp]
         L.nncv_hip_resnet18_destroy.restype = None
         L.nncv_hip_resnet18_forward.argtypes = [vp, vp, i, i, i, vp, vp]

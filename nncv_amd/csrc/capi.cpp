@@ -472,7 +472,7 @@ void forward_abi(nncv_memref2d* dst, nncv_memref4d* src, void* params, int dt) {
 }
 
 struct nncv_hip_model_impl {
-  std::unique_ptr<ResNet18> m;
+  std::shared_ptr<ResNet18> m;  // shared with the handle's clones
   HandleState st;
 };
 struct nncv_hip_conv_impl {
@@ -652,6 +652,17 @@ nncv_hip_model* nncv_hip_resnet18_create(const void* params, int64_t n_elems, in
       h = nullptr;
       throw;
     }
+  });
+  return rc == 0 ? h : nullptr;
+}
+
+nncv_hip_model* nncv_hip_resnet18_clone(nncv_hip_model* m) {
+  nncv_hip_model* h = nullptr;
+  const int rc = guarded([&] {
+    NNCV_REQUIRE(m && m->m, "null argument");
+    NNCV_REQUIRE(m->m->dtype() == kF16, "clone: fp16 models only (an fp32 model's K-split tickets belong to its layers)");
+    h = new nncv_hip_model();
+    h->m = m->m;
   });
   return rc == 0 ? h : nullptr;
 }

@@ -127,6 +127,15 @@ class Model:
                                                           tap_stage, tap.data_ptr(), None))
         return logits, tap
 
+    def clone(self):
+        """Another handle on the same device weights (nncv_hip_resnet18_clone), with a workspace of its own."""
+        c = Model.__new__(Model)
+        c.dt = self.dt
+        c.h = abi.lib().nncv_hip_resnet18_clone(self.h)
+        if not c.h:
+            raise abi.NncvHipError(abi.lib().nncv_hip_last_error().decode())
+        return c
+
     def close(self):
         if self.h and abi is not None:
             abi.lib().nncv_hip_resnet18_destroy(self.h)

@@ -19,6 +19,7 @@ import threading
 
 import numpy as np
 import pytest
+import torch  # before the library is loaded: one HIP runtime per process (see nncv_amd/abi.py)
 
 import oracle
 from nncv_amd import abi, build, modelbin, synth
@@ -192,7 +193,8 @@ def test_overlap_hint_changes_the_launch_shapes_not_the_results(blob):
 
     try:
         abi.check(L.nncv_hip_set_overlap_hint(4))
-        ms = [Model(hb, abi.F16, abi.ALGO_AUTO) for _ in range(4)]
+        ms = [Model(hb, abi.F16, abi.ALGO_AUTO)]
+        ms += [ms[0].clone() for _ in range(3)]  # three more handles on the same device weights, each with its own workspace
         xd = [dev(x, abi.F16) for x in xs]
         alone, rep = tags(ms[0], xd[0])
         print("hint 4:", rep, flush=True)
@@ -225,3 +227,27 @@ def test_overlap_hint_changes_the_launch_shapes_not_the_results(blob):
             m.close()
     finally:
         abi.check(L.nncv_hip_set_overlap_hint(1))
+
+
+def test_clones_share_the_weights_and_outlive_the_first_handle(blob):
+    """nncv_hip_resnet18_clone: the clone gives the bits of the model it was made from, keeps working after that model's
+    handle is destroyed (the weights live until the last handle goes), and is refused for fp32 models, whose K-split
+    tickets belong to the layers."""
+    import pytest
+    from gpu_util import Model, dev, host
+    hb = synth.round_fp16(blob)
+    x = dev(synth.round_fp16(synth.uniform(9700, (3, 3, 96, 128), 0.0, 1.0)), abi.F16)
+    first = Model(hb, abi.F16, abi.ALGO_AUTO)
+    want = host(first(x))
+    twin = first.clone()
+    assert np.array_equal(host(twin(x)), want)
+    first.close()
+    assert np.array_equal(host(twin(x)), want)
+    again = twin.clone()
+    twin.close()
+    assert np.array_equal(host(again(x)), want)
+    again.close()
+    m32 = Model(blob, abi.F32, abi.ALGO_AUTO)
+    with pytest.raises(abi.NncvHipError, match="fp16 models only"):
+        m32.clone()
+    m32.close()

@@ -614,10 +614,12 @@ bool stream_config(int N, int H, int W, int C, int F, bool act, int only_pg, Str
     // 64-filter form on 28x28x128: 18.1 / 66.4 us against 18.8 / 68.5 at batch 64 / 256 (448 / 512 workgroups).  With
     // about one workgroup per CU (224 at batch 32; 214 on 14x14x256 at batch 64) it is ahead on some runs (10.4 against
     // 10.5, 16.6 against 17.2) and far behind on others (13.9), depending on where the workgroups land, and with 108
-    // (14x14x256 at batch 32) it loses outright (15.0 against 10.2): it is taken from 400 workgroups up.
+    // (14x14x256 at batch 32) it loses outright (15.0 against 10.2): it is taken from 400 workgroups up, and from 160
+    // where a tile walks four slabs or more (14x14x256, same box, three runs each: 160 workgroups at batch 48 15.6
+    // against 17.8 us, 214 at batch 64 18.1 against 19.2, 320 at batch 96 31.2 against 32.5).
     // When the caller keeps three or more passes in flight it is taken wherever it fits: half the workgroups hold the
     // CUs' slots for about the same time (four passes in flight, ResNet-18 at batch 32: 0.163 against 0.168 ms per pass).
-    if (c.WF == 4) c.cost = (wgs >= 400 || overlap_hint() >= 3) ? 0 : (1ll << 60);
+    if (c.WF == 4) c.cost = (wgs >= 400 || (wgs >= 160 && C >= 256) || overlap_hint() >= 3) ? 0 : (1ll << 60);
     if (!found || c.cost < best->cost) {
       *best = c;
       found = true;

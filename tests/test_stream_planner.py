@@ -73,6 +73,7 @@ def test_invariants_on_random_shapes(plan):
     (32, 28, 28, 128, 128, dict(TH=4, aligned=1, tiles=224, WF=2, WK=2, FB=2)),       # layer2, the roofline kernel's shape
     (32, 14, 14, 256, 256, dict(TH=9, aligned=0, S=15, WF=2, FB=4)),                  # layer3: images one zero row apart
     (64, 28, 28, 128, 128, dict(TH=4, tiles=448, WF=4, WK=1, FB=1)),                  # batch 64: 128 filters per workgroup, no K groups
+    (64, 14, 14, 256, 256, dict(TH=9, aligned=0, WF=4, WK=1, FB=2, Wpf=107)),         # four slabs per tile: 128 filters from 160 workgroups
     (1, 28, 28, 128, 128, dict(WF=1, WK=4)),                                          # batch 1: 32-filter blocks fill more CUs
 ])
 def test_resnet18_plans(plan, N, H, W, C, F, expect):

@@ -157,10 +157,12 @@ int nncv_hip_set_overlap_hint(int passes);
  * (a plan that overflows LDS or the loader would fault on the device). */
 int nncv_hip_conv3x3_patch_plan(int stride, int N, int OH, int OW, int F, int slabs, int* plan);
 /* Diagnostic, host arithmetic only: the launch plan of the fp16 3x3 stride-1 stream kernel for N x H x W pixels, C
- * channels and F filters.  plan[12] = {TH virtual rows per tile, S virtual rows per image, top (1: the images are one
+ * channels and F filters.  plan[14] = {TH virtual rows per tile, S virtual rows per image, top (1: the images are one
  * zero row apart), aligned (1: tiles never leave their image), tiles, NSEG seven-cell segments per patch row, PG pixel
  * groups, WF filter groups, WK K groups of a workgroup, filter blocks, workgroups per filter block (= the tile step of a
- * workgroup), row segments one patch buffer holds}.  Returns 0, or 1 when the kernel does not take the shape.
+ * workgroup), row segments one patch buffer holds, spare bytes behind the segments of a patch row (they bring the row
+ * pitch to 9 W sixteen-byte units mod 16, which keeps the pixel reads free of bank conflicts; 0: plain segment rows),
+ * bytes of one patch buffer}.  Returns 0, or 1 when the kernel does not take the shape.
  * No counterpart in the reference: it lets the CPU test suite check that a plan never outgrows the kernel's LDS. */
 int nncv_hip_conv3x3_stream_plan(int N, int H, int W, int C, int F, int* plan);
 

@@ -201,7 +201,7 @@ bool launch_conv3x3_stream(const IgemmArgs& a, hipStream_t s);
 // The stream kernel's launch plan for N images of H x W with C channels and F filters: out = {TH, S, top, aligned, tiles,
 // segments per patch row, pixel groups, filter groups, K groups, filter blocks, workgroups per filter block, segment
 // capacity of a patch buffer}; host arithmetic only (no device needed); false = no plan.
-bool conv3x3_stream_plan(int N, int H, int W, int C, int F, int out[12]);
+bool conv3x3_stream_plan(int N, int H, int W, int C, int F, int out[14]);
 size_t weight_frag32_bytes(int F, int C);
 void launch_weight_frag32(const void* w, int w_dt, void* dst, int F, int C, hipStream_t s);
 // Stride-2 image convolutions over pixel pairs (C = 8, fp16, 6x3 and 3x2 windows, at most 64 filters):

@@ -21,8 +21,15 @@
 //    row apart and tiles run across image borders (gap form: that shared row is the halo of both images);
 //    14x14 and 7x7 images fill 126 of 128 slots that way instead of 98.
 //  * Patch cells (the 64 channels of one pixel, 128 bytes) are 144 bytes apart in LDS, which keeps the 16-byte
-//    reads of 32 neighbouring cells off each other's banks.  A load instruction fills a row segment of seven
-//    cells: 63 lanes x 16 bytes = 7 x 144 (lane 63 writes what lane 0 of the next segment overwrites).
+//    reads of 16 neighbouring cells off each other's banks (64 banks of 4 bytes: a read is conflict-free when its
+//    16-byte units differ mod 16 within every 16 lanes, and 9 is odd).  Consecutive pixel slots wrap from the
+//    end of one patch row to the start of the next, so the pitch of a patch row is chosen to continue that
+//    sequence: row pitch = 9 W units (mod 16), which for W a multiple of seven is one 16-byte unit more than the
+//    row's segments.  Slots past the last pixel of a tile read the cell of the slot 16, 32 .. before them (same
+//    bank group, never a conflict).  Measured with a micro-benchmark of the read alone: 28 and 14 pixel rows at
+//    the plain segment pitch cost 1.6x and 2.1x the cycles of a conflict-free read, at this pitch 1.0x.
+//    A load instruction fills a row segment of seven cells: 63 lanes x 16 bytes = 7 x 144 (lane 63 writes what
+//    lane 0 of the next segment overwrites, or the spare unit at the end of the row).
 //    Which pixel a lane fetches is worked out once per tile, one segment per lane, and dealt to the nine
 //    load instructions of a wave with ds_bpermute; a lane whose cell is padding, halo outside the image or
 //    past the tile asks for an offset beyond the buffer and gets zeros.  Every wave issues all nine loads
@@ -52,10 +59,11 @@ constexpr int kPitchS = 144;                      // LDS bytes per patch cell: 1
 constexpr int kSegCells = 7;                      // patch cells one load instruction fills: 63 lanes x 16 bytes = 7 x 144
 constexpr int kSegB = kSegCells * kPitchS;        // 1008 bytes
 constexpr int kLoadsPerWave = 9;                  // patch load instructions per wave and stage, always all issued
-// row segments per patch buffer and its bytes (the segments and the 16 bytes the last lane of the last one writes) for a
-// workgroup of nw waves: 36352 bytes for four waves, 72640 for eight
+// row segments per patch buffer and its bytes (the segments, the 16 bytes the last lane of the last one writes and
+// the units that bring the row pitch to 9 W mod 16) for a workgroup of nw waves: 39424 bytes for four waves, 75712 for eight
 constexpr int seg_cap(int nw) { return nw * kLoadsPerWave; }
-constexpr int patch_bytes(int nw) { return seg_cap(nw) * kSegB + 64; }
+constexpr int kRowPadB = 3072;
+constexpr int patch_bytes(int nw) { return seg_cap(nw) * kSegB + 64 + kRowPadB; }
 constexpr unsigned kOOBs = 0x80000000u;           // buffer offsets at or above this are out of range
 constexpr int kRing = 9;                          // weight fragments in flight per wave (K steps ahead)
 constexpr int kXcds = 8;
@@ -78,7 +86,7 @@ struct StreamArgs {
   unsigned N_TH;               // N | TH << 24
   unsigned geom;               // H | W << 8 | S << 16 | NSEG << 24
   unsigned pixB;               // bytes between input pixels
-  unsigned spare;
+  unsigned rowx_rnseg;         // bytes a patch row is longer than its segments | ceil(2^16 / NSEG) << 16 (0 when NSEG is 1)
   // ---- the end of a tile needs these ----
   void* out;              // NHWC [N][H][W][ldo]
   const float* scale;     // [F] or null
@@ -123,7 +131,9 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
   const unsigned top = (a.tstep_nslab_flags >> 26) & 1u;
   const unsigned N = a.N_TH & 0xffffffu, TH = a.N_TH >> 24;
   const unsigned H = a.geom & 0xffu, W = (a.geom >> 8) & 0xffu, S = (a.geom >> 16) & 0xffu, NSEG = a.geom >> 24;
-  const int PWp = (int)NSEG * kSegCells;  // cells per patch row in LDS
+  const int XB = (int)(a.rowx_rnseg & 0xffffu);  // spare bytes behind the segments of a patch row
+  const int RPB = (int)NSEG * kSegB + XB;        // LDS bytes from one patch row to the next
+  const unsigned rnseg = a.rowx_rnseg >> 16;
   // 32-slot rows of the tile this wave's pixel group holds: four, or what is left of the tile's
   const int trows = (int)((TH * W + 31u) >> 5);
   const int nrows = PG == 1 ? 4 : (trows - 4 * pg < 4 ? (trows - 4 * pg < 0 ? 0 : trows - 4 * pg) : 4);
@@ -179,7 +189,7 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
   const int perm0 = (int)lcell * 4;  // permute address of this lane's cell in the wave's first segment
   // the cell this lane computes offsets for: number lane of the wave's 63 (+ the first of the next wave's)
   const unsigned cseg = (unsigned)wave * kLoadsPerWave + (((unsigned)lane * 37u) >> 8);  // its segment: lane / 7
-  const unsigned crow = NSEG == 1 ? cseg : (cseg * (65535u / NSEG + 1u)) >> 16;            // its patch row: cseg / NSEG
+  const unsigned crow = NSEG == 1 ? cseg : (cseg * rnseg) >> 16;                           // its patch row: cseg / NSEG
   const unsigned ccol = (cseg - crow * NSEG) * kSegCells + ((unsigned)lane - (((unsigned)lane * 37u) >> 8) * 7u) - 1u;  // image column
   const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(a.in, a.in_bytes);
   unsigned celloff = kOOBs;  // tensor offset of that cell for the tile being loaded
@@ -201,6 +211,13 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
     pc_lchslab = lchoff + (unsigned)slab * 128u;
     pc_dst = dstbuf + wave * (kLoadsPerWave * kSegB);
   };
+  // segment 9 * wave + pp starts its row's spare bytes times its row further down than in a row of segments alone
+  int segx[kLoadsPerWave];
+#pragma unroll
+  for (int pp = 0; pp < kLoadsPerWave; ++pp) {
+    const unsigned sg = (unsigned)wave * kLoadsPerWave + (unsigned)pp;
+    segx[pp] = pp * kSegB + (int)(NSEG == 1 ? sg : (sg * rnseg) >> 16) * XB;
+  }
   unsigned pc_vo = 0;
   auto patch_piece_perm = [&](auto p_c) {  // the lanes' cell offsets for piece p
     constexpr int pp = decltype(p_c)::value;
@@ -210,7 +227,7 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
     constexpr int pp = decltype(p_c)::value;
     // out of range stays out of range under this sum, except for the pad chunk of a cell that is itself out of
     // range (the two flags cancel): that unit then loads the tensor's first bytes into a pad nobody reads
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_in, (lds_ptr_t)(smem + pc_dst + pp * kSegB), 16, pc_vo + pc_lchslab, 0, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_in, (lds_ptr_t)(smem + pc_dst + segx[pp]), 16, pc_vo + pc_lchslab, 0, 0, 0);
   };
   // the first patch of a workgroup: nothing to hide the permutes' latency under, so all nine go out before the loads
   auto patch_all = [&]() {
@@ -219,7 +236,7 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
     for (int pp = 0; pp < kLoadsPerWave; ++pp) pv[pp] = (unsigned)__builtin_amdgcn_ds_bpermute(perm0 + 28 * pp, (int)celloff);
 #pragma unroll
     for (int pp = 0; pp < kLoadsPerWave; ++pp)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_in, (lds_ptr_t)(smem + pc_dst + pp * kSegB), 16, pv[pp] + pc_lchslab, 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_in, (lds_ptr_t)(smem + pc_dst + segx[pp]), 16, pv[pp] + pc_lchslab, 0, 0, 0);
   };
 
   patch_tile(tile, true);
@@ -258,11 +275,15 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
   int rowbase[3][4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const unsigned s = (unsigned)(pg * kSlots + j * 32 + lrow);
+    unsigned s = (unsigned)(pg * kSlots + j * 32 + lrow);
+    const unsigned live = TH * W;
+    if (s >= live) {  // a slot without a pixel reads with the last slot that has one and sits a multiple of 16 before it
+      const unsigned back = (((s - live) >> 4) + 1u) << 4;
+      s = s >= back ? s - back : 0u;
+    }
     const unsigned ty = (s * a.mW16) >> 16, tx = s - ty * W;
-    const int cell = ty < TH ? (int)(ty * (unsigned)PWp + tx) : 0;
 #pragma unroll
-    for (int r = 0; r < 3; ++r) rowbase[r][j] = (cell + r * PWp) * kPitchS + (lchunk + 2 * wk * KPG) * 16;
+    for (int r = 0; r < 3; ++r) rowbase[r][j] = (int)(ty + r) * RPB + (int)tx * kPitchS + (lchunk + 2 * wk * KPG) * 16;
   }
   const int f0 = fb * BF + wf * 32 + 16 * lchunk;    // this lane's 16 consecutive output channels
   unsigned obase[NOWN];  // of the slot groups wk*NOWN .. +NOWN-1, the ones this wave finishes
@@ -284,7 +305,7 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
 
   floatx16 acc[4];
   // the first patch is older than the six fragments and the two scale / shift loads requested after it
-  __builtin_amdgcn_s_waitcnt(vmcnt_only(8));
+  __builtin_amdgcn_s_waitcnt(vmcnt_only(kRing - 1));
   __syncthreads();
 
   int stage_no = 0;
@@ -508,6 +529,7 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
 
 struct StreamGeom {
   int TH = 0, NSEG = 0, S = 0, top = 0, aligned = 0, n_tiles = 0;
+  int rowx = 0;  // spare bytes behind the segments of a patch row in LDS
 };
 
 unsigned recip32(unsigned d) { return d == 1 ? 0u : (unsigned)(0xffffffffull / d + 1); }  // ceil(2^32 / d) for d >= 2
@@ -530,6 +552,15 @@ bool stream_geometry(int N, int H, int W, int slots, int segcap, StreamGeom* g) 
   const long long tiles_g = (rows_g + thmax - 1) / thmax;
   const bool gap = tiles_g < tiles_a;
   g->NSEG = NSEG;
+  // The pitch of a patch row in 16-byte units is 9 W mod 16: the slot after the last pixel of a row then reads the bank
+  // group after that pixel's, like a neighbour in the row.  At least one unit (the last lane of the row's last load
+  // instruction writes it).  When that outgrows the buffer (every segment a wave may load needs a place, also the ones
+  // below the patch) the rows stay segments alone, with the bank conflicts that brings.
+  {
+    const int units = NSEG * (kSegB / 16) + 1, pad = ((9 * W - units) % 16 + 16) % 16;
+    g->rowx = 16 * (1 + pad);
+    if (segcap * kSegB + ((segcap - 1) / NSEG) * g->rowx + 16 > segcap * kSegB + 64 + kRowPadB) g->rowx = 0;
+  }
   if (gap) {
     g->TH = thmax; g->S = H + 1; g->top = 1; g->aligned = 0; g->n_tiles = (int)tiles_g;
   } else {
@@ -651,12 +682,13 @@ void launch_weight_frag32(const void* w, int w_dt, void* dst, int F, int C, hipS
   NNCV_HIP_CHECK(hipGetLastError());
 }
 
-bool conv3x3_stream_plan(int N, int H, int W, int C, int F, int out[12]) {
+bool conv3x3_stream_plan(int N, int H, int W, int C, int F, int out[14]) {
   StreamConfig c;
   if (!stream_config(N, H, W, C, F, false, 0, &c)) return false;
   const StreamGeom& g = c.geo;
   out[0] = g.TH; out[1] = g.S; out[2] = g.top; out[3] = g.aligned; out[4] = g.n_tiles; out[5] = g.NSEG;
   out[6] = c.PG; out[7] = c.WF; out[8] = c.WK; out[9] = c.FB; out[10] = c.Wpf; out[11] = seg_cap(4 * c.PG);
+  out[12] = g.rowx; out[13] = patch_bytes(4 * c.PG);
   return true;
 }
 
@@ -727,6 +759,7 @@ bool launch_conv3x3_stream(const IgemmArgs& g, hipStream_t s) {
   a.N_TH = (unsigned)g.N | ((unsigned)geo.TH << 24);
   a.geom = (unsigned)g.H | ((unsigned)g.W << 8) | ((unsigned)geo.S << 16) | ((unsigned)geo.NSEG << 24);
   a.pixB = (unsigned)pix * 2u;
+  a.rowx_rnseg = (unsigned)geo.rowx | (geo.NSEG == 1 ? 0u : (unsigned)(65535 / geo.NSEG + 1) << 16);
   a.mW16 = (unsigned)((65536 + g.W - 1) / g.W);
   const double P = (double)g.N * g.H * g.W;
   const double flops = 2.0 * P * g.C * 9.0 * g.F;

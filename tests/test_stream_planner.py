@@ -10,7 +10,7 @@ import pytest
 
 from nncv_amd import abi
 
-KEYS = ("TH", "S", "top", "aligned", "tiles", "NSEG", "PG", "WF", "WK", "FB", "Wpf", "segcap")
+KEYS = ("TH", "S", "top", "aligned", "tiles", "NSEG", "PG", "WF", "WK", "FB", "Wpf", "segcap", "rowx", "patch_bytes")
 
 
 @pytest.fixture(scope="module")
@@ -20,7 +20,7 @@ def plan():
     L.nncv_hip_conv3x3_stream_plan.restype = ctypes.c_int
 
     def call(N, H, W, C, F):
-        out = (ctypes.c_int * 12)()
+        out = (ctypes.c_int * 14)()
         if L.nncv_hip_conv3x3_stream_plan(N, H, W, C, F, out) != 0:
             return None
         return dict(zip(KEYS, out))
@@ -34,7 +34,24 @@ def check(p, N, H, W, C, F):
     assert 1 <= p["TH"] and p["TH"] * W <= slots                         # every pixel of a tile has an MFMA slot
     assert p["NSEG"] * 7 >= W + 2                                        # a patch row holds the row and its two halo cells
     assert (p["TH"] + 2) * p["NSEG"] <= p["segcap"]                      # the patch fits one LDS buffer
-    assert 2 * (p["segcap"] * 1008 + 64) + 2 * 32 * p["WF"] * 4 <= (80 if p["PG"] == 1 else 160) * 1024  # two workgroups per CU (one of eight waves)
+    assert 2 * p["patch_bytes"] + 2 * 32 * p["WF"] * 4 <= (80 if p["PG"] == 1 else 160) * 1024  # two workgroups per CU (one of eight waves)
+    # rows of the patch in LDS: NSEG segments of 1008 bytes and `rowx` spare bytes.  Every segment a wave may load (also
+    # the ones below the patch, which load zeros) and the 16 bytes its last lane writes stay inside the buffer
+    assert p["rowx"] % 16 == 0 and 0 <= p["rowx"] <= 256
+    last = p["segcap"] - 1
+    assert last * 1008 + (last // p["NSEG"]) * p["rowx"] + 1008 + 16 <= p["patch_bytes"]
+    if p["rowx"]:
+        # the pitch continues the bank sequence of a row: the slot after a row's last pixel is the next row's first
+        assert ((p["NSEG"] * 1008 + p["rowx"]) // 16 - 9 * W) % 16 == 0
+        slots_cells = []
+        for s in range(slots):
+            e = s
+            if e >= p["TH"] * W:
+                e = max(0, e - (((e - p["TH"] * W) >> 4) + 1) * 16)
+            slots_cells.append(((e // W) * (p["NSEG"] * 1008 + p["rowx"]) + (e % W) * 144) // 16)
+        if p["TH"] * W >= 16:
+            for g0 in range(0, slots, 16):
+                assert len({u % 16 for u in slots_cells[g0:g0 + 16]}) == 16, (N, H, W, g0)  # no two of 16 lanes share a bank group
     assert 2 <= p["S"] <= 255
     if p["aligned"]:
         assert p["top"] == 0 and p["S"] % p["TH"] == 0 and p["S"] >= H   # a whole number of tiles per image

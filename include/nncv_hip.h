@@ -87,6 +87,26 @@ typedef struct nncv_hip_model nncv_hip_model;
 /* params: HOST pointer to the flat blob (n_elems elements of `dtype`). Uploads, folds BN, re-lays
  * and transforms the filters once. */
 nncv_hip_model* nncv_hip_resnet18_create(const void* params, int64_t n_elems, int dtype, int algo3x3);
+/* The same, for a caller that keeps `passes_in_flight` forward passes in flight at once (this handle and its clones, each
+ * on a stream of its own; nncv_hip_pick_streams finds streams that overlap).  The value belongs to the handle: from 3 up
+ * its launches take the shapes that measured faster when launches of several passes share the chip (fewer, larger
+ * workgroups in the fp16 3x3 kernel; no lingering of tensors in the workspace; average pool and FC as two small
+ * launches): ResNet-18 fp16 at batch 32 with four passes in flight 0.159 against 0.168 ms per pass, but 0.275 against
+ * 0.256 ms with one pass at a time.  Results are the same tensors either way, and handles with different values work
+ * side by side in one process.  0 = follow the process-wide default (nncv_hip_set_overlap_hint).  No counterpart in the
+ * reference, whose compiled forward is one synchronous CPU call (examples/Res18/main.cpp:95-99). */
+nncv_hip_model* nncv_hip_resnet18_create_ex(const void* params, int64_t n_elems, int dtype, int algo3x3, int passes_in_flight);
+/* the value the handle plans with (its own, or the process-wide default); -1 for a null handle */
+int nncv_hip_resnet18_passes_in_flight(const nncv_hip_model* m);
+/* `want` (1..8) HIP streams for keeping several passes in flight, written to streams[0..want) as hipStream_t.  Streams
+ * of one process share a few hardware queues, and queues share the command processor's four pipes; work on two streams
+ * overlaps only when they landed on different pipes, which cannot be asked, so the library measures it once per process
+ * (about 40 ms: chains of short one-wave kernels on eight candidate streams, pairwise) and hands out the streams that ran
+ * side by side first.  *overlapping (may be NULL) = how many of the returned streams overlap pairwise; the rest fill the
+ * list up.  More hardware queues (GPU_MAX_HW_QUEUES=8 in the environment before the process first touches HIP) make
+ * four overlapping streams more likely.  The streams have the default priority, belong to the library and live until
+ * the process ends.  No counterpart in the reference. */
+int nncv_hip_pick_streams(int want, void** streams, int* overlapping);
 void nncv_hip_resnet18_destroy(nncv_hip_model* m);
 /* A second handle on the SAME device weights (fp16 models only; an fp32 model keeps the tickets of its K-split launches
  * with its layers, which two passes at once would share): its own workspace, so its passes overlap with those of
@@ -94,7 +114,7 @@ void nncv_hip_resnet18_destroy(nncv_hip_model* m);
  * 23 MB of filters in memory and in the caches (four passes in flight: 0.160 against 0.163 ms per pass).  The weights
  * live until the last handle on them is destroyed.  NULL on error.  No counterpart in the reference, whose compiled
  * forward is stateless (examples/Res18/main.cpp:95-99). */
-nncv_hip_model* nncv_hip_resnet18_clone(nncv_hip_model* m);
+nncv_hip_model* nncv_hip_resnet18_clone(nncv_hip_model* m);  /* inherits passes_in_flight */
 /* src: DEVICE NCHW [N,3,H,W] of the model's dtype; logits: DEVICE [N,1000] fp32.  `stream`: the caller's HIP stream
  * (the call only enqueues), or NULL for the library's own stream (the call then returns when the pass is done).
  * A handle owns its workspace: passes of different handles on different streams run concurrently (two passes in
@@ -125,7 +145,10 @@ int nncv_hip_conv_forward(nncv_hip_conv* c, const void* in, int N, int H, int W,
  * workspace the layer's kernels need (the partial sums and ticket counters of the K split of fp32 3x3 layers) is a
  * device array of the library, 4 MiB + 1 KiB on every GPU it runs on, held until the process ends; the call allocates
  * and frees nothing.  A layer/shape whose workspace is larger fails with an error that says so.  All calls on one GPU
- * share the array: calls that overlap in time on one GPU race (calls on one stream, or ordered by events, do not). */
+ * share the array.  Outside a capture the library orders them itself: a call on another stream than the previous one
+ * first waits for the event that call left behind.  On a stream that is being captured it neither waits nor records
+ * (either would end the capture): the recorded launches run when the caller's graph does, and keeping two such graphs,
+ * or a graph and eager calls, from overlapping in time on one GPU is then the caller's business -- they would race. */
 int nncv_hip_conv_forward_noalloc(nncv_hip_conv* c, const void* in, int N, int H, int W, const void* residual, void* out,
                                   void* stream);
 /* Measurement helper: `reps` NHWC launches of the layer back to back on `stream` between one pair
@@ -140,14 +163,11 @@ int nncv_hip_conv_time(nncv_hip_conv* c, const void* in, int N, int H, int W, co
  * `params` (all of them when `params` is NULL) are dropped and rebuilt on the next call.  Returns 0.  No counterpart
  * in the reference, whose compiled forward re-reads the blob on every call (examples/Res18/main.cpp:95-99). */
 int nncv_hip_params_invalidate(const void* params);
-/* Tells the library how many forward passes the caller keeps in flight at once (different network handles on
- * different streams; 1 = one pass after the other, the initial value unless NNCV_HIP_OVERLAP says otherwise).  From 3
- * up the planners choose the launch shapes that measured faster when launches of several passes share the chip (fewer,
- * larger workgroups in the fp16 3x3 kernel; no lingering of tensors in the workspace; average pool and FC as two small
- * launches): ResNet-18 fp16 at batch 32 with four passes in flight 0.159 against 0.168 ms per pass, but 0.275 against
- * 0.256 ms with one pass at a time.  Results are the same tensors either way.  A change waits for the device and drops
- * the captured graphs of every handle, so call it between phases, not per pass.  Returns 0.  No counterpart in the
- * reference, whose compiled forward is one synchronous CPU call (examples/Res18/main.cpp:95-99). */
+/* The process-wide DEFAULT of passes_in_flight (see nncv_hip_resnet18_create_ex): what handles created without a value
+ * of their own, the operator-list executor and the single-layer entry points plan with (1 = one pass after the other,
+ * the initial value unless NNCV_HIP_OVERLAP says otherwise).  Handles that carry their own value are not affected.  A
+ * change waits for the device and drops every captured graph, so call it between phases, not per pass.  Returns 0.
+ * No counterpart in the reference. */
 int nncv_hip_set_overlap_hint(int passes);
 /* Diagnostic, host arithmetic only (works without a GPU): the tile plan of the 3x3 LDS-patch kernel for
  * N x OH x OW output pixels at `stride` (1 | 2), F filters and `slabs` 128-byte channel slabs.

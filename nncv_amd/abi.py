@@ -36,7 +36,7 @@ EXPORTS = [
     "nncv_hip_profile_enable", "nncv_hip_profile_report",
     "nncv_hip_resnet18_create", "nncv_hip_resnet18_clone", "nncv_hip_resnet18_destroy", "nncv_hip_resnet18_forward",
     "nncv_hip_resnet18_forward_tap",
-    "nncv_hip_conv_create", "nncv_hip_conv_destroy", "nncv_hip_conv_algo", "nncv_hip_conv_forward", "nncv_hip_conv_forward_noalloc", "nncv_hip_conv_time", "nncv_hip_conv3x3_patch_plan", "nncv_hip_conv3x3_stream_plan", "nncv_hip_params_invalidate", "nncv_hip_set_overlap_hint",
+    "nncv_hip_conv_create", "nncv_hip_conv_destroy", "nncv_hip_conv_algo", "nncv_hip_conv_forward", "nncv_hip_conv_forward_noalloc", "nncv_hip_conv_time", "nncv_hip_conv3x3_patch_plan", "nncv_hip_conv3x3_stream_plan", "nncv_hip_params_invalidate", "nncv_hip_set_overlap_hint", "nncv_hip_resnet18_create_ex", "nncv_hip_resnet18_passes_in_flight", "nncv_hip_pick_streams",
     "nncv_hip_plan_arena", "nncv_hip_preprocess_u8", "nncv_hip_argmax", "nncv_hip_resnet18_classify_u8",
     "nncv_hip_matmul_f32", "nncv_hip_matmul_time", "nncv_hip_wino43_filter", "nncv_hip_wino43_input", "nncv_hip_wino43_gemm",
     "nncv_hip_wino43_output", "nncv_hip_maxpool3x3s2", "nncv_hip_global_avgpool",
@@ -111,6 +111,10 @@ def lib():
         L.nncv_hip_resnet18_create.restype = vp
         L.nncv_hip_resnet18_clone.argtypes = [vp]
         L.nncv_hip_resnet18_clone.restype = vp
+        L.nncv_hip_resnet18_create_ex.argtypes = [vp, i64, i, i, i]
+        L.nncv_hip_resnet18_create_ex.restype = vp
+        L.nncv_hip_resnet18_passes_in_flight.argtypes = [vp]
+        L.nncv_hip_pick_streams.argtypes = [i, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_int)]
         L.nncv_hip_resnet18_destroy.argtypes = [vp]
         L.nncv_hip_resnet18_destroy.restype = None
         L.nncv_hip_resnet18_forward.argtypes = [vp, vp, i, i, i, vp, vp]

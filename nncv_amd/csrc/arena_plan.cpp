@@ -19,8 +19,17 @@ std::atomic<int>& overlap_state() {
 }
 }  // namespace
 
-int overlap_hint() { return overlap_state().load(std::memory_order_relaxed); }
+namespace {
+thread_local int tl_overlap = 0;  // the value of the handle whose call this thread is serving; 0 = none
+}
+
+int overlap_hint() { return tl_overlap > 0 ? tl_overlap : overlap_state().load(std::memory_order_relaxed); }
+int overlap_default() { return overlap_state().load(std::memory_order_relaxed); }
 void set_overlap_hint(int passes) { overlap_state().store(passes < 1 ? 1 : passes, std::memory_order_relaxed); }
+OverlapScope::OverlapScope(int passes) : prev_(tl_overlap) {
+  if (passes > 0) tl_overlap = passes;
+}
+OverlapScope::~OverlapScope() { tl_overlap = prev_; }
 
 namespace {
 int linger_env() {

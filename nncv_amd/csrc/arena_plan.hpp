@@ -43,7 +43,22 @@ bool arena_linger_forced();
 // lingering) and average pool and FC as two small launches instead of the fused head's 1024 workgroups that each pool
 // their image again.  ResNet-18 at batch 32 with four passes in flight: 0.160 against 0.174 ms per pass; one pass at a
 // time the same choices cost 7 % (0.275 against 0.256).
+// The value belongs to the network handle (nncv_hip_resnet18_create_ex; clones inherit it): while an entry point serves a
+// handle that has one, OverlapScope makes it the answer of overlap_hint() on that thread, so two handles with different
+// values plan, capture and replay side by side.  Handles without a value, the single-layer entry points and the operator-
+// list executor follow the process-wide default (overlap_default).
 int overlap_hint();
+int overlap_default();
 void set_overlap_hint(int passes);
+class OverlapScope {
+ public:
+  explicit OverlapScope(int passes);  // passes <= 0: leaves the thread's current value alone
+  ~OverlapScope();
+  OverlapScope(const OverlapScope&) = delete;
+  OverlapScope& operator=(const OverlapScope&) = delete;
+
+ private:
+  int prev_;
+};
 
 }  // namespace nncv_hip

@@ -40,21 +40,18 @@ void Context::init(int device) {
   (void)noalloc_scratch();  // the scratch array's address on this device, resolved with the device current
 }
 
+// The event is recorded by the call that leaves work pending, on its own (then certainly live) stream; a later call on
+// another stream only waits for the event, so a caller stream destroyed in between is never touched again.
 void Context::order_after_previous(hipStream_t s) {
   if (!tail_pending_ || tail_stream_ == s) return;
-  // the previous caller stream may have been destroyed since: then wait for the whole device instead
-  if (hipEventRecord(tail_event_, tail_stream_) == hipSuccess && hipStreamWaitEvent(s, tail_event_, 0) == hipSuccess) {
-    tail_pending_ = false;
-    return;
-  }
-  (void)hipGetLastError();
-  NNCV_HIP_CHECK(hipDeviceSynchronize());
+  NNCV_HIP_CHECK(hipStreamWaitEvent(s, tail_event_, 0));
   tail_pending_ = false;
 }
 
 void Context::note_stream(hipStream_t s, bool pending) {
   tail_stream_ = s;
   tail_pending_ = pending;
+  if (pending) NNCV_HIP_CHECK(hipEventRecord(tail_event_, s));
 }
 
 }  // namespace nncv_hip
@@ -93,20 +90,39 @@ void guarded_abort(const char* what, const std::function<void()>& fn) {
 // arrives on a different stream than the previous one first makes its stream wait for everything the
 // previous stream was given (an event recorded there now: the mutex is held, so that is exactly the
 // earlier calls' work).  Calls that stay on one stream pay nothing.
+// A caller stream that is being captured into a HIP graph takes neither the wait nor the event: both would reach
+// outside the capture and end it.  The captured launches then run whenever the caller's graph does, and ordering
+// them against other users of the library's shared workspace is the caller's business, as for the graph itself.
+bool stream_is_capturing(hipStream_t s) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &st) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return st == hipStreamCaptureStatusActive;
+}
+
 struct Sync {
   hipStream_t s;
   bool own;
+  bool capturing;
   explicit Sync(void* user) : s(user ? static_cast<hipStream_t>(user) : Context::get().stream()), own(user == nullptr) {
-    Context::get().order_after_previous(s);
+    capturing = !own && stream_is_capturing(s);
+    if (!capturing) Context::get().order_after_previous(s);
   }
   bool done = false;
   void finish() {
     if (own) NNCV_HIP_CHECK(hipStreamSynchronize(s));
-    Context::get().note_stream(s, /*pending=*/!own);
+    if (!capturing) Context::get().note_stream(s, /*pending=*/!own);
     done = true;
   }
   ~Sync() {  // left early by an exception: whatever was enqueued may still be running
-    if (!done) Context::get().note_stream(s, true);
+    if (!done && !capturing) {
+      try {
+        Context::get().note_stream(s, true);
+      } catch (...) {
+      }
+    }
   }
 };
 
@@ -131,26 +147,31 @@ struct HandleSync {
   bool own;
   bool done = false;
   HandleSync(HandleState& hs, void* user) : h(hs), s(user ? static_cast<hipStream_t>(user) : Context::get().stream()), own(user == nullptr) {
+    // the event was recorded when the previous call ended, on its stream: that stream is not touched again here
     if (h.pending && h.tail != s) {
-      if (!h.ev) NNCV_HIP_CHECK(hipEventCreateWithFlags(&h.ev, hipEventDisableTiming));
-      // the previous caller stream may have been destroyed since: then wait for the whole device instead
-      if (!(hipEventRecord(h.ev, h.tail) == hipSuccess && hipStreamWaitEvent(s, h.ev, 0) == hipSuccess)) {
-        (void)hipGetLastError();
-        NNCV_HIP_CHECK(hipDeviceSynchronize());
-      }
+      NNCV_HIP_CHECK(hipStreamWaitEvent(s, h.ev, 0));
       h.pending = false;
+    }
+  }
+  void leave(bool pending) {
+    h.tail = s;
+    h.pending = pending;
+    if (pending) {
+      if (!h.ev) NNCV_HIP_CHECK(hipEventCreateWithFlags(&h.ev, hipEventDisableTiming));
+      NNCV_HIP_CHECK(hipEventRecord(h.ev, s));
     }
   }
   void finish() {
     if (own) NNCV_HIP_CHECK(hipStreamSynchronize(s));
-    h.tail = s;
-    h.pending = !own;
+    leave(!own);
     done = true;
   }
   ~HandleSync() {  // left early by an exception: whatever was enqueued may still be running
     if (!done) {
-      h.tail = s;
-      h.pending = true;
+      try {
+        leave(true);
+      } catch (...) {
+      }
     }
   }
 };
@@ -234,11 +255,31 @@ std::vector<CachedModel>& model_cache() {
 
 void drop_graphs_of(const void* m);
 
-// cheap change detector for a parameter blob that lives at the same address: 4096 strided samples
+// cheap change detector for a parameter blob that lives at the same address: 4096 strided samples.  A caller written
+// against the reference (whose compiled forward re-reads the blob on every call) and rewriting parameters in place
+// between the samples would go unnoticed: NNCV_HIP_PARAMS_HASH=full hashes every byte instead (about 5 ms per call
+// for ResNet-18's 47 MB).
 uint64_t fingerprint(const void* p, long long n, size_t es) {
   NNCV_REQUIRE(p && n > 0, "params: empty memref");
   const unsigned char* b = static_cast<const unsigned char*>(p);
   uint64_t h = 1469598103934665603ull ^ (uint64_t)n;
+  static const bool full = [] {
+    const char* e = getenv("NNCV_HIP_PARAMS_HASH");
+    return e && !strcmp(e, "full");
+  }();
+  if (full) {
+    const size_t bytes = (size_t)n * es, words = bytes / 8;
+    uint64_t h2 = 0x9e3779b97f4a7c15ull;
+    for (size_t i = 0; i + 1 < words; i += 2) {  // two independent chains: the multiplies overlap
+      uint64_t a, c;
+      memcpy(&a, b + i * 8, 8);
+      memcpy(&c, b + i * 8 + 8, 8);
+      h = (h ^ a) * 1099511628211ull;
+      h2 = (h2 ^ c) * 0x100000001b3ull + 0x632be59bd9b4e019ull;
+    }
+    for (size_t k = (words & ~size_t(1)) * 8; k < bytes; ++k) h = (h ^ b[k]) * 1099511628211ull;
+    return h ^ (h2 * 0xff51afd7ed558ccdull);
+  }
   const long long step = std::max<long long>(1, n / 4096);
   for (long long i = 0; i < n; i += step)
     for (size_t k = 0; k < es; ++k) h = (h ^ b[i * es + k]) * 1099511628211ull;
@@ -259,18 +300,14 @@ ResNet18& cached_model(const void* host, long long n, int dt, hipStream_t s) {
   auto& cache = model_cache();
   for (auto& e : cache)
     if (e.host_ptr == host && e.n == n && e.dt == dt) {
-      if (e.fingerprint != fp) {  // same address, new contents: rebuild (captured passes of the old object die with it)
-        drop_graphs_of(e.model.get());
+      if (e.fingerprint != fp) {  // same address, new contents: rebuild
         e.model.reset();
         e.model = build_model(host, n, dt, kAlgoAuto, s);
         e.fingerprint = fp;
       }
       return *e.model;
     }
-  if (cache.size() >= 4) {
-    drop_graphs_of(cache.front().model.get());
-    cache.erase(cache.begin());
-  }
+  if (cache.size() >= 4) cache.erase(cache.begin());
   cache.push_back(CachedModel{host, n, dt, fp, build_model(host, n, dt, kAlgoAuto, s)});
   return *cache.back().model;
 }
@@ -286,7 +323,7 @@ ResNet18& cached_model(const void* host, long long n, int dt, hipStream_t s) {
 // 0.260 ms): NNCV_HIP_GRAPH=size replays only launch-bound passes (up to two / four 224x224 images),
 // NNCV_HIP_GRAPH=0 none.  The pass contains no memset nodes; the event profiler bypasses replay.
 struct GraphEntry {
-  const void* m;  // the ResNet18 or Graph object the launches belong to
+  const void* m;  // the handle (its HandleState) the pass was captured for: clones of one model capture their own
   const void* src;
   const float* logits;
   int N, H, W;
@@ -317,7 +354,7 @@ void drop_graphs_of(const void* m) {
   }
 }
 
-// `run` enqueues the whole pass on `s`; `owner` identifies the model it belongs to.
+// `run` enqueues the whole pass on `s`; `owner` identifies the handle it belongs to.
 void replay(const void* owner, const std::function<void()>& run, const void* src, int N, int H, int W, const float* logits, void* ws,
             hipStream_t s, bool launch_bound) {
   static const int mode = [] {  // -1 by size, 0 never, 1 always (the default)
@@ -360,9 +397,9 @@ void replay(const void* owner, const std::function<void()>& run, const void* src
   NNCV_HIP_CHECK(hipGraphLaunch(hit->exec, s));
 }
 
-void forward_replay(const ResNet18& m, const void* src, int N, int H, int W, float* logits, void* ws, hipStream_t s) {
+void forward_replay(const void* owner, const ResNet18& m, const void* src, int N, int H, int W, float* logits, void* ws, hipStream_t s) {
   // 18 launches: launch-bound up to about two 224x224 images
-  replay(&m, [&] { m.forward(src, N, H, W, logits, ws, s); }, src, N, H, W, logits, ws, s, (long long)N * H * W <= 2ll * 224 * 224);
+  replay(owner, [&] { m.forward(src, N, H, W, logits, ws, s); }, src, N, H, W, logits, ws, s, (long long)N * H * W <= 2ll * 224 * 224);
 }
 
 // ---- the MobileNetV3 object behind the handle-less reference ABI ----------------------------
@@ -403,17 +440,13 @@ Graph& cached_mobilenetv3(const void* host, long long n, int dt, hipStream_t s) 
   for (auto& e : cache)
     if (e.host_ptr == host && e.n == n && e.dt == dt) {
       if (e.fingerprint != fp) {
-        drop_graphs_of(e.graph.get());
         e.graph.reset();
         e.graph = make();
         e.fingerprint = fp;
       }
       return *e.graph;
     }
-  if (cache.size() >= 4) {
-    drop_graphs_of(cache.front().graph.get());
-    cache.erase(cache.begin());
-  }
+  if (cache.size() >= 4) cache.erase(cache.begin());
   cache.push_back(CachedGraph{host, n, dt, fp, make()});
   return *cache.back().graph;
 }
@@ -474,6 +507,7 @@ void forward_abi(nncv_memref2d* dst, nncv_memref4d* src, void* params, int dt) {
 struct nncv_hip_model_impl {
   std::shared_ptr<ResNet18> m;  // shared with the handle's clones
   HandleState st;
+  int passes = 0;  // forward passes the caller keeps in flight next to this handle's; 0 = the process-wide default
 };
 struct nncv_hip_conv_impl {
   std::unique_ptr<ConvLayer> c;
@@ -584,7 +618,7 @@ int nncv_hip_conv3x3_patch_plan(int stride, int N, int OH, int OW, int F, int sl
 int nncv_hip_set_overlap_hint(int passes) {
   return guarded([&] {
     const int want = passes < 1 ? 1 : passes;
-    if (want == overlap_hint()) return;
+    if (want == overlap_default()) return;
     // captured passes hold the launch shapes and workspace offsets of the old setting
     (void)hipDeviceSynchronize();
     auto& gc = graph_cache();
@@ -600,7 +634,6 @@ int nncv_hip_params_invalidate(const void* params) {
     auto& mc = model_cache();
     for (size_t i = 0; i < mc.size();)
       if (!params || mc[i].host_ptr == params) {
-        drop_graphs_of(mc[i].model.get());
         mc.erase(mc.begin() + i);
       } else {
         ++i;
@@ -608,7 +641,6 @@ int nncv_hip_params_invalidate(const void* params) {
     auto& gc = graph_model_cache();
     for (size_t i = 0; i < gc.size();)
       if (!params || gc[i].host_ptr == params) {
-        drop_graphs_of(gc[i].graph.get());
         gc.erase(gc.begin() + i);
       } else {
         ++i;
@@ -638,13 +670,19 @@ const char* nncv_hip_device_arch(void) {
 }
 
 nncv_hip_model* nncv_hip_resnet18_create(const void* params, int64_t n_elems, int dtype, int algo3x3) {
+  return nncv_hip_resnet18_create_ex(params, n_elems, dtype, algo3x3, 0);
+}
+
+nncv_hip_model* nncv_hip_resnet18_create_ex(const void* params, int64_t n_elems, int dtype, int algo3x3, int passes_in_flight) {
   nncv_hip_model* h = nullptr;
   const int rc = guarded([&] {
     NNCV_REQUIRE(params, "null params");
     NNCV_REQUIRE(dtype == kF32 || dtype == kF16, "dtype must be 1 (fp32) or 2 (fp16)");
+    NNCV_REQUIRE(passes_in_flight >= 0 && passes_in_flight <= 64, "passes_in_flight must be 0 (the default) .. 64");
     Context& ctx = Context::get();
     ctx.init(-1);
     h = new nncv_hip_model();
+    h->passes = passes_in_flight;
     try {
       h->m = build_model(params, n_elems, dtype, algo3x3, ctx.stream());
     } catch (...) {
@@ -663,15 +701,30 @@ nncv_hip_model* nncv_hip_resnet18_clone(nncv_hip_model* m) {
     NNCV_REQUIRE(m->m->dtype() == kF16, "clone: fp16 models only (an fp32 model's K-split tickets belong to its layers)");
     h = new nncv_hip_model();
     h->m = m->m;
+    h->passes = m->passes;
   });
   return rc == 0 ? h : nullptr;
+}
+
+int nncv_hip_resnet18_passes_in_flight(const nncv_hip_model* m) { return m ? (m->passes > 0 ? m->passes : overlap_default()) : -1; }
+
+int nncv_hip_pick_streams(int want, void** streams, int* overlapping) {
+  return guarded([&] {
+    NNCV_REQUIRE(streams && want >= 1 && want <= 8, "pick_streams: want must be 1..8 and streams non-null");
+    Context::get().init(-1);
+    int found = 0;
+    const std::vector<hipStream_t> v = pick_streams(want, &found);
+    NNCV_REQUIRE((int)v.size() == want, "pick_streams: fewer streams than asked for");
+    for (int i = 0; i < want; ++i) streams[i] = v[i];
+    if (overlapping) *overlapping = found;
+  });
 }
 
 void nncv_hip_resnet18_destroy(nncv_hip_model* m) {
   if (!m) return;
   guarded([&] {
     (void)hipDeviceSynchronize();
-    drop_graphs_of(m->m.get());
+    drop_graphs_of(&m->st);  // this handle's captured passes only: clones keep theirs
     delete m;
   });
 }
@@ -680,9 +733,10 @@ int nncv_hip_resnet18_forward(nncv_hip_model* m, const void* src, int N, int H, 
   return guarded([&] {
     NNCV_REQUIRE(m && m->m && src && logits, "null argument");
     HandleSync sy(m->st, stream);
+    OverlapScope hint(m->passes);
     const size_t wsb = m->m->workspace_bytes(N, H, W);
-    m->st.arena.reserve(wsb + 1024, sy.s);
-    forward_replay(*m->m, src, N, H, W, logits, m->st.arena.take(wsb), sy.s);
+    if (m->st.arena.reserve(wsb + 1024, sy.s)) drop_graphs_of(&m->st);  // captured against the old workspace
+    forward_replay(&m->st, *m->m, src, N, H, W, logits, m->st.arena.take(wsb), sy.s);
     sy.finish();
   });
 }
@@ -713,6 +767,7 @@ int nncv_hip_resnet18_classify_u8(nncv_hip_model* m, const void* hwc_u8, int N, 
   return guarded([&] {
     NNCV_REQUIRE(m && m->m && hwc_u8 && logits && top1, "null argument");
     HandleSync sy(m->st, stream);
+    OverlapScope hint(m->passes);
     const int dt = m->m->dtype();
     const size_t in_b = align256((size_t)N * 3 * H * W * dtype_size(dt));
     const size_t wsb = m->m->workspace_bytes(N, H, W);
@@ -731,6 +786,7 @@ int nncv_hip_resnet18_forward_tap(nncv_hip_model* m, const void* src, int N, int
     NNCV_REQUIRE(m && m->m && src && logits && tap, "null argument");
     NNCV_REQUIRE(stage >= 0 && stage <= 4, "stage must be 0..4");
     HandleSync sy(m->st, stream);
+    OverlapScope hint(m->passes);
     const size_t wsb = m->m->workspace_bytes(N, H, W);
     m->st.arena.reserve(wsb + 1024, sy.s);
     m->m->forward(src, N, H, W, logits, m->st.arena.take(wsb), sy.s, stage, tap);
@@ -1001,7 +1057,7 @@ void nncv_hip_graph_destroy(nncv_hip_graph* g) {
   if (!g) return;
   guarded([&] {
     (void)hipDeviceSynchronize();
-    drop_graphs_of(g->g.get());
+    drop_graphs_of(&g->st);
     delete g;
   });
 }
@@ -1022,10 +1078,10 @@ int nncv_hip_graph_forward(nncv_hip_graph* g, const void* src, int N, int H, int
     gr.output_shape(H, W, &C, &OH, &OW);
     NNCV_REQUIRE(out_elems == (int64_t)N * C * OH * OW, "graph: out_elems does not match the output shape");
     const size_t wsb = gr.workspace_bytes(N, H, W);
-    g->st.arena.reserve(wsb + 1024, sy.s);
+    if (g->st.arena.reserve(wsb + 1024, sy.s)) drop_graphs_of(&g->st);  // captured against the old workspace
     void* ws = g->st.arena.take(wsb);
     // 49-73 launches: launch-bound up to about four 224x224 images
-    replay(&gr, [&] { gr.forward(src, N, H, W, out, ws, sy.s); }, src, N, H, W, out, ws, sy.s, (long long)N * H * W <= 4ll * 224 * 224);
+    replay(&g->st, [&] { gr.forward(src, N, H, W, out, ws, sy.s); }, src, N, H, W, out, ws, sy.s, (long long)N * H * W <= 4ll * 224 * 224);
     sy.finish();
   });
 }

@@ -64,12 +64,16 @@ class PinnedBuffer {
 // grows the backing store if the plan does not fit; pointers are handed out 256-byte aligned.
 class Arena {
  public:
-  void reserve(size_t bytes, hipStream_t s) {
+  // true when the backing store was replaced (pointers handed out before are gone)
+  bool reserve(size_t bytes, hipStream_t s) {
+    bool grown = false;
     if (bytes > buf_.bytes()) {
       NNCV_HIP_CHECK(hipStreamSynchronize(s));  // nobody may still be using the old block
       buf_.reset(bytes + bytes / 8);
+      grown = true;
     }
     off_ = 0;
+    return grown;
   }
   void* take(size_t bytes) {
     const size_t a = (off_ + 255) & ~size_t(255);
@@ -93,6 +97,9 @@ constexpr size_t kNoAllocWorkspaceBytes = size_t(4) << 20;
 constexpr size_t kNoAllocScratchBytes = kNoAllocCounterBytes + kNoAllocWorkspaceBytes;
 void* noalloc_scratch();
 void launch_clear_words(void* p, int n_words, hipStream_t s);
+
+// stream_probe.hip: up to `want` library-owned streams, the first *found of which were measured to overlap pairwise
+std::vector<hipStream_t> pick_streams(int want, int* found);
 
 // Process-wide state.  All public entry points serialise on `mu`.
 class Context {

@@ -103,10 +103,13 @@ class Conv:
 class Model:
     """nncv_hip_resnet18_* handle."""
 
-    def __init__(self, blob, dt, algo=abi.ALGO_AUTO):
+    def __init__(self, blob, dt, algo=abi.ALGO_AUTO, passes=0):
         blob = np.ascontiguousarray(blob, abi.np_dtype(dt))
         self.dt = dt
-        self.h = abi.lib().nncv_hip_resnet18_create(blob.ctypes.data, blob.size, dt, algo)
+        if passes:  # the handle plans for that many passes in flight (nncv_hip_resnet18_create_ex)
+            self.h = abi.lib().nncv_hip_resnet18_create_ex(blob.ctypes.data, blob.size, dt, algo, passes)
+        else:
+            self.h = abi.lib().nncv_hip_resnet18_create(blob.ctypes.data, blob.size, dt, algo)
         if not self.h:
             raise abi.NncvHipError(abi.lib().nncv_hip_last_error().decode())
 

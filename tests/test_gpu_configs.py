@@ -66,3 +66,45 @@ def test_resnet18_fp16_batch32_full_size():
     perm = np.random.default_rng(7).permutation(32)
     got_p = host(m(dev(x[perm], abi.F16)))
     assert np.array_equal(got_p, got[perm])
+
+
+def _tags_and_logits(m, xd):
+    """One eager pass under the event profiler: the logits and how often each kernel instance was launched."""
+    host(m(xd))
+    abi.profile_enable(True)
+    try:
+        abi.profile_report()
+        got = host(m(xd))
+        rep = abi.profile_report()
+    finally:
+        abi.profile_enable(False)
+    return got, {k: v["launches"] for k, v in rep.items()}
+
+
+@pytest.mark.parametrize("passes", [1, 4])
+def test_resnet18_fp16_every_image_of_the_batch_against_the_oracle(passes):
+    """BASELINE config 4, all 32 images (examples/Res18/main.cpp:103-111 takes the top-1 of every image): every row of the
+    logits within the fp16 bar of the CPU oracle (its OpenMP x AVX2 convolution, itself checked against the scalar one)
+    and the same top-1 on every image -- with the launch shapes of one pass at a time, and with the shapes a handle
+    planned for four passes in flight takes (the ones the benchmark's headline runs), asserted from the launch tags.
+    The same for batch 1."""
+    hb = synth.round_fp16(synth.resnet18_params())
+    x = synth.round_fp16(synth.cfg4_input(32))
+    want = oracle.hwp_resnet18_forward(x, hb)
+    m = Model(hb, abi.F16, abi.ALGO_AUTO, passes=passes)
+    got, rep = _tags_and_logits(m, dev(x, abi.F16))
+    print("passes", passes, rep, flush=True)
+    count = lambda prefix: sum(v for k, v in rep.items() if k.startswith(prefix))
+    if passes == 4:
+        assert rep.get("conv3x3_stream<f16,1x4x1>", 0) == 6 and count("conv3x3_stream") == 6 and count("conv3x3_patch") == 7
+        assert "avgpool_fc" not in rep and rep.get("global_avgpool", 0) == 1
+    else:
+        assert rep.get("conv3x3_stream<f16,1x2x2>", 0) == 10 and count("conv3x3_patch") == 3 and rep.get("avgpool_fc", 0) == 1
+    assert count("conv3x3s2_patch") == 3 and rep.get("stem_conv7x7_bn_relu_maxpool<f16>", 0) == 1
+    errs = [rel_l2(got[i], want[i]) for i in range(32)]
+    print("worst image rel_l2 %.2e" % max(errs), flush=True)
+    assert max(errs) < FP16_REL_L2
+    assert np.array_equal(got.argmax(1), want.argmax(1))
+    one, rep1 = _tags_and_logits(m, dev(x[7:8], abi.F16))
+    assert rel_l2(one, want[7:8]) < FP16_REL_L2 and one.argmax(1) == want[7:8].argmax(1)
+    m.close()

@@ -229,6 +229,99 @@ def test_overlap_hint_changes_the_launch_shapes_not_the_results(blob):
         abi.check(L.nncv_hip_set_overlap_hint(1))
 
 
+def test_handles_with_different_passes_in_flight_work_side_by_side(blob):
+    """nncv_hip_resnet18_create_ex: the number of passes in flight belongs to the handle.  One handle planned for four
+    passes and one planned for one pass, alive together in one process, each launch the shapes of its own setting (also
+    when their calls alternate and replay captured graphs), a clone inherits the value, the process-wide default stays
+    what it was, and both agree with the oracle."""
+    import torch
+    import oracle
+    from gpu_util import Model, dev, host, rel_l2, FP16_REL_L2
+    L = abi.lib()
+    hb = synth.round_fp16(blob)
+    N = 16
+    x = synth.round_fp16(synth.uniform(9800, (N, 3, 224, 224), 0.0, 1.0))
+    xd = dev(x, abi.F16)
+    wide = Model(hb, abi.F16, abi.ALGO_AUTO, passes=4)
+    plain = Model(hb, abi.F16, abi.ALGO_AUTO, passes=1)
+    twin = wide.clone()
+    assert L.nncv_hip_resnet18_passes_in_flight(wide.h) == 4 and L.nncv_hip_resnet18_passes_in_flight(twin.h) == 4
+    assert L.nncv_hip_resnet18_passes_in_flight(plain.h) == 1
+
+    def tags(m):
+        abi.profile_enable(True)
+        try:
+            abi.profile_report()
+            got = host(m(xd))
+            rep = abi.profile_report()
+        finally:
+            abi.profile_enable(False)
+        return got, {k: v["launches"] for k, v in rep.items()}
+
+    count = lambda r, prefix: sum(v for k, v in r.items() if k.startswith(prefix))
+    for _ in range(2):  # alternating: neither handle's setting leaks into the other's plans
+        got_w, rep_w = tags(wide)
+        got_p, rep_p = tags(plain)
+        assert rep_w.get("conv3x3_stream<f16,1x4x1>", 0) == 6 and "avgpool_fc" not in rep_w, rep_w
+        assert count(rep_p, "conv3x3_stream") == 10 and rep_p.get("avgpool_fc", 0) == 1, rep_p
+    got_t, rep_t = tags(twin)
+    assert rep_t == rep_w and np.array_equal(got_t, got_w)
+    want = oracle.hwp_resnet18_forward(x, hb)
+    for got in (got_w, got_p):
+        assert rel_l2(got, want) < FP16_REL_L2 and (got.argmax(1) == want.argmax(1)).all()
+    # replayed graphs (third call on): each handle keeps reproducing its own bits while the calls alternate
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    ow = torch.zeros((N, 1000), dtype=torch.float32, device="cuda")
+    op = torch.zeros((N, 1000), dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    for _ in range(5):
+        abi.check(L.nncv_hip_resnet18_forward(wide.h, xd.data_ptr(), N, 224, 224, ow.data_ptr(), s1.cuda_stream))
+        abi.check(L.nncv_hip_resnet18_forward(plain.h, xd.data_ptr(), N, 224, 224, op.data_ptr(), s2.cuda_stream))
+    torch.cuda.synchronize()
+    assert np.array_equal(ow.cpu().numpy(), got_w) and np.array_equal(op.cpu().numpy(), got_p)
+    # destroying one handle leaves the other's captured passes alone
+    wide.close()
+    abi.check(L.nncv_hip_resnet18_forward(plain.h, xd.data_ptr(), N, 224, 224, op.data_ptr(), s2.cuda_stream))
+    abi.check(L.nncv_hip_resnet18_forward(twin.h, xd.data_ptr(), N, 224, 224, ow.data_ptr(), s1.cuda_stream))
+    torch.cuda.synchronize()
+    assert np.array_equal(ow.cpu().numpy(), got_w) and np.array_equal(op.cpu().numpy(), got_p)
+    plain.close()
+    twin.close()
+
+
+def test_pick_streams_returns_usable_streams(blob):
+    """nncv_hip_pick_streams: four library-owned streams, at least one of them counted as overlapping, the same list on a
+    second call, and passes enqueued on them give the bits of passes run alone."""
+    import ctypes
+    import torch
+    from gpu_util import Model, dev, host
+    L = abi.lib()
+    st = (ctypes.c_void_p * 4)()
+    found = ctypes.c_int(0)
+    abi.check(L.nncv_hip_pick_streams(4, st, ctypes.byref(found)))
+    print("overlapping streams:", found.value, flush=True)
+    assert 1 <= found.value <= 4 and all(st[i] for i in range(4)) and len({st[i] for i in range(4)}) == 4
+    st2 = (ctypes.c_void_p * 4)()
+    abi.check(L.nncv_hip_pick_streams(4, st2, None))
+    assert [st2[i] for i in range(4)] == [st[i] for i in range(4)]
+    assert L.nncv_hip_pick_streams(9, st, None) != 0
+    hb = synth.round_fp16(blob)
+    ms = [Model(hb, abi.F16, abi.ALGO_AUTO, passes=4)]
+    ms += [ms[0].clone() for _ in range(3)]
+    xs = [dev(synth.round_fp16(synth.uniform(9900 + i, (4, 3, 64, 64), 0.0, 1.0)), abi.F16) for i in range(4)]
+    wants = [host(ms[i](xs[i])) for i in range(4)]
+    outs = [torch.zeros((4, 1000), dtype=torch.float32, device="cuda") for _ in range(4)]
+    torch.cuda.synchronize()
+    for _ in range(4):
+        for i in range(4):
+            abi.check(L.nncv_hip_resnet18_forward(ms[i].h, xs[i].data_ptr(), 4, 64, 64, outs[i].data_ptr(), st[i]))
+    torch.cuda.synchronize()
+    for i in range(4):
+        assert np.array_equal(outs[i].cpu().numpy(), wants[i]), i
+    for m in ms:
+        m.close()
+
+
 def test_clones_share_the_weights_and_outlive_the_first_handle(blob):
     """nncv_hip_resnet18_clone: the clone gives the bits of the model it was made from, keeps working after that model's
     handle is destroyed (the weights live until the last handle goes), and is refused for fp32 models, whose K-split

@@ -75,3 +75,46 @@ def test_noalloc_refuses_what_the_scratch_cannot_hold():
     got, want = run_pair(layer, abi.F32, 1, 8, 8, 9500)
     assert max_rel(got, want) < FP32_MAX_REL
     layer.close()
+
+
+@pytest.mark.parametrize("dt", [abi.F32, abi.F16])
+def test_noalloc_under_graph_capture(dt):
+    """Two calls of the entry point recorded into one HIP graph on a capturing stream (kernel nodes only: the tickets are
+    cleared by a fill kernel, the library neither waits for nor records events on a capturing stream), replayed three
+    times with eager work and synchronisations in between; every replay gives the bits of nncv_hip_conv_forward."""
+    C = F = 512
+    w = synth.normal(9600, (F, C, 3, 3), std=float(np.sqrt(2.0 / (C * 9))))
+    if dt == abi.F16:
+        w = synth.round_fp16(w)
+    layer = Conv(dt, w, 1, 1, relu=True, algo=abi.ALGO_IGEMM)
+    shapes = ((1, 8, 8, 9700), (1, 4, 4, 9800))
+    xs, wants, outs = [], [], []
+    for (N, H, W, seed) in shapes:
+        x = synth.normal(seed, (N, H, W, C))
+        if dt == abi.F16:
+            x = synth.round_fp16(x)
+        xd = dev(x, dt)
+        xs.append(xd)
+        wants.append(host(layer(xd, abi.NHWC)))
+        out = empty((N, H, W, F), dt)
+        # once eagerly: one-time kernel attribute set-up must not fall into the capture
+        abi.check(abi.lib().nncv_hip_conv_forward_noalloc(layer.h, xd.data_ptr(), N, H, W, None, out.data_ptr(), None))
+        outs.append(out)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.graph(g, stream=side):
+        s = torch.cuda.current_stream().cuda_stream
+        for (N, H, W, _), xd, out in zip(shapes, xs, outs):
+            abi.check(abi.lib().nncv_hip_conv_forward_noalloc(layer.h, xd.data_ptr(), N, H, W, None, out.data_ptr(), s))
+    for rep in range(3):
+        for out in outs:
+            out.fill_(float(rep + 3))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for out, want in zip(outs, wants):
+            assert np.array_equal(host(out), want), ("replay", rep)
+        # the library's own eager work between replays
+        assert np.array_equal(host(layer(xs[0], abi.NHWC)), wants[0])
+    layer.close()

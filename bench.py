@@ -44,49 +44,26 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 # Hardware queues of this process (the HIP runtime's own setting, read when it initialises; default 4).  Streams that
 # share a queue run their work one after the other; where the environment does not fix the number, eight queues make that
-# rarer.  Which streams actually overlap is measured below (concurrent_streams), whatever the number is.
+# rarer.  Which streams actually overlap is measured by the library (nncv_hip_pick_streams), whatever the number is.
 os.environ.setdefault("GPU_MAX_HW_QUEUES", "8")
 IN_FLIGHT_CANDIDATES = (2, 3, 4)
 
 
-def concurrent_streams(torch, run_pass, want, candidates=8):
-    """`want` streams from torch's pool whose work overlaps, and what the probe found.
+def library_streams(L, want):
+    """`want` HIP streams from the library (nncv_hip_pick_streams), and what its probe found.
 
     Two streams overlap only when the runtime gave them different hardware queues AND those queues sit on different
-    pipes of the command processor (four pipes; queue q of a process is served by pipe q mod 4): passes on two streams
-    that share a queue run one after the other, on two queues of one pipe they gain 14 %.  Which queue a stream gets
-    depends on every stream the process created before it, so the streams are chosen by measurement: run_pass(h, s)
-    enqueues one short pass of handle h on stream s; a candidate is taken when a pass on it next to a pass on each
-    stream already taken costs less than 1.5 passes."""
-    objs = [torch.cuda.Stream() for _ in range(candidates)]
+    pipes of the command processor (four pipes; queue q of a process is served by pipe q mod 4): work on two streams
+    that share a queue runs one after the other, on two queues of one pipe it gains 14 %.  Which queue a stream gets
+    depends on every stream the process created before it, so the library chooses its streams by measurement (chains
+    of short kernels on eight candidates, pairwise) and hands out the ones that overlap first."""
+    import ctypes
+    st = (ctypes.c_void_p * want)()
+    found = ctypes.c_int(0)
+    if L.nncv_hip_pick_streams(want, st, ctypes.byref(found)) != 0:
+        raise RuntimeError(L.nncv_hip_last_error().decode())
+    return [st[i] for i in range(want)], {"candidates": 8, "overlapping": int(found.value), "by": "nncv_hip_pick_streams"}
 
-    def ms(a, b, n):
-        for _ in range(n):
-            run_pass(0, a.cuda_stream)
-            if b is not None:
-                run_pass(1, b.cuda_stream)
-        torch.cuda.synchronize()
-
-    t_w = time.perf_counter()
-    while (time.perf_counter() - t_w) * 1e3 < CLOCK_WARMUP_MS:
-        ms(objs[0], None, 20)
-
-    def cost(a, b):
-        ms(a, b, 5)
-        t0 = time.perf_counter()
-        ms(a, b, 30)
-        return (time.perf_counter() - t0) / 30
-
-    alone = cost(objs[0], None)
-    taken = [objs[0]]
-    for c in objs[1:]:
-        if len(taken) >= want:
-            break
-        if all(cost(m, c) < 1.5 * alone for m in taken):
-            taken.append(c)
-    found = len(taken)
-    taken += [c for c in objs if c not in taken][:max(0, want - found)]
-    return taken, {"candidates": candidates, "overlapping": found}
 
 MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 matrix peak
 MFMA_F32_PEAK_TFLOPS = 157.3    # MI355X fp32 matrix peak
@@ -109,6 +86,10 @@ DOMINANT_TRAFFIC = {  # profiles/resnet18_fp16_bs32_hbm_counters.txt, launches w
     "conv3x3_patch<f16,4,1>": (13341 + 12544) * 1024,
     "conv3x3_patch<f16,1,4>": (17301 + 1568) * 1024,
 }
+
+
+# the same for the launch plan of three or more passes in flight
+IN_FLIGHT_TRAFFIC = {}  # filled from profiles/resnet18_fp16_bs32_in_flight_plan_hbm_counters.txt
 
 
 def main():
@@ -187,36 +168,52 @@ def main():
     # Passes in flight: handle i and stream i serve steps i, i + K, i + 2K ...  A handle owns its workspace, so passes of
     # different handles overlap on the GPU (one pass's launch gaps, prologues and tails fill with the other's work); every
     # pass is still a whole forward over one batch of N images, into its own logits buffer.
+    # The number of passes in flight is a property of the handles (nncv_hip_resnet18_create_ex; clones inherit it): the
+    # library plans their launches for it.  One set of handles per value tried, each set one model and its clones.
     asked1 = 1 if args.no_batch1 else args.in_flight_batch1
     KMAX = max(args.in_flight, asked1, max(IN_FLIGHT_CANDIDATES) if 0 in (args.in_flight, asked1) else 1)
-    models, outs = [model], [logits]
-    for _ in range(1, KMAX):
-        h = L.nncv_hip_resnet18_clone(model)  # its own workspace on the same device weights
-        if not h:
-            raise RuntimeError(L.nncv_hip_last_error().decode())
-        models.append(h)
-        outs.append(torch.empty((N, 1000), dtype=torch.float32, device="cuda"))
+    outs = [logits] + [torch.empty((N, 1000), dtype=torch.float32, device="cuda") for _ in range(1, KMAX)]
+    handle_sets = {1: [model]}
+    all_handles = [model]
 
-    x1 = xd[:1].contiguous()
+    def handles_for(k_in_flight):
+        passes = 1 if args.no_overlap_hint else k_in_flight
+        hs = handle_sets.get(passes)
+        if hs is None:
+            first = L.nncv_hip_resnet18_create_ex(blob.ctypes.data, blob.size, abi.F16, algo, passes)
+            if not first:
+                raise RuntimeError(L.nncv_hip_last_error().decode())
+            hs = handle_sets[passes] = [first]
+            all_handles.append(first)
+        while len(hs) < k_in_flight:
+            h = L.nncv_hip_resnet18_clone(hs[0])  # its own workspace on the same device weights
+            if not h:
+                raise RuntimeError(L.nncv_hip_last_error().decode())
+            hs.append(h)
+            all_handles.append(h)
+        return hs
+
+    # every handle reads its own copy of the input (passes in flight must not share one cached tensor)
+    xds = [xd] + [xd.clone() for _ in range(1, KMAX)]
+    x1s = [t[:1].contiguous() for t in xds]
+    x1 = x1s[0]
     l1 = [torch.empty((1, 1000), dtype=torch.float32, device="cuda") for _ in range(KMAX)]
-    pool_objs, stream_probe = [], None  # the stream objects stay alive to the end of main
+    pool_streams, stream_probe = [], None
     if KMAX > 1:
-        pool_objs, stream_probe = concurrent_streams(
-            torch, lambda h, s: abi.check(L.nncv_hip_resnet18_forward(models[h], x1.data_ptr(), 1, H, H, l1[h].data_ptr(), s)), KMAX)
-    pool_streams = [t.cuda_stream for t in pool_objs]
+        pool_streams, stream_probe = library_streams(L, KMAX)
 
     def step(xt, out, n):
         abi.check(L.nncv_hip_resnet18_forward(model, xt.data_ptr(), n, H, H, out.data_ptr(), stream))
 
-    def timed(xt, out_list, n, warmup, steps, k_in_flight):
+    def timed(xts, out_list, n, warmup, steps, k_in_flight):
+        hs = handles_for(k_in_flight)
+
         def go(i):
             j = i % k_in_flight
-            # with several passes in flight every handle gets a stream of its own from torch's pool; one pass at a time
-            # stays on the default stream, like every other measurement of this script
+            # with several passes in flight every handle gets a stream of its own, measured to overlap with the others
+            # (nncv_hip_pick_streams); one pass at a time stays on the default stream, like every other measurement here
             sj = stream if k_in_flight == 1 else pool_streams[j]
-            abi.check(L.nncv_hip_resnet18_forward(models[j], xt.data_ptr(), n, H, H, out_list[j].data_ptr(), sj))
-        # the library plans its launches for the number of passes the caller keeps in flight
-        abi.check(L.nncv_hip_set_overlap_hint(1 if args.no_overlap_hint else k_in_flight))
+            abi.check(L.nncv_hip_resnet18_forward(hs[j], xts[j].data_ptr(), n, H, H, out_list[j].data_ptr(), sj))
         # clock warm-up: untimed steps until CLOCK_WARMUP_MS of wall time have passed, then the W asked for
         t_w = time.perf_counter()
         while (time.perf_counter() - t_w) * 1e3 < CLOCK_WARMUP_MS:
@@ -231,26 +228,25 @@ def main():
             go(i)
         torch.cuda.synchronize()  # every stream
         dt = time.perf_counter() - t0
-        abi.check(L.nncv_hip_set_overlap_hint(1))
         return dt / steps
 
-    def pick_in_flight(asked, xt, out_list, n):
+    def pick_in_flight(asked, xts, out_list, n):
         """(passes in flight, {candidate: ms per pass in the trial})"""
         if asked > 0:
             return asked, None
-        trial = {k: timed(xt, out_list, n, 20, max(30, args.steps // 2), k) for k in IN_FLIGHT_CANDIDATES}
+        trial = {k: timed(xts, out_list, n, 20, max(30, args.steps // 2), k) for k in IN_FLIGHT_CANDIDATES}
         return min(trial, key=trial.get), {str(k): round(v * 1e3, 4) for k, v in trial.items()}
 
-    K, k_trial = pick_in_flight(args.in_flight, xd, outs, N)
-    sec = timed(xd, outs, N, args.warmup, args.steps, K)
-    sec_serial = sec if K == 1 else timed(xd, outs, N, args.warmup, args.steps, 1)
+    K, k_trial = pick_in_flight(args.in_flight, xds, outs, N)
+    sec = timed(xds, outs, N, args.warmup, args.steps, K)
+    sec_serial = sec if K == 1 else timed(xds, outs, N, args.warmup, args.steps, 1)
     ips = N / sec
     flops_step = spec.flops_per_image(H) * N
 
     # batch 1 (the other half of the headline metric)
-    K1, k1_trial = (1, None) if args.no_batch1 else pick_in_flight(args.in_flight_batch1, x1, l1, 1)
-    sec1 = None if args.no_batch1 else timed(x1, l1, 1, args.warmup, max(args.steps, 50), K1)
-    sec1_serial = None if args.no_batch1 else (sec1 if K1 == 1 else timed(x1, l1, 1, args.warmup, max(args.steps, 50), 1))
+    K1, k1_trial = (1, None) if args.no_batch1 else pick_in_flight(args.in_flight_batch1, x1s, l1, 1)
+    sec1 = None if args.no_batch1 else timed(x1s, l1, 1, args.warmup, max(args.steps, 50), K1)
+    sec1_serial = None if args.no_batch1 else (sec1 if K1 == 1 else timed(x1s, l1, 1, args.warmup, max(args.steps, 50), 1))
 
     # event-timed per-kernel pass (separate from the timed region above: the events serialise launches)
     abi.profile_enable(True)
@@ -313,6 +309,17 @@ def main():
         roofline.update({"achieved": round(achieved, 3), "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 5),
                          "avg_launch_us": round(d["ms"] / d["launches"] * 1e3, 3), "launches": d["launches"],
                          "timing": "one HIP event pair per launch (includes ~4 us of event latency)"})
+    # The same leg for what `value` runs: with three or more passes in flight the handles launch the 128-filter form of the
+    # stream kernel on layer2 / layer3 (six launches per pass: the instance with the most time in that mode).  Its layer
+    # alone, planned for K passes in flight (single layers plan with the process-wide default), back to back as above.
+    roofline_in_flight = None
+    if K >= 3 and not args.no_overlap_hint and N == 32:
+        roofline_in_flight = layer_roofline(L, stream, N, 128, 128, 28, K)
+        roofline_in_flight["traffic"] = IN_FLIGHT_TRAFFIC.get(roofline_in_flight["kernel"])
+        roofline_in_flight["launches_per_step"] = 6
+        roofline_in_flight["note"] = ("the dominant kernel instance of the launch plan `value` runs (passes_in_flight >= 3), timed "
+                                      "alone; in the timed region its launches share the chip with those of the other passes "
+                                      "and have no duration of their own")
     roofline["launch_shapes"] = ("those of one pass at a time (overlap hint 1), which the summaries under profiles/ hold; with "
                                  "three or more passes in flight layer2 / layer3 run the same kernel's 128-filter form and "
                                  "layer1 the patch kernel (see config.passes_in_flight), where a launch of one pass has no "
@@ -328,8 +335,10 @@ def main():
                    "batch": N, "image": H, "algo3x3": args.algo, "input_resident_in_hbm": True,
                    "passes_in_flight": K, "passes_in_flight_trial_ms": k_trial, "stream_probe": stream_probe,
                    "passes_in_flight_note": "step k runs on model handle and HIP stream k mod %d, each handle with its own "
-                                            "workspace and logits buffer; every step is one whole forward pass over one batch "
-                                            "of %d images; `one_pass_at_a_time` is the same loop on one handle and one stream" % (K, N)},
+                                            "workspace, input copy and logits buffer; every step is one whole forward pass over "
+                                            "one batch of %d images; ms_per_step is elapsed time / steps, i.e. the reciprocal "
+                                            "of the pass rate, not the latency of a pass; `one_pass_at_a_time` is the same loop "
+                                            "on one handle and one stream, where the two coincide" % (K, N)},
         "tflops_effective": round(flops_step / sec / 1e12, 3),
         "frac_of_fp16_mfma_peak": round(flops_step / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 5),
         "conv3x3s1_gflop_per_step": round(conv3x3_flops / 1e9, 2),
@@ -341,6 +350,7 @@ def main():
                                                                     "ms_per_image": round(sec1_serial * 1e3, 4)}},
         "model_create_ms": round(t_create * 1e3, 2),
         "roofline": roofline,
+        "roofline_in_flight": roofline_in_flight,
         "kernels": kernels,
         "device": L.nncv_hip_device_arch().decode(),
     }
@@ -357,9 +367,46 @@ def main():
         torch.cuda.synchronize()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(blob32, x)
-    for h in models:
+    for h in all_handles:
         L.nncv_hip_resnet18_destroy(h)
     print(json.dumps(out))
+
+
+def layer_roofline(L, stream, N, C, F, HW, passes, reps=200):
+    """One fp16 3x3 stride-1 layer [N,HW,HW,C] -> F with BN + ReLU alone, planned for `passes` passes in flight: `reps`
+    launches back to back between one HIP event pair on the launch stream, after a clock warm-up of the same launches."""
+    import ctypes
+    import numpy as np
+    import torch
+    from nncv_amd import abi, synth
+    w = synth.normal(77, (F, C, 3, 3), std=float(np.sqrt(2.0 / (C * 9)))).astype(np.float16)
+    bn = [synth.uniform(78 + i, (F,), 0.5, 1.5).astype(np.float16) for i in range(4)]
+    conv = L.nncv_hip_conv_create(abi.F16, w.ctypes.data, F, C, 3, 3, 1, 1, *[b.ctypes.data for b in bn], 1, abi.ALGO_IGEMM)
+    if not conv:
+        raise RuntimeError(L.nncv_hip_last_error().decode())
+    xin = torch.randn((N, HW, HW, C), device="cuda", dtype=torch.float16)
+    yout = torch.empty((N, HW, HW, F), device="cuda", dtype=torch.float16)
+    avg = ctypes.c_float(0.0)
+    abi.check(L.nncv_hip_set_overlap_hint(passes))
+    try:
+        abi.profile_enable(True)
+        abi.profile_report()
+        abi.check(L.nncv_hip_conv_forward(conv, xin.data_ptr(), N, HW, HW, abi.NHWC, None, yout.data_ptr(), stream))
+        tags = list(abi.profile_report())
+        abi.profile_enable(False)
+        abi.check(L.nncv_hip_conv_time(conv, xin.data_ptr(), N, HW, HW, None, yout.data_ptr(), 4000, stream, ctypes.byref(avg)))  # clocks
+        abi.check(L.nncv_hip_conv_time(conv, xin.data_ptr(), N, HW, HW, None, yout.data_ptr(), reps, stream, ctypes.byref(avg)))
+    finally:
+        abi.profile_enable(False)
+        abi.check(L.nncv_hip_set_overlap_hint(1))
+        L.nncv_hip_conv_destroy(conv)
+    us = float(avg.value)
+    flops = 2.0 * N * HW * HW * F * C * 9
+    achieved = flops / (us * 1e-6) / 1e12
+    return {"kernel": tags[0] if tags else None, "bound": "mfma", "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "achieved": round(achieved, 3), "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 5), "avg_launch_us": round(us, 3),
+            "launches": reps, "flops_per_launch": flops, "planned_for_passes_in_flight": passes,
+            "timing": "layer [%d,%d,%d,%d]->%d alone, %d back-to-back launches between one HIP event pair" % (N, HW, HW, C, F, reps)}
 
 
 def host_abi(blob16, x16, calls=60):
@@ -566,11 +613,9 @@ def bench_graph(args, L):
     stream = torch.cuda.current_stream().cuda_stream
     x1 = xd[:1].contiguous()
     r1 = [torch.empty((1, per_image), dtype=torch.float32, device="cuda") for _ in range(KMAX)]
-    pool_objs, stream_probe = [], None
+    pool_streams, stream_probe = [], None
     if KMAX > 1:
-        pool_objs, stream_probe = concurrent_streams(
-            torch, lambda h, s: abi.check(L.nncv_hip_graph_forward(gs[h], x1.data_ptr(), 1, H, H, r1[h].data_ptr(), per_image, s)), KMAX)
-    pool_streams = [t.cuda_stream for t in pool_objs]
+        pool_streams, stream_probe = library_streams(L, KMAX)
 
     def step(xt, out, n):
         abi.check(L.nncv_hip_graph_forward(g, xt.data_ptr(), n, H, H, out.data_ptr(), n * per_image, stream))
@@ -580,7 +625,7 @@ def bench_graph(args, L):
             j = i % k_in_flight
             sj = stream if k_in_flight == 1 else pool_streams[j]  # see main: pool streams when passes overlap
             abi.check(L.nncv_hip_graph_forward(gs[j], xt.data_ptr(), n, H, H, out_list[j].data_ptr(), n * per_image, sj))
-        # the library plans its launches for the number of passes the caller keeps in flight
+        # the operator-list executor plans with the process-wide default of passes in flight
         abi.check(L.nncv_hip_set_overlap_hint(1 if args.no_overlap_hint else k_in_flight))
         # clock warm-up: untimed steps until CLOCK_WARMUP_MS of wall time have passed, then the W asked for
         t_w = time.perf_counter()

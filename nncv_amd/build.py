@@ -17,7 +17,7 @@ RT_LIB = os.path.join(HERE, "lib", "libnncv_rt.so")
 DRIVER = os.path.join(HERE, "lib", "res18_main")
 
 DEVICE_SOURCES = ["igemm.hip", "igemm_fast.hip", "conv3x3_patch.hip", "conv3x3_f16.hip", "conv_pairs.hip", "stem_pool.hip", "gemm_nn.hip", "winograd.hip", "pool_layout.hip", "elementwise.hip", "noalloc.hip", "stream_probe.hip"]
-HOST_SOURCES = ["model.cpp", "capi.cpp", "datatype.cpp", "profiler.cpp", "arena_plan.cpp", "graph.cpp"]
+HOST_SOURCES = ["model.cpp", "capi.cpp", "datatype.cpp", "profiler.cpp", "arena_plan.cpp", "graph.cpp", "hostcopy.cpp"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-Wall", "-Wno-unused-function"]

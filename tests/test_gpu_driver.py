@@ -111,6 +111,53 @@ def test_forward_from_two_threads_at_once(blob):
             assert np.array_equal(r.view(np.uint32), serial[k].view(np.uint32))
 
 
+def test_host_abi_on_a_large_batch_stages_its_upload(blob):
+    """_mlir_ciface_forward_f16 on 16 host images (examples/Res18/main.cpp:95-99 with a batch): the input goes to pinned
+    staging memory in pieces copied by several host threads, or straight from the caller's buffer when that is pinned.
+    Either way the logits are the bits of the device entry point on the same batch, on every one of five calls; they meet
+    the fp16 bar and the oracle's top-1 on every image; and a second thread calling with another batch at the same time
+    changes nothing."""
+    import torch
+    from gpu_util import Model, dev, host, rel_l2, FP16_REL_L2
+    hb = synth.round_fp16(blob)
+    b16 = hb.astype(np.float16)
+    x = synth.round_fp16(synth.uniform(9250, (16, 3, 224, 224), 0.0, 1.0))
+    x16 = x.astype(np.float16)
+    calls = [abi.forward(x16, b16).astype(np.float32) for _ in range(5)]
+    for c in calls[1:]:
+        assert np.array_equal(c, calls[0])
+    m = Model(hb, abi.F16, abi.ALGO_AUTO)
+    alone = host(m(dev(x, abi.F16))).astype(np.float16).astype(np.float32)
+    assert np.array_equal(calls[0], alone)
+    m.close()
+    want = oracle.hwp_resnet18_forward(x, hb)
+    assert rel_l2(calls[0], want) < FP16_REL_L2 and np.array_equal(calls[0].argmax(1), want.argmax(1))
+    pinned = torch.from_numpy(x16).pin_memory()
+    assert np.array_equal(abi.forward(pinned.numpy(), b16).astype(np.float32), calls[0])
+    other = synth.round_fp16(synth.uniform(9251, (20, 3, 96, 96), 0.0, 1.0)).astype(np.float16)
+    other_alone = abi.forward(other, b16)
+    results, errors = [[], []], []
+
+    def work(k, arr):
+        try:
+            for _ in range(4):
+                results[k].append(abi.forward(arr, b16))
+        except Exception as e:  # noqa: BLE001 - reported below
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(0, x16)), threading.Thread(target=work, args=(1, other))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(100)
+        assert not t.is_alive()
+    assert not errors, errors
+    for r in results[0]:
+        assert np.array_equal(r.astype(np.float32), calls[0])
+    for r in results[1]:
+        assert np.array_equal(r, other_alone)
+
+
 def test_device_calls_on_two_streams_do_not_overlap_in_the_shared_workspace(blob):
     """The device entry point on two caller streams alternately, without synchronising in between: the
     library orders the second stream behind the first (they share the activation arena), so both

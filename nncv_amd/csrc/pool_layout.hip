@@ -61,6 +61,117 @@ __global__ __launch_bounds__(256) void maxpool3x3s2_kernel(const T* __restrict__
   *reinterpret_cast<V*>(out + (((long long)n * OH + oy) * OW + ox) * C + cg * VN) = o;
 }
 
+// The same pooling for whole images at a time: one workgroup per output row, one thread per pair of neighbouring output
+// pixels and 16-byte channel group (the two windows share a column: 15 loads for two results instead of 18), 32-bit
+// index arithmetic throughout (the generic kernel above spends more time dividing 64-bit indices than loading).
+// fp16 keeps the halves packed: the running maximum is
+// v_pk_max_f16, which returns the other operand when one is a NaN, so NaNs are tracked next to it as the unsigned maximum
+// of the magnitudes (a NaN is a magnitude above infinity's 0x7c00) and put back at the end -- arith.maximumf
+// (tests/Nets/Pool2DMax.mlir:24) propagates them.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned short ushort8_t __attribute__((ext_vector_type(8)));
+typedef half_t half8_t __attribute__((ext_vector_type(8)));
+
+template <typename T>
+__global__ __launch_bounds__(256) void maxpool3x3s2_rows_kernel(const T* __restrict__ in, T* __restrict__ out, int H, int W, int C,
+                                                                int OH, int OW, unsigned in_bytes, unsigned inv_cg, unsigned n_rows) {
+  constexpr int VN = Vec16<T>::n;
+  const int CG = C / VN, pairs = (OW + 1) >> 1;
+  // Hardware deals workgroups to the 8 XCDs round-robin; neighbouring output rows share an input row, so each XCD takes a
+  // contiguous band of rows and its L2 serves the shared row (otherwise every shared row is fetched by two L2s).
+  const unsigned per_xcd = (n_rows + 7u) >> 3;
+  const unsigned row = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);  // n * OH + oy
+  if (row >= n_rows) return;
+  const unsigned n = row / (unsigned)OH, oy = row - n * (unsigned)OH;
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(in), 0, (int)in_bytes, 0x00020000);
+  const unsigned pix_b = (unsigned)C * sizeof(T);
+  for (unsigned e = threadIdx.x; e < (unsigned)(pairs * CG); e += 256) {
+    const unsigned px = __umulhi(e, inv_cg), cg = e - px * (unsigned)CG;  // e / CG, e % CG
+    const int ox0 = 2 * (int)px, ix0 = 2 * ox0 - 1;
+    // Coordinates outside the image are clamped to its border instead of being answered with -inf: a window that hangs
+    // over the border by its one halo row or column then reads a pixel it holds anyway, and a maximum does not mind
+    // seeing a value twice.  (The second output pixel of a last, odd pair reads clamped columns and is not stored.)
+    u32x4 v[3][5];
+    unsigned coff[5];
+#pragma unroll
+    for (int c = 0; c < 5; ++c) coff[c] = (unsigned)min(max(ix0 + c, 0), W - 1) * pix_b + cg * 16u;
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+      const int iy = min(max(2 * (int)oy - 1 + r, 0), H - 1);
+      const unsigned roff = (n * (unsigned)H + (unsigned)iy) * (unsigned)W * pix_b;
+#pragma unroll
+      for (int c = 0; c < 5; ++c) v[r][c] = __builtin_amdgcn_raw_buffer_load_b128(rs, roff + coff[c], 0, 0);
+    }
+    T* o = out + ((size_t)row * OW + ox0) * C + cg * VN;
+    if constexpr (sizeof(T) == 2) {
+      // Packed halves, one instruction per dword and operation, written out: the compiler's own rendering of the vector
+      // maximum canonicalises every operand first and splits the 16-bit masks into byte moves (600 instructions per
+      // thread, which made the kernel issue-bound).
+      const u32x4 ninf4 = {0xfc00fc00u, 0xfc00fc00u, 0xfc00fc00u, 0xfc00fc00u};  // -inf in both halves
+      u32x4 m0 = ninf4, m1 = ninf4, a0 = {0u, 0u, 0u, 0u}, a1 = a0;
+      auto fmax2 = [](unsigned x, unsigned y) {
+        unsigned d;
+        asm("v_pk_max_f16 %0, %1, %2" : "=v"(d) : "v"(x), "v"(y));
+        return d;
+      };
+      auto umax2 = [](unsigned x, unsigned y) {
+        unsigned d;
+        asm("v_pk_max_u16 %0, %1, %2" : "=v"(d) : "v"(x), "v"(y));
+        return d;
+      };
+#pragma unroll
+      for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int c = 0; c < 5; ++c)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const unsigned x = v[r][c][q], mag = x & 0x7fff7fffu;
+            if (c <= 2) {
+              m0[q] = fmax2(m0[q], x);
+              a0[q] = umax2(a0[q], mag);
+            }
+            if (c >= 2) {
+              m1[q] = fmax2(m1[q], x);
+              a1[q] = umax2(a1[q], mag);
+            }
+          }
+      // a magnitude above infinity's 0x7c00 among the nine: the result is a NaN
+      auto with_nans = [&](u32x4 m, u32x4 a) {
+        u32x4 o4;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const unsigned lo = (a[q] & 0xffffu) > 0x7c00u ? 0xffffu : 0u, hi = (a[q] >> 16) > 0x7c00u ? 0xffff0000u : 0u;
+          const unsigned mk = lo | hi;
+          o4[q] = (m[q] & ~mk) | (mk & 0x7e007e00u);
+        }
+        return o4;
+      };
+      *reinterpret_cast<u32x4*>(o) = with_nans(m0, a0);
+      if (ox0 + 1 < OW) *reinterpret_cast<u32x4*>(o + C) = with_nans(m1, a1);
+    } else {
+      float m0[4], m1[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) m0[q] = m1[q] = -INFINITY;
+#pragma unroll
+      for (int r = 0; r < 3; ++r) {
+#pragma unroll
+        for (int c = 0; c < 5; ++c) {
+          typedef float f4v __attribute__((ext_vector_type(4)));
+          const f4v vf = __builtin_bit_cast(f4v, v[r][c]);  // the whole vector: a bit cast of one element reads element 0
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            if (c <= 2) m0[q] = max_nan(m0[q], vf[q]);
+            if (c >= 2) m1[q] = max_nan(m1[q], vf[q]);
+          }
+        }
+      }
+      typedef float f4 __attribute__((ext_vector_type(4)));
+      *reinterpret_cast<f4*>(o) = f4{m0[0], m0[1], m0[2], m0[3]};
+      if (ox0 + 1 < OW) *reinterpret_cast<f4*>(o + C) = f4{m1[0], m1[1], m1[2], m1[3]};
+    }
+  }
+}
+
 void launch_maxpool3x3s2_nhwc(const void* in, void* out, int dt, int N, int H, int W, int C, hipStream_t s) {
   const int OH = (H + 2 - 3) / 2 + 1, OW = (W + 2 - 3) / 2 + 1;
   const int vn = dt == kF16 ? 8 : 4;
@@ -69,6 +180,21 @@ void launch_maxpool3x3s2_nhwc(const void* in, void* out, int dt, int N, int H, i
   const long long grid = (work + 255) / 256;
   NNCV_REQUIRE(grid < (1ll << 31), "maxpool: grid too large");
   ProfScope prof("maxpool3x3s2", 0.0, (double)dtype_size(dt) * N * C * ((double)H * W + (double)OH * OW), s);
+  const long long in_bytes = (long long)N * H * W * C * (long long)dtype_size(dt);
+  static const bool generic = getenv("NNCV_HIP_MAXPOOL_GENERIC") != nullptr;
+  // the row form addresses the input with 32-bit byte offsets and wants rows that give a workgroup something to do
+  if (!generic && in_bytes < (1ll << 31) && (long long)N * OH < (1ll << 31) && C / vn >= 2 && ((OW + 1) / 2) * (C / vn) >= 64) {
+    const unsigned inv_cg = C / vn == 1 ? 0u : (unsigned)(0xffffffffull / (unsigned)(C / vn) + 1);
+    const unsigned grid_rows = ((unsigned)(N * OH) + 7u) / 8u * 8u;
+    if (dt == kF16)
+      hipLaunchKernelGGL((maxpool3x3s2_rows_kernel<half_t>), dim3(grid_rows), dim3(256), 0, s, (const half_t*)in, (half_t*)out, H, W, C, OH, OW,
+                         (unsigned)in_bytes, inv_cg, (unsigned)(N * OH));
+    else
+      hipLaunchKernelGGL((maxpool3x3s2_rows_kernel<float>), dim3(grid_rows), dim3(256), 0, s, (const float*)in, (float*)out, H, W, C, OH, OW,
+                         (unsigned)in_bytes, inv_cg, (unsigned)(N * OH));
+    NNCV_HIP_CHECK(hipGetLastError());
+    return;
+  }
   if (dt == kF16)
     hipLaunchKernelGGL((maxpool3x3s2_kernel<half_t>), dim3((unsigned)grid), dim3(256), 0, s, (const half_t*)in, (half_t*)out, N, H, W, C, OH, OW);
   else

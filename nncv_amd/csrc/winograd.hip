@@ -251,8 +251,13 @@ struct WinoLds {
   static constexpr int VW = 16 / (int)sizeof(T);  // channels per thread
   static constexpr int CG = 64 / VW;              // channel groups per 64 channels
   static constexpr int kTiles = 240 / (6 * CG);   // fp16: 5, fp32: 2
+  // floats per row of 64 channels in LDS: four more than it holds.  The lanes of a wave are (channel group, u) pairs and u
+  // moves by one row: at a pitch of 64 floats all six u would meet in the same banks, at 68 the 16-byte accesses of any
+  // 16 neighbouring lanes fall into 16 different bank groups.
+  static constexpr int kRow = 68;
   typedef T Vec __attribute__((ext_vector_type(VW)));
 };
+typedef float wf4 __attribute__((ext_vector_type(4)));
 
 template <typename T>
 __global__ __launch_bounds__(256) void wino43_input_lds_kernel(const T* __restrict__ in, T* __restrict__ V, int N, int C, int H,
@@ -260,10 +265,14 @@ __global__ __launch_bounds__(256) void wino43_input_lds_kernel(const T* __restri
   typedef WinoLds<T> L;
   constexpr int VW = L::VW, CG = L::CG, KT = L::kTiles;
   typedef typename L::Vec Vec;
-  __shared__ __align__(16) float mid[KT][6][6][64];
+  __shared__ __align__(16) float mid[KT][6][6][L::kRow];
   const int tid = threadIdx.x;
   const long long tiles = (long long)N * TH * TW;
-  const long long tile0 = (long long)blockIdx.x * KT;
+  // Workgroups go to the 8 XCDs round-robin; tile rows share two input rows with the row below, so each XCD takes a
+  // contiguous range of tile blocks and its L2 serves the shared rows (measured: 1.64x the input bytes fetched otherwise).
+  const unsigned per_xcd = (gridDim.x + 7u) >> 3;
+  const unsigned blk = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+  const long long tile0 = (long long)blk * KT;
   const int c0 = blockIdx.y * 64;
   const int cg = tid % CG, u = (tid / CG) % 6, tl = tid / (6 * CG);
   const long long tile = tile0 + tl;
@@ -283,6 +292,7 @@ __global__ __launch_bounds__(256) void wino43_input_lds_kernel(const T* __restri
         for (int e = 0; e < VW; ++e) v[e] = (T)0.0f;
       d[y] = v;
     }
+    float t[6][VW];
 #pragma unroll
     for (int e = 0; e < VW; ++e) {
       float col[6], o[6];
@@ -290,31 +300,40 @@ __global__ __launch_bounds__(256) void wino43_input_lds_kernel(const T* __restri
       for (int y = 0; y < 6; ++y) col[y] = (float)d[y][e];
       bt6(col, o);
 #pragma unroll
-      for (int i = 0; i < 6; ++i) mid[tl][i][u][cg * VW + e] = o[i];
+      for (int i = 0; i < 6; ++i) t[i][e] = o[i];
     }
+#pragma unroll
+    for (int i = 0; i < 6; ++i)
+#pragma unroll
+      for (int e0 = 0; e0 < VW; e0 += 4)
+        *reinterpret_cast<wf4*>(&mid[tl][i][u][cg * VW + e0]) = wf4{t[i][e0], t[i][e0 + 1], t[i][e0 + 2], t[i][e0 + 3]};
   }
   __syncthreads();
   if (live) {  // pass 2: u = row i
+    // all VW channels of the lane at once: every store is 16 bytes, eight neighbouring lanes fill one 128-byte line
+    // (four channels at a time, the fp16 lanes wrote every line of V in two half-filled passes)
+    float o[6][VW];
 #pragma unroll
     for (int e0 = 0; e0 < VW; e0 += 4) {
-      float o[6][4];
+      wf4 rx[6];
+#pragma unroll
+      for (int x = 0; x < 6; ++x) rx[x] = *reinterpret_cast<const wf4*>(&mid[tl][u][x][cg * VW + e0]);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         float row[6], r[6];
 #pragma unroll
-        for (int x = 0; x < 6; ++x) row[x] = mid[tl][u][x][cg * VW + e0 + e];
+        for (int x = 0; x < 6; ++x) row[x] = rx[x][e];
         bt6(row, r);
 #pragma unroll
-        for (int j = 0; j < 6; ++j) o[j][e] = r[j];
+        for (int j = 0; j < 6; ++j) o[j][e0 + e] = r[j];
       }
+    }
 #pragma unroll
-      for (int j = 0; j < 6; ++j) {
-        typedef T V4 __attribute__((ext_vector_type(4)));
-        V4 w;
+    for (int j = 0; j < 6; ++j) {
+      Vec w;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) w[e] = (T)o[j][e];
-        *reinterpret_cast<V4*>(V + ((long long)(u * 6 + j) * tiles + tile) * C + c0 + cg * VW + e0) = w;
-      }
+      for (int e = 0; e < VW; ++e) w[e] = (T)o[j][e];
+      *reinterpret_cast<Vec*>(V + ((long long)(u * 6 + j) * tiles + tile) * C + c0 + cg * VW) = w;
     }
   }
 }
@@ -324,7 +343,7 @@ __global__ __launch_bounds__(256) void wino43_output_lds_kernel(const WinoOutArg
   typedef WinoLds<T> L;
   constexpr int VW = L::VW, CG = L::CG, KT = L::kTiles;
   typedef typename L::Vec Vec;
-  __shared__ __align__(16) float mid[KT][4][6][64];
+  __shared__ __align__(16) float mid[KT][4][6][L::kRow];
   const int tid = threadIdx.x;
   const long long tiles = (long long)a.N * TH * TW;
   const long long tile0 = (long long)blockIdx.x * KT;
@@ -337,6 +356,7 @@ __global__ __launch_bounds__(256) void wino43_output_lds_kernel(const WinoOutArg
     Vec m[6];
 #pragma unroll
     for (int i = 0; i < 6; ++i) m[i] = *reinterpret_cast<const Vec*>(M + ((long long)(i * 6 + u) * tiles + tile) * a.F + f0 + cg * VW);
+    float t[4][VW];
 #pragma unroll
     for (int e = 0; e < VW; ++e) {
       float col[6], o[4];
@@ -344,8 +364,13 @@ __global__ __launch_bounds__(256) void wino43_output_lds_kernel(const WinoOutArg
       for (int i = 0; i < 6; ++i) col[i] = (float)m[i][e];
       at6(col, o);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) mid[tl][r][u][cg * VW + e] = o[r];
+      for (int r = 0; r < 4; ++r) t[r][e] = o[r];
     }
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+      for (int e0 = 0; e0 < VW; e0 += 4)
+        *reinterpret_cast<wf4*>(&mid[tl][r][u][cg * VW + e0]) = wf4{t[r][e0], t[r][e0 + 1], t[r][e0 + 2], t[r][e0 + 3]};
   }
   __syncthreads();
   if (live && u < 4) {  // pass 2: u = row r
@@ -357,14 +382,21 @@ __global__ __launch_bounds__(256) void wino43_output_lds_kernel(const WinoOutArg
       const int f = f0 + cg * VW;
       float y[4][VW];
 #pragma unroll
-      for (int e = 0; e < VW; ++e) {
-        float row[6], o[4];
+      for (int e0 = 0; e0 < VW; e0 += 4) {
+        wf4 rj[6];
 #pragma unroll
-        for (int j = 0; j < 6; ++j) row[j] = mid[tl][u][j][cg * VW + e];
-        at6(row, o);
-        const float sc = a.scale ? a.scale[f + e] : 1.0f, sh = a.shift ? a.shift[f + e] : 0.0f;
+        for (int j = 0; j < 6; ++j) rj[j] = *reinterpret_cast<const wf4*>(&mid[tl][u][j][cg * VW + e0]);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) y[q][e] = o[q] * sc + sh;
+        for (int e1 = 0; e1 < 4; ++e1) {
+          const int e = e0 + e1;
+          float row[6], o[4];
+#pragma unroll
+          for (int j = 0; j < 6; ++j) row[j] = rj[j][e1];
+          at6(row, o);
+          const float sc = a.scale ? a.scale[f + e] : 1.0f, sh = a.shift ? a.shift[f + e] : 0.0f;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) y[q][e] = o[q] * sc + sh;
+        }
       }
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
@@ -425,10 +457,10 @@ void launch_wino43_input(const void* in, int in_dt, Strides4 st, void* V, int v_
       getenv("NNCV_HIP_WINO_SIMPLE") == nullptr) {
     const long long tiles = (long long)N * TH * TW;
     if (in_dt == kF16) {
-      dim3 g((unsigned)((tiles + WinoLds<half_t>::kTiles - 1) / WinoLds<half_t>::kTiles), C / 64);
+      dim3 g((unsigned)(((tiles + WinoLds<half_t>::kTiles - 1) / WinoLds<half_t>::kTiles + 7) / 8 * 8), C / 64);
       hipLaunchKernelGGL((wino43_input_lds_kernel<half_t>), g, dim3(256), 0, s, (const half_t*)in, (half_t*)V, N, C, H, W, pad, TH, TW);
     } else {
-      dim3 g((unsigned)((tiles + WinoLds<float>::kTiles - 1) / WinoLds<float>::kTiles), C / 64);
+      dim3 g((unsigned)(((tiles + WinoLds<float>::kTiles - 1) / WinoLds<float>::kTiles + 7) / 8 * 8), C / 64);
       hipLaunchKernelGGL((wino43_input_lds_kernel<float>), g, dim3(256), 0, s, (const float*)in, (float*)V, N, C, H, W, pad, TH, TW);
     }
     NNCV_HIP_CHECK(hipGetLastError());

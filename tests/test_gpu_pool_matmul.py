@@ -11,12 +11,18 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("dt", [abi.F32, abi.F16])
-@pytest.mark.parametrize("N,C,H,W", [(2, 64, 16, 16), (1, 8, 9, 7), (3, 16, 5, 6)])
+# the last three take the row form (a workgroup per output row, two output pixels per thread): odd and even widths,
+# a last pair with one pixel, the stem's own shape
+@pytest.mark.parametrize("N,C,H,W", [(2, 64, 16, 16), (1, 8, 9, 7), (3, 16, 5, 6), (2, 64, 37, 35), (3, 128, 20, 34), (1, 64, 112, 112)])
 def test_maxpool(dt, N, C, H, W):
     x = synth.normal(300, (N, C, H, W))
     if dt == abi.F16:
         x = synth.round_fp16(x)
     x[0, 1, 2, 2] = np.nan  # arith.maximumf propagates NaN
+    x[N - 1, C - 1, H - 1, W - 1] = np.nan
+    x[0, 3, H // 2, :] = -np.inf  # a window of nothing but -inf stays -inf
+    x[0, 3, H // 2 - 1, :] = -np.inf
+    x[0, 3, H // 2 + 1, :] = -np.inf
     want = oracle.maxpool3x3s2(x)
     OH, OW = want.shape[2:]
     out = empty((N, OH, OW, C), dt)

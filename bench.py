@@ -72,6 +72,7 @@ CLOCK_WARMUP_MS = 60.0          # untimed work ahead of a timed loop (see the mo
 # kernel tag -> (C, F, H=W) of the ResNet-18 layer at batch 32 that the tag's instance runs most
 DOMINANT_LAYER = {
     "conv3x3_stream<f16,1x2x2>": (128, 128, 28),
+    "conv3x3_stream<f16,1x4x1>": (128, 128, 28),
     "conv3x3_stream<f16,1x1x4>": (256, 256, 14),
     "conv3x3_patch<f16,4,1>": (64, 64, 56),
     "conv3x3_patch<f16,2,2>": (128, 128, 28),
@@ -89,7 +90,9 @@ DOMINANT_TRAFFIC = {  # profiles/resnet18_fp16_bs32_hbm_counters.txt, launches w
 
 
 # the same for the launch plan of three or more passes in flight
-IN_FLIGHT_TRAFFIC = {}  # filled from profiles/resnet18_fp16_bs32_in_flight_plan_hbm_counters.txt
+IN_FLIGHT_TRAFFIC = {  # profiles/resnet18_fp16_bs32_in_flight_plan_hbm_counters.txt, the layer alone, no residual input
+    "conv3x3_stream<f16,1x4x1>": (8980 + 6272) * 1024,
+}
 
 
 def main():

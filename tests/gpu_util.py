@@ -41,6 +41,15 @@ def max_rel(got, want):
     return float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
 
 
+def max_rel_elementwise(got, want, floor=1e-2):
+    """max over elements of |got - want| / max(|want|, floor * max|want|): the relative error of every element, with an
+    absolute floor for elements near zero (an element one hundredth of the largest or smaller is held to the error a
+    value of that size may have)."""
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    denom = np.maximum(np.abs(want), floor * max(np.abs(want).max(), 1e-30))
+    return float((np.abs(got - want) / denom).max())
+
+
 def rel_l2(got, want):
     got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
     return float(np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30))

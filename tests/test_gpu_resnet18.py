@@ -7,7 +7,7 @@ import torch
 
 import oracle
 from nncv_amd import abi, modelbin, synth
-from gpu_util import Model, dev, host, nchw, max_rel, rel_l2, FP32_MAX_REL, FP16_REL_L2
+from gpu_util import Model, dev, host, nchw, max_rel, max_rel_elementwise, rel_l2, FP32_MAX_REL, FP16_REL_L2
 
 pytestmark = pytest.mark.gpu
 
@@ -31,6 +31,8 @@ def test_fp32_small_image_with_taps(blob, algo):
     err = max_rel(host(logits), want_logits)
     print("logits max_rel", err, flush=True)
     assert err < FP32_MAX_REL
+    # every logit on its own, not only against the largest one (elements below 1 % of the largest against that floor)
+    assert max_rel_elementwise(host(logits), want_logits) < FP32_MAX_REL
     assert (host(logits).argmax(1) == want_logits.argmax(1)).all()
 
 
@@ -49,6 +51,7 @@ def test_cfg3_fp32_256_through_reference_abi(blob, tmp_path):
     print("cfg3 logits max_rel", err, "top1", got.argmax(1), want.argmax(1), flush=True)
     assert got.shape == (1, 1000)
     assert err < FP32_MAX_REL
+    assert max_rel_elementwise(got, want) < FP32_MAX_REL  # element by element, with a floor of 1 % of the largest logit
     assert (got.argmax(1) == want.argmax(1)).all()
     # second call hits the cached device model; a strided input view must give the same answer
     xs = np.zeros((1, 3, 256, 512), np.float32)[:, :, :, ::2]

@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 import torch
 
+import oracle
 from nncv_amd import abi, synth
 from gpu_util import Conv, dev, empty, host
 
@@ -49,6 +50,17 @@ def test_noalloc_matches_conv_forward_twice(dt):
     for (N, H, W, seed) in ((1, 8, 8, 9200), (1, 4, 4, 9300)):  # the K-split shape of config 3's last stage, then a smaller one
         print("noalloc case", dt, N, H, W, flush=True)
         got, want = run_pair(layer, dt, N, H, W, seed)
+        # against the CPU oracle as well, so that this file stands on its own: conv + BatchNorm + residual + ReLU
+        x = synth.normal(seed, (N, H, W, C))
+        res = synth.normal(seed + 1, (N, H, W, F))
+        if dt == abi.F16:
+            x, res = synth.round_fp16(x), synth.round_fp16(res)
+        ref = oracle.conv2d_nchw_fchw(oracle.pad_nchw(np.ascontiguousarray(x.transpose(0, 3, 1, 2)), 1), w, stride=1)
+        ref = oracle.relu(oracle.batchnorm(ref, *bn) + res.transpose(0, 3, 1, 2)).transpose(0, 2, 3, 1)
+        if dt == abi.F32:
+            assert max_rel(got, ref) < FP32_MAX_REL
+        else:
+            assert float(np.linalg.norm(got - ref) / np.linalg.norm(ref)) < FP16_REL_L2
         if dt == abi.F32:
             assert max_rel(got, want) < FP32_MAX_REL
         else:

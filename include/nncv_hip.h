@@ -104,8 +104,9 @@ int nncv_hip_resnet18_passes_in_flight(const nncv_hip_model* m);
  * (about 40 ms: chains of short one-wave kernels on eight candidate streams, pairwise) and hands out the streams that ran
  * side by side first.  *overlapping (may be NULL) = how many of the returned streams overlap pairwise; the rest fill the
  * list up.  More hardware queues (GPU_MAX_HW_QUEUES=8 in the environment before the process first touches HIP) make
- * four overlapping streams more likely.  The streams have the default priority, belong to the library and live until
- * the process ends.  No counterpart in the reference. */
+ * four overlapping streams more likely.  Call it while the device is otherwise idle (other work disturbs the timing).
+ * The streams have the default priority, belong to the library and live until the process ends.  No counterpart in
+ * the reference. */
 int nncv_hip_pick_streams(int want, void** streams, int* overlapping);
 void nncv_hip_resnet18_destroy(nncv_hip_model* m);
 /* A second handle on the SAME device weights (fp16 models only; an fp32 model keeps the tickets of its K-split launches

@@ -91,7 +91,7 @@ DOMINANT_TRAFFIC = {  # profiles/resnet18_fp16_bs32_hbm_counters.txt, launches w
 
 # the same for the launch plan of three or more passes in flight
 IN_FLIGHT_TRAFFIC = {  # profiles/resnet18_fp16_bs32_in_flight_plan_hbm_counters.txt, the layer alone, no residual input
-    "conv3x3_stream<f16,1x4x1>": (8980 + 6272) * 1024,
+    "conv3x3_stream<f16,1x4x1>": (8981 + 6272) * 1024,
 }
 
 

@@ -9,7 +9,8 @@
 //      (one 16-byte write per pair),
 //      so that one filter row (8 px x 4 ch = 32 halves) is 64 contiguous bytes starting at the
 //      pair of the output pixel (stride 2 = one pair per output pixel): every MFMA operand is one
-//      aligned 16-byte LDS read at a constant offset, with no im2col anywhere;
+//      aligned 16-byte LDS read at a constant offset, with no im2col anywhere (the eighth pixel of a row is the
+//      image pixel left of the window under a zero weight: a non-finite pixel there turns into NaN);
 //   2. K = 7 filter rows x 32 halves; the 64x224 filter matrix sits in registers for the whole
 //      life of the (persistent) workgroup, so the tap loop is 14 x (2 LDS reads + 4 MFMAs);
 //   3. scale/shift + ReLU in fp32, one rounding to fp16, tile to LDS ([pixel][64 ch], 16-byte writes: the MFMA rows

@@ -171,7 +171,7 @@ def _stage0(m, x16, N, H, W):
     return host(logits), nchw(host(tap))
 
 
-@pytest.mark.parametrize("shape", [(2, 64, 64), (1, 96, 160), (1, 70, 90), (3, 224, 224), (1, 34, 32)])
+@pytest.mark.parametrize("shape", [(2, 64, 64), (1, 96, 160), (1, 70, 90), (3, 224, 224), (1, 34, 32), (2, 226, 250)])
 def test_fp16_fused_stem_and_pool(blob, shape):
     """conv7x7 + BN + ReLU + max-pool in one launch: pooled activation and logits vs the oracle for
     square, wide, odd-sized and minimum images (partial tiles on every edge)."""
@@ -199,6 +199,30 @@ def test_fp16_fused_stem_propagates_nan(blob):
     assert np.isnan(want_tap).any() and not np.isnan(want_tap).all()
     assert np.array_equal(np.isnan(tap), np.isnan(want_tap))
     ok = ~np.isnan(want_tap)
+    assert rel_l2(tap[ok], want_tap[ok]) < 2e-3
+
+
+def test_fp16_fused_stem_nan_and_inf_at_tile_borders(blob):
+    """NaNs and infinities where the fused kernel's tiles meet (a pooled tile is 7 rows x 8 columns: image rows 28 k,
+    columns 32 k), in the image corners and in the last, partial tile: the same outputs are poisoned as in the oracle,
+    +inf stays +inf, and every other value is untouched.  The pixels sit in odd columns: the kernel's K axis pads a
+    filter row from seven to eight pixels with a zero weight on the even column left of the window, so a non-finite
+    pixel in an even column also reaches the window one further right as 0 x inf = NaN (a documented difference from
+    the reference, which images with finite pixels never see)."""
+    hb = synth.round_fp16(blob)
+    H, W = 120, 136
+    x = synth.round_fp16(synth.uniform(4310, (2, 3, H, W), -1.0, 1.0))
+    for (n, c, y, xx) in [(0, 0, 0, 1), (0, 2, 27, 31), (0, 1, 28, 33), (1, 0, 55, 63), (1, 2, H - 1, W - 1), (1, 1, 112, 5)]:
+        x[n, c, y, xx] = np.nan
+    x[0, 1, 60, 101] = np.inf
+    x[1, 0, 3, 131] = -np.inf
+    _, want_tap = oracle.resnet18_forward(x, hb, tap_layer=0)
+    m = Model(hb, abi.F16)
+    _, tap = _stage0(m, x, 2, H, W)
+    assert np.isnan(want_tap).any() and not np.isnan(want_tap).all()
+    assert np.array_equal(np.isnan(tap), np.isnan(want_tap))
+    assert np.array_equal(np.isposinf(tap), np.isposinf(want_tap))
+    ok = np.isfinite(want_tap)
     assert rel_l2(tap[ok], want_tap[ok]) < 2e-3
 
 

@@ -70,6 +70,13 @@ constexpr int kXcds = 8;
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
+// 16 bytes per lane from global memory straight into LDS: lane l to lds + 16 l.  A function of its own: with the builtin
+// called from the kernel template itself, the host pass of hipcc 7.2 can emit no launch stub for the kernel (and no
+// message), depending on the code around the call.
+__device__ __forceinline__ void load_to_lds16(__amdgpu_buffer_rsrc_t rs, unsigned char* lds, unsigned voffset) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)lds, 16, voffset, 0, 0, 0);
+}
+
 // s_waitcnt immediate that waits for all but the n youngest vector-memory operations and for nothing else
 constexpr int vmcnt_only(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0070 | 0x0f00; }
 
@@ -116,8 +123,9 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
   constexpr int BF = 32 * WF;        // filters per workgroup
   static_assert(kSteps % kRing == 0 || kRing % kSteps == 0, "the weight ring must tile a stage");
   constexpr int kPieceSteps = KPG >= 2 ? 9 : 5;  // K steps of a stage that carry the next patch's load instructions
-  static_assert(kPieceSteps < kSteps, "patch pieces per step");
-  // weight refills younger than the last patch piece at the end of a stage: what the wait for the patch may leave in flight
+  static_assert(kPieceSteps + 1 < kSteps, "the last piece is loaded in step kPieceSteps, the residual rows one step later");
+  // weight refills younger than the last patch piece (loaded in step kPieceSteps, ahead of that step's refill) at the end of
+  // a stage: what the wait for the patch may leave in flight
   constexpr int kYoung = kSteps - kPieceSteps < kRing ? kSteps - kPieceSteps : kRing;
   extern __shared__ __align__(16) unsigned char smem[];
 
@@ -218,16 +226,19 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
     const unsigned sg = (unsigned)wave * kLoadsPerWave + (unsigned)pp;
     segx[pp] = pp * kSegB + (int)(NSEG == 1 ? sg : (sg * rnseg) >> 16) * XB;
   }
-  unsigned pc_vo = 0;
+  // A piece's permute goes out a whole K step (five MFMAs) ahead of its load: LDS answers in order, so a load that
+  // follows its permute by one MFMA waits for every LDS read in flight, the next step's pixel operands included.
+  constexpr int kVo = 2 * ((kLoadsPerWave + kPieceSteps - 1) / kPieceSteps);  // permute results in flight
+  unsigned pc_vo[kVo];
   auto patch_piece_perm = [&](auto p_c) {  // the lanes' cell offsets for piece p
     constexpr int pp = decltype(p_c)::value;
-    pc_vo = (unsigned)__builtin_amdgcn_ds_bpermute(perm0 + 28 * pp, (int)celloff);
+    pc_vo[pp % kVo] = (unsigned)__builtin_amdgcn_ds_bpermute(perm0 + 28 * pp, (int)celloff);
   };
   auto patch_piece_load = [&](auto p_c) {
     constexpr int pp = decltype(p_c)::value;
     // out of range stays out of range under this sum, except for the pad chunk of a cell that is itself out of
     // range (the two flags cancel): that unit then loads the tensor's first bytes into a pad nobody reads
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_in, (lds_ptr_t)(smem + pc_dst + segx[pp]), 16, pc_vo + pc_lchslab, 0, 0, 0);
+    load_to_lds16(rs_in, smem + pc_dst + segx[pp], pc_vo[pp % kVo] + pc_lchslab);
   };
   // the first patch of a workgroup: nothing to hide the permutes' latency under, so all nine go out before the loads
   auto patch_all = [&]() {
@@ -236,7 +247,7 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
     for (int pp = 0; pp < kLoadsPerWave; ++pp) pv[pp] = (unsigned)__builtin_amdgcn_ds_bpermute(perm0 + 28 * pp, (int)celloff);
 #pragma unroll
     for (int pp = 0; pp < kLoadsPerWave; ++pp)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_in, (lds_ptr_t)(smem + pc_dst + segx[pp]), 16, pv[pp] + pc_lchslab, 0, 0, 0);
+      load_to_lds16(rs_in, smem + pc_dst + segx[pp], pv[pp] + pc_lchslab);
   };
 
   patch_tile(tile, true);
@@ -371,18 +382,23 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
             if constexpr (st + 1 < kSteps) {
               if (rowlive) ldp1(std::integral_constant<int, st + 1>(), j);
             }
-            // the next patch: kLoadsPerWave pieces over the first K steps of the stage
+            // the next patch: kLoadsPerWave pieces, their permutes over the first kPieceSteps K steps of the stage,
+            // each load one step behind its permute
             if constexpr (st * PPS < kLoadsPerWave) {
               if (j == 0) patch_piece_perm(std::integral_constant<int, st * PPS>());
-              if (j == 1) patch_piece_load(std::integral_constant<int, st * PPS>());
               if constexpr (PPS == 2 && st * PPS + 1 < kLoadsPerWave) {
                 if (j == 2) patch_piece_perm(std::integral_constant<int, st * PPS + 1>());
-                if (j == 3) patch_piece_load(std::integral_constant<int, st * PPS + 1>());
+              }
+            }
+            if constexpr (st >= 1 && (st - 1) * PPS < kLoadsPerWave) {
+              if (j == 1) patch_piece_load(std::integral_constant<int, (st - 1) * PPS>());
+              if constexpr (PPS == 2 && (st - 1) * PPS + 1 < kLoadsPerWave) {
+                if (j == 3) patch_piece_load(std::integral_constant<int, (st - 1) * PPS + 1>());
               }
             }
             // the residual rows this wave finishes go out in the tile's last stage, behind the patch pieces (no
             // residual: a buffer of no bytes, the loads return zeros without touching memory)
-            if constexpr (st == kPieceSteps) {
+            if constexpr (st == kPieceSteps + 1) {
               if (j < NOWN && last) {
                 rv[j % NOWN][0] = __builtin_amdgcn_raw_buffer_load_b128(rs_res, obase[j % NOWN], 0, 0);
                 rv[j % NOWN][1] = __builtin_amdgcn_raw_buffer_load_b128(rs_res, obase[j % NOWN], 16, 0);

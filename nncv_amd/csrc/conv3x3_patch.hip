@@ -500,9 +500,13 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
     obase[j] = ok ? (((n0 + nl) * OH + y0 + ty) * OW + x0 + tx) * a.ldo : -1;
   }
 
-  floatx16 acc[2][2];  // [filter half][pixel half]; with NI = 1 only acc[0] is used
+  // [filter half][pixel half]; with NI = 1 only acc[0] is used.  The first step of the first slab starts the sums from a
+  // zero C operand: clearing the registers instead cost 64 moves between the patch barrier and the first MFMA.
+  // (fp16 instances; the fp32 ones, four chained MFMAs per product, are at their register limit and keep the moves.)
+  constexpr bool kZeroC = sizeof(T) == 2;
+  floatx16 acc[2][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = kZeroC ? 1 : 0; i < 2; ++i)  // fp16, NI = 1: acc[1] is never written by an MFMA and never read for a result
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -532,6 +536,16 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
       else  // filter columns 0, 1, 2 = even column, the odd one after it, the next even one
         ring[st % kDepth][j] = *reinterpret_cast<const u32x4*>(patch + rowbase[t / 3][j] + (t % 3 == 1 ? odd_col : 0) + (t % 3 == 2 ? kPitch : 0) + k * 32);
   };
+  auto ldp1 = [&](auto step_c, int j) {
+    constexpr int st = decltype(step_c)::value;
+    constexpr int t = st / KPG, k = st % KPG;
+    if constexpr (ST == 1)
+      ring[st % kDepth][j] = *reinterpret_cast<const u32x4*>(patch + rowbase[t / 3][j] + (t % 3) * kPitch + k * 32);
+    else
+      ring[st % kDepth][j] = *reinterpret_cast<const u32x4*>(patch + rowbase[t / 3][j] + (t % 3 == 1 ? odd_col : 0) + (t % 3 == 2 ? kPitch : 0) + k * 32);
+  };
+  // the fp16 instances spread a step's other instructions between its MFMAs (see the tap loop)
+  constexpr bool kSpread = sizeof(T) == 2;
   auto prime = [&](auto self, auto d_c) -> void {  // the first kDepth-1 steps of a fresh patch
     constexpr int d = decltype(d_c)::value;
     if constexpr (d < kDepth - 1) {
@@ -551,18 +565,40 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
       constexpr int st = decltype(step_c)::value;
       if constexpr (st < kSteps) {
         constexpr int t = st / KPG, k = st % KPG, set = t % NSET;
-        if constexpr (st + kDepth - 1 < kSteps) ldp(std::integral_constant<int, st + kDepth - 1>());
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 0; i < NI; ++i)
-#pragma unroll
-          for (int j = 0; j < 2; ++j) Mma<T>::run(wregs[set][k * NI + i], ring[st % kDepth][j], acc[i][j]);
         const int it_next = slab * 9 + t + NSET;
         const int wso = it_next < niter ? wbase + it_next * 8192 : 0;  // past the end: re-read block 0 (never used)
+        if constexpr (kSpread) {
+          // every MFMA is followed by its share of the step's other instructions (an LDS read of the step kDepth - 1
+          // ahead, a weight refill), so that they issue under it instead of behind the four: 7x7x512 at batch 32
+          // 13.3 -> 12.9 us (one wave per SIMD), the stride-2 launches 10.0 -> 9.4, 56x56x64 14.4 -> 14.05
 #pragma unroll
-        for (int i = 0; i < NI; ++i)
-          wregs[set][k * NI + i] = __builtin_amdgcn_raw_buffer_load_b128(rs_wf, wlane, wso + wfrag(k, i), 0);
-        __builtin_amdgcn_sched_barrier(0);
+          for (int i = 0; i < NI; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              if (kZeroC && st == 0 && slab == 0) Mma<T>::start(wregs[set][k * NI + i], ring[st % kDepth][j], acc[i][j]);
+              else Mma<T>::run(wregs[set][k * NI + i], ring[st % kDepth][j], acc[i][j]);
+              __builtin_amdgcn_sched_barrier(0);
+              if constexpr (st + kDepth - 1 < kSteps) {
+                if (i == 0) ldp1(std::integral_constant<int, st + kDepth - 1>(), j);
+              }
+              if (j == 1) wregs[set][k * NI + i] = __builtin_amdgcn_raw_buffer_load_b128(rs_wf, wlane, wso + wfrag(k, i), 0);
+              __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+          if constexpr (st + kDepth - 1 < kSteps) ldp(std::integral_constant<int, st + kDepth - 1>());
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int i = 0; i < NI; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              if (kZeroC && st == 0 && slab == 0) Mma<T>::start(wregs[set][k * NI + i], ring[st % kDepth][j], acc[i][j]);
+              else Mma<T>::run(wregs[set][k * NI + i], ring[st % kDepth][j], acc[i][j]);
+            }
+#pragma unroll
+          for (int i = 0; i < NI; ++i)
+            wregs[set][k * NI + i] = __builtin_amdgcn_raw_buffer_load_b128(rs_wf, wlane, wso + wfrag(k, i), 0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
         self(self, std::integral_constant<int, st + 1>());
       }
     };

@@ -20,6 +20,11 @@ struct Mma<half_t> {  // lane = row l%32, k = 8*(l/32) .. +7
   static __device__ __forceinline__ void run(const u32x4& a, const u32x4& b, floatx16& c) {
     c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0, 0, 0);
   }
+  // the first product of a sum: a zero C operand instead of sixteen cleared registers
+  static __device__ __forceinline__ void start(const u32x4& a, const u32x4& b, floatx16& c) {
+    const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), zero, 0, 0, 0);
+  }
 };
 template <>
 struct Mma<float> {  // lane = row l%32, k = l/32; the 4 floats of a chunk feed 4 MFMAs
@@ -27,6 +32,13 @@ struct Mma<float> {  // lane = row l%32, k = l/32; the 4 floats of a chunk feed 
     const floatx4 fa = __builtin_bit_cast(floatx4, a), fb = __builtin_bit_cast(floatx4, b);
 #pragma unroll
     for (int j = 0; j < 4; ++j) c = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[j], fb[j], c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ void start(const u32x4& a, const u32x4& b, floatx16& c) {
+    const floatx4 fa = __builtin_bit_cast(floatx4, a), fb = __builtin_bit_cast(floatx4, b);
+    const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[0], fb[0], zero, 0, 0, 0);
+#pragma unroll
+    for (int j = 1; j < 4; ++j) c = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[j], fb[j], c, 0, 0, 0);
   }
 };
 

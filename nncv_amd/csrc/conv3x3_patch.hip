@@ -550,6 +550,7 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
     constexpr int d = decltype(d_c)::value;
     if constexpr (d < kDepth - 1) {
       ldp(d_c);
+      __builtin_amdgcn_sched_barrier(0);  // in step order: left alone the compiler issued the first step's reads last
       self(self, std::integral_constant<int, d + 1>());
     }
   };

@@ -33,13 +33,7 @@ struct Mma<float> {  // lane = row l%32, k = l/32; the 4 floats of a chunk feed 
 #pragma unroll
     for (int j = 0; j < 4; ++j) c = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[j], fb[j], c, 0, 0, 0);
   }
-  static __device__ __forceinline__ void start(const u32x4& a, const u32x4& b, floatx16& c) {
-    const floatx4 fa = __builtin_bit_cast(floatx4, a), fb = __builtin_bit_cast(floatx4, b);
-    const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    c = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[0], fb[0], zero, 0, 0, 0);
-#pragma unroll
-    for (int j = 1; j < 4; ++j) c = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[j], fb[j], c, 0, 0, 0);
-  }
+  static __device__ __forceinline__ void start(const u32x4& a, const u32x4& b, floatx16& c) { run(a, b, c); }  // fp32 sums are cleared by their owner
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, unsigned bytes) {

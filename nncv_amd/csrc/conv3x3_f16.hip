@@ -81,11 +81,11 @@ __device__ __forceinline__ void load_to_lds16(__amdgpu_buffer_rsrc_t rs, unsigne
 constexpr int vmcnt_only(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0070 | 0x0f00; }
 
 struct StreamArgs {
-  // ---- what the first requests need: these 16 dwords arrive preloaded in SGPRs, ahead of the scalar load
-  //      that brings the rest ----
+  // ---- what the first requests need.  The kernel takes these 14 dwords as plain leading arguments: those arrive
+  //      preloaded in SGPRs at wave launch (a struct passed by value does not: its fields come by scalar loads, three
+  //      of them in a row here before the first weight request could go out), the rest follows as a struct ----
   const void* in;         // NHWC [N][H][W][pix]
   const void* wf;         // launch_weight_frag32 order
-  unsigned in_bytes, wf_bytes;
   unsigned G, div, mdiv;  // workgroup -> (filter block, first tile): see launch_conv3x3_stream
   unsigned mS32;          // ceil(2^32 / S)
   unsigned n_tiles;
@@ -95,14 +95,18 @@ struct StreamArgs {
   unsigned pixB;               // bytes between input pixels
   unsigned rowx_rnseg;         // bytes a patch row is longer than its segments | ceil(2^16 / NSEG) << 16 (0 when NSEG is 1)
   // ---- the end of a tile needs these ----
-  void* out;              // NHWC [N][H][W][ldo]
-  const float* scale;     // [F] or null
-  const float* shift;     // [F] or null
-  const void* residual;   // like out, or null
-  unsigned out_bytes, mW16;  // mW16 = ceil(2^16 / W)
-  int F, act, ldo;
+  struct Tail {
+    void* out;              // NHWC [N][H][W][ldo]
+    const float* scale;     // [F] or null
+    const float* shift;     // [F] or null
+    const void* residual;   // like out, or null
+    unsigned out_bytes, mW16;  // mW16 = ceil(2^16 / W)
+    int F, act, ldo;
+  } t;
 };
-static_assert(offsetof(StreamArgs, out) == 64, "sixteen preloaded dwords");
+// Input and weights are addressed through descriptors of 2^31 bytes: every offset the kernel forms for a cell or a
+// fragment that exists lies inside its tensor (the host checks the sizes), and what must read as zero carries kOOBs.
+constexpr unsigned kWholeRange = 0x80000000u;
 
 // Geometry: rows of all images are stacked into virtual rows, image n's row y being v = n*S + top + y; tile t
 // covers virtual rows [top + t*TH, +TH) and W columns.  The patch of a tile is its TH + 2 rows of W + 2 cells,
@@ -113,7 +117,13 @@ static_assert(offsetof(StreamArgs, out) == 64, "sixteen preloaded dwords");
 // eight waves: one, whose waves w and w + 4 share a SIMD -- one of each pixel group, so that a tile of seven
 // rows (four + three) loads all SIMDs alike.
 template <int PG, int WF, int WK, bool ACT>
-__global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv3x3_f16_stream_kernel(const StreamArgs a) {
+__global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv3x3_f16_stream_kernel(
+    const void* in_p, const void* wf_p, unsigned G_p, unsigned div_p, unsigned mdiv_p, unsigned mS32_p, unsigned n_tiles_p,
+    unsigned flags_p, unsigned N_TH_p, unsigned geom_p, unsigned pixB_p, unsigned rowx_rnseg_p, const StreamArgs::Tail tail) {
+  StreamArgs a;
+  a.in = in_p; a.wf = wf_p; a.G = G_p; a.div = div_p; a.mdiv = mdiv_p; a.mS32 = mS32_p; a.n_tiles = n_tiles_p;
+  a.tstep_nslab_flags = flags_p; a.N_TH = N_TH_p; a.geom = geom_p; a.pixB = pixB_p; a.rowx_rnseg = rowx_rnseg_p;
+  a.t = tail;
   static_assert(WF * WK == 4 && (PG == 1 || PG == 2), "four or eight waves");
   constexpr int NW = PG * WF * WK;
   constexpr int kPatchB = patch_bytes(NW);
@@ -158,7 +168,7 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
   const int tend = (int)a.n_tiles;
   if (tile >= tend) return;
 
-  const __amdgpu_buffer_rsrc_t rs_wf = make_rsrc(a.wf, a.wf_bytes);
+  const __amdgpu_buffer_rsrc_t rs_wf = make_rsrc(a.wf, kWholeRange);
 
   // ---- weights: fragment (filter group g, iteration it = slab*9 + tap, sub-step kk) is the kilobyte at
   //      ((g*niter + it)*4 + kk)*1024; a wave streams its KPG sub-steps of every iteration ----
@@ -199,7 +209,7 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
   const unsigned cseg = (unsigned)wave * kLoadsPerWave + (((unsigned)lane * 37u) >> 8);  // its segment: lane / 7
   const unsigned crow = NSEG == 1 ? cseg : (cseg * rnseg) >> 16;                           // its patch row: cseg / NSEG
   const unsigned ccol = (cseg - crow * NSEG) * kSegCells + ((unsigned)lane - (((unsigned)lane * 37u) >> 8) * 7u) - 1u;  // image column
-  const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(a.in, a.in_bytes);
+  const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(a.in, kWholeRange);
   unsigned celloff = kOOBs;  // tensor offset of that cell for the tile being loaded
   unsigned pc_lchslab = 0;   // lchoff + the channel slab's byte offset in a pixel
   int pc_dst = 0;            // LDS offset of this wave's first segment in the buffer being filled
@@ -213,7 +223,10 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
     const unsigned n = nS - 1u, y = vS - nS * S - top;
     const unsigned bad = (unsigned)(y >= H) | (unsigned)(n >= N) | (unsigned)(ccol >= W) | (unsigned)(crow >= TH + 2u) |
                          (unsigned)(aligned & (n != nt)) | (unsigned)!live;
-    celloff = (((n * H + y) * W + ccol) * a.pixB) | (bad ? kOOBs : 0u);
+    // a cell that is not there gets exactly kOOBs, not its (meaningless) offset with the flag set: the pad lane of such a
+    // cell adds a second kOOBs, the flags cancel, and what is left must be an offset inside the tensor (its first bytes,
+    // into a pad nobody reads) -- the descriptor spans 2^31 bytes and would not stop anything else
+    celloff = bad ? kOOBs : ((n * H + y) * W + ccol) * a.pixB;
   };
   auto patch_begin = [&](int slab, int dstbuf) {
     pc_lchslab = lchoff + (unsigned)slab * 128u;
@@ -263,8 +276,8 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
   __builtin_amdgcn_sched_barrier(0);
 
   // ---- everything below needs the rest of the arguments ----
-  const __amdgpu_buffer_rsrc_t rs_out = make_rsrc(a.out, a.out_bytes);
-  const __amdgpu_buffer_rsrc_t rs_res = make_rsrc(a.residual ? a.residual : a.out, a.residual ? a.out_bytes : 0u);
+  const __amdgpu_buffer_rsrc_t rs_out = make_rsrc(a.t.out, a.t.out_bytes);
+  const __amdgpu_buffer_rsrc_t rs_res = make_rsrc(a.t.residual ? a.t.residual : a.t.out, a.t.residual ? a.t.out_bytes : 0u);
 
   // Scale and shift of the block's filters wait in LDS behind the patch buffers (32 registers less across
   // the taps).  They are requested here and written at the end of the first stage: writing them now would
@@ -275,8 +288,8 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
   {
     const unsigned off = (unsigned)(fb * BF + 4 * (ss_shift ? sse - BF / 4 : sse)) * 4u;
     // a missing vector is a buffer of no bytes: the load returns zeros and the select later fills in 1 / 0
-    const __amdgpu_buffer_rsrc_t rs_sc = make_rsrc(a.scale ? a.scale : a.in, a.scale ? (unsigned)a.F * 4u : 0u);
-    const __amdgpu_buffer_rsrc_t rs_sh = make_rsrc(a.shift ? a.shift : a.in, a.shift ? (unsigned)a.F * 4u : 0u);
+    const __amdgpu_buffer_rsrc_t rs_sc = make_rsrc(a.t.scale ? a.t.scale : a.in, a.t.scale ? (unsigned)a.t.F * 4u : 0u);
+    const __amdgpu_buffer_rsrc_t rs_sh = make_rsrc(a.t.shift ? a.t.shift : a.in, a.t.shift ? (unsigned)a.t.F * 4u : 0u);
     vsc = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rs_sc, off, 0, 0));
     vsh = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rs_sh, off, 0, 0));
   }
@@ -292,7 +305,7 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
       const unsigned back = (((s - live) >> 4) + 1u) << 4;
       s = s >= back ? s - back : 0u;
     }
-    const unsigned ty = (s * a.mW16) >> 16, tx = s - ty * W;
+    const unsigned ty = (s * a.t.mW16) >> 16, tx = s - ty * W;
 #pragma unroll
     for (int r = 0; r < 3; ++r) rowbase[r][j] = (int)(ty + r) * RPB + (int)tx * kPitchS + (lchunk + 2 * wk * KPG) * 16;
   }
@@ -303,13 +316,13 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
 #pragma unroll
     for (int j = 0; j < NOWN; ++j) {
       const unsigned s = (unsigned)(pg * kSlots + (wk * NOWN + j) * 32 + lrow);
-      const unsigned ty = (s * a.mW16) >> 16, tx = s - ty * W;
+      const unsigned ty = (s * a.t.mW16) >> 16, tx = s - ty * W;
       const unsigned v = v0 + ty;
       const unsigned n = __umulhi(v, a.mS32);
       const unsigned y = v - n * S - top;
       const unsigned bad = (unsigned)(ty >= TH) | (unsigned)(y >= H) | (unsigned)(n >= N);
       const unsigned pixel = (n * H + y) * W + tx;
-      obase[j] = ((pixel * (unsigned)a.ldo + (unsigned)f0) * 2u) | (bad ? kOOBs : 0u);
+      obase[j] = ((pixel * (unsigned)a.t.ldo + (unsigned)f0) * 2u) | (bad ? kOOBs : 0u);
     }
   };
   tile_outputs(tile);
@@ -425,7 +438,7 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
       __builtin_amdgcn_sched_barrier(0);
       if (ss_pending) {
         asm volatile("" : "+v"(vsc), "+v"(vsh));  // keeps this arithmetic (and its wait for the two loads) here
-        const float one = a.scale ? 0.0f : 1.0f;  // added to the zeros of a missing scale vector
+        const float one = a.t.scale ? 0.0f : 1.0f;  // added to the zeros of a missing scale vector
         floatx4 ssv;
 #pragma unroll
         for (int q = 0; q < 4; ++q) ssv[q] = ss_shift ? vsh[q] : vsc[q] + one;
@@ -500,9 +513,9 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
         for (int q = 0; q < 4; ++q)
 #pragma unroll
           for (int e = 0; e < 4; ++e) y[4 * q + e] = acc[j][4 * q + e] * sc4[q][e] + sh4[q][e];
-        const bool res_after = ACT && (a.act & kActResidualAfter);
+        const bool res_after = ACT && (a.t.act & kActResidualAfter);
         float rf[FPL];
-        if (a.residual) {
+        if (a.t.residual) {
           const half8 r0 = __builtin_bit_cast(half8, rv[o][0]), r1 = __builtin_bit_cast(half8, rv[o][1]);
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
@@ -514,13 +527,13 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
             for (int e = 0; e < FPL; ++e) y[e] += rf[e];
           }
         }
-        if (a.act == kActRelu) {
+        if (a.t.act == kActRelu) {
 #pragma unroll
           for (int e = 0; e < FPL; ++e) y[e] = relu_ugt(y[e]);
-        } else if (ACT && a.act) {
-          act_apply_n<true>(y, a.act & 0xff);
+        } else if (ACT && a.t.act) {
+          act_apply_n<true>(y, a.t.act & 0xff);
         }
-        if (a.residual && res_after) {
+        if (a.t.residual && res_after) {
 #pragma unroll
           for (int e = 0; e < FPL; ++e) y[e] += rf[e];
         }
@@ -745,7 +758,8 @@ static void launch_stream_cfg(const StreamArgs& a, int grid, double flops, doubl
   }();
   (void)attr;
   ProfScope prof(tag, flops, bytes, s);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), smem, s, a);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), smem, s, a.in, a.wf, a.G, a.div, a.mdiv, a.mS32, a.n_tiles, a.tstep_nslab_flags, a.N_TH, a.geom,
+                     a.pixB, a.rowx_rnseg, a.t);
 }
 
 bool launch_conv3x3_stream(const IgemmArgs& g, hipStream_t s) {
@@ -761,11 +775,9 @@ bool launch_conv3x3_stream(const IgemmArgs& g, hipStream_t s) {
   NNCV_REQUIRE(Wpf < 65536 && g.C / 64 < 256, "conv3x3_stream: tile step / slab count out of range");
   StreamArgs a{};
   const int pix = g.pix_stride ? g.pix_stride : g.C;
-  a.in = g.in; a.wf = g.wt_frag32; a.out = g.out; a.scale = g.scale; a.shift = g.shift; a.residual = g.residual;
-  a.F = g.F; a.act = g.relu; a.ldo = g.ldo;
-  a.in_bytes = g.in_bytes ? g.in_bytes : (unsigned)((size_t)g.N * g.H * g.W * pix * 2);
-  a.wf_bytes = (unsigned)wbytes;
-  a.out_bytes = (unsigned)((size_t)g.N * g.H * g.W * g.ldo * 2);
+  a.in = g.in; a.wf = g.wt_frag32; a.t.out = g.out; a.t.scale = g.scale; a.t.shift = g.shift; a.t.residual = g.residual;
+  a.t.F = g.F; a.t.act = g.relu; a.t.ldo = g.ldo;
+  a.t.out_bytes = (unsigned)((size_t)g.N * g.H * g.W * g.ldo * 2);
   a.G = (unsigned)G;
   a.div = (unsigned)(by_filter ? Wpf : FB);
   a.mdiv = recip32(a.div);
@@ -776,7 +788,7 @@ bool launch_conv3x3_stream(const IgemmArgs& g, hipStream_t s) {
   a.geom = (unsigned)g.H | ((unsigned)g.W << 8) | ((unsigned)geo.S << 16) | ((unsigned)geo.NSEG << 24);
   a.pixB = (unsigned)pix * 2u;
   a.rowx_rnseg = (unsigned)geo.rowx | (geo.NSEG == 1 ? 0u : (unsigned)(65535 / geo.NSEG + 1) << 16);
-  a.mW16 = (unsigned)((65536 + g.W - 1) / g.W);
+  a.t.mW16 = (unsigned)((65536 + g.W - 1) / g.W);
   const double P = (double)g.N * g.H * g.W;
   const double flops = 2.0 * P * g.C * 9.0 * g.F;
   const double bytes = 2.0 * (P * g.C + 9.0 * g.C * g.F + P * g.F * (g.residual ? 2 : 1));

@@ -128,3 +128,62 @@ def test_invariants_hold_under_the_overlap_hint(plan):
     finally:
         assert L.nncv_hip_set_overlap_hint(1) == 0
     assert plan(32, 14, 14, 256, 256)["WF"] == 2
+
+
+def _loader_offsets(p, N, H, W, C):
+    """The byte offsets the kernel's patch loader forms (conv3x3_f16.hip, patch_tile / patch_piece_load), in the
+    kernel's own 32-bit arithmetic: for every tile, the pass behind the last tile, every wave, piece, lane and slab."""
+    M, OOB = 0xFFFFFFFF, 0x80000000
+    TH, S, top, NSEG = p["TH"], p["S"], p["top"], p["NSEG"]
+    mS32 = (M // S + 1) & M
+    rnseg = 65535 // NSEG + 1 if NSEG > 1 else 0
+    pixB = C * 2
+    out = []
+    for wave in range(4 * p["PG"]):
+        cells = []  # (crow, ccol) of the cell each lane works out
+        for lane in range(64):
+            cseg = wave * 9 + ((lane * 37) >> 8)
+            crow = cseg if NSEG == 1 else (cseg * rnseg) >> 16
+            ccol = ((cseg - crow * NSEG) * 7 + (lane - ((lane * 37) >> 8) * 7) - 1) & M
+            cells.append((crow, ccol))
+        for t in list(range(p["tiles"])) + [None]:
+            live = t is not None
+            tt = t if live else p["tiles"] + 3
+            v0 = (top + tt * TH) & M
+            nt = (v0 * mS32) >> 32
+            celloff = []
+            for crow, ccol in cells:
+                vS = (v0 - 1 + crow + S) & M
+                nS = (vS * mS32) >> 32
+                n = (nS - 1) & M
+                y = (vS - nS * S - top) & M
+                bad = y >= H or n >= N or ccol >= W or crow >= TH + 2 or (p["aligned"] == 1 and n != nt) or not live
+                celloff.append(OOB if bad else (((n * H + y) * W + ccol) * pixB) & M)
+            for pp in range(9):
+                for lane in range(64):
+                    lcell = (lane * 57) >> 9
+                    lch = lane - 9 * lcell
+                    lchoff = OOB if lch == 8 else lch * 16
+                    vo = celloff[lcell + 7 * pp]
+                    for slab in range(C // 64):
+                        out.append((vo + lchoff + slab * 128) & M)
+    return np.array(out, dtype=np.int64)
+
+
+@pytest.mark.parametrize("shape", [(8, 28, 28, 128, 128), (16, 14, 14, 256, 256), (4, 56, 56, 64, 64), (3, 7, 7, 512, 512),
+                                   (5, 20, 24, 64, 96), (2, 9, 100, 128, 32)])
+def test_loader_offsets_are_out_of_range_or_inside_the_tensor(plan, shape):
+    """The kernel addresses its input through a descriptor of 2^31 bytes (the tensor's size is not among the
+    arguments that arrive preloaded), so the range check stops nothing below 2^31: every offset the loader forms must
+    either carry the out-of-range flag or lie inside the tensor -- also for cells that do not exist, for the pad lane
+    of such a cell (two flags that cancel) and for the pass behind the last tile."""
+    N, H, W, C, F = shape
+    p = plan(N, H, W, C, F)
+    if p is None:
+        pytest.skip("no stream plan for this shape")
+    off = _loader_offsets(p, N, H, W, C)
+    in_bytes = N * H * W * C * 2
+    inside = off + 16 <= in_bytes
+    flagged = off >= 0x80000000
+    assert (inside | flagged).all(), (shape, [hex(int(v)) for v in off[~(inside | flagged)][:4]])
+    assert inside.any() and flagged.any()

@@ -325,7 +325,7 @@ def main():
                                       "and have no duration of their own")
     roofline["launch_shapes"] = ("those of one pass at a time (overlap hint 1), which the summaries under profiles/ hold; with "
                                  "three or more passes in flight layer2 / layer3 run the same kernel's 128-filter form and "
-                                 "layer1 the patch kernel (see config.passes_in_flight), where a launch of one pass has no "
+                                 "layer1 its resident-weight form on half the places (see config.passes_in_flight), where a launch of one pass has no "
                                  "duration of its own")
     conv3x3_flops = 13 * 2 * 56 * 56 * 64 * 64 * 9 * N  # the 13 stride-1 3x3 layers all cost the same per image
     out = {

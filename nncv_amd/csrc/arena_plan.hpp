@@ -36,8 +36,9 @@ bool arena_linger_forced();
 // told otherwise, NNCV_HIP_OVERLAP sets the initial value).  From three up the planners pick the forms that measured
 // faster when launches of different passes share the chip -- what counts then is how long a launch's workgroups hold
 // their LDS and register slots, not how soon the launch ends: the 128-filter form of the 3x3 stream kernel wherever
-// the filter count allows it (half the workgroups of the 64-filter form, no exchange between K groups) and the patch
-// kernel's 256-slot form where it does not; in ResNet-18 from batch 16 up also no lingering in the arena (the penalty
+// the filter count allows it (half the workgroups of the 64-filter form, no exchange between K groups), for one-slab
+// layers the 64-filter form with resident weights on half the places, and the patch kernel where neither fits; in
+// ResNet-18 from batch 16 up also no lingering in the arena (the penalty
 // it avoids belongs to launches that have the chip to themselves; four smaller working sets share the caches better:
 // 0.165 against 0.168 ms -- MobileNetV3's small tensors measured the other way, 0.169 against 0.162, and keep
 // lingering) and average pool and FC as two small launches instead of the fused head's 1024 workgroups that each pool

@@ -116,7 +116,10 @@ constexpr unsigned kWholeRange = 0x80000000u;
 // groups of 32 (the workgroup's filter block is 32*WF filters), WK K groups.  Four waves: two workgroups per CU;
 // eight waves: one, whose waves w and w + 4 share a SIMD -- one of each pixel group, so that a tile of seven
 // rows (four + three) loads all SIMDs alike.
-template <int PG, int WF, int WK, bool ACT>
+//
+// RES: a layer of one channel slab (64 channels) has kSteps weight fragments per wave in all; they stay in registers for
+// the life of the workgroup instead of passing through the ring again for every tile.
+template <int PG, int WF, int WK, bool ACT, bool RES = false>
 __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv3x3_f16_stream_kernel(
     const void* in_p, const void* wf_p, unsigned G_p, unsigned div_p, unsigned mdiv_p, unsigned mS32_p, unsigned n_tiles_p,
     unsigned flags_p, unsigned N_TH_p, unsigned geom_p, unsigned pixB_p, unsigned rowx_rnseg_p, const StreamArgs::Tail tail) {
@@ -132,11 +135,13 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
   constexpr int NOWN = 4 / WK;       // pixel groups of 32 slots a wave finishes in the epilogue
   constexpr int BF = 32 * WF;        // filters per workgroup
   static_assert(kSteps % kRing == 0 || kRing % kSteps == 0, "the weight ring must tile a stage");
+  constexpr int kW = RES ? kSteps : kRing;  // weight fragments a wave holds
   constexpr int kPieceSteps = KPG >= 2 ? 9 : 5;  // K steps of a stage that carry the next patch's load instructions
   static_assert(kPieceSteps + 1 < kSteps, "the last piece is loaded in step kPieceSteps, the residual rows one step later");
   // weight refills younger than the last patch piece (loaded in step kPieceSteps, ahead of that step's refill) at the end of
   // a stage: what the wait for the patch may leave in flight
-  constexpr int kYoung = kSteps - kPieceSteps < kRing ? kSteps - kPieceSteps : kRing;
+  // (resident weights: no refills; the residual rows' loads of the stage are what follows the last piece)
+  constexpr int kYoung = RES ? 2 * NOWN : (kSteps - kPieceSteps < kRing ? kSteps - kPieceSteps : kRing);
   extern __shared__ __align__(16) unsigned char smem[];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -144,7 +149,7 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
   const int pg = wave / 4, wf = (wave % 4) % WF, wk = (wave % 4) / WF;
   const int lrow = lane & 31, lchunk = lane >> 5;
 
-  const int tstep = (int)(a.tstep_nslab_flags & 0xffffu), nslab = (int)((a.tstep_nslab_flags >> 16) & 0xffu);
+  const int tstep = (int)(a.tstep_nslab_flags & 0xffffu), nslab = RES ? 1 : (int)((a.tstep_nslab_flags >> 16) & 0xffu);
   const bool by_filter = (a.tstep_nslab_flags >> 24) & 1u, aligned = (a.tstep_nslab_flags >> 25) & 1u;
   const unsigned top = (a.tstep_nslab_flags >> 26) & 1u;
   const unsigned N = a.N_TH & 0xffffffu, TH = a.N_TH >> 24;
@@ -176,7 +181,7 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
   const int wbase = ((fb * WF + wf) * niter * 4 + wk * KPG) * 1024;
   const unsigned wlane = lane * 16;
   const int wwrap = niter * 4096;
-  u32x4 wring[kRing];
+  u32x4 wring[kW];
   // step L (counted over the whole stream of the wave, KPG per iteration) lives at wbase + (L / KPG) * 4096 + (L % KPG) * 1024
   auto wload_at = [&](int soff) { return __builtin_amdgcn_raw_buffer_load_b128(rs_wf, wlane, wbase + soff, 0); };
   auto ring_fill = [&](auto q_c) {
@@ -267,12 +272,14 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
   patch_begin(0, 0);
   patch_all();
   __builtin_amdgcn_sched_barrier(0);
-  ring_fill(std::integral_constant<int, 3>());
-  ring_fill(std::integral_constant<int, 4>());
-  ring_fill(std::integral_constant<int, 5>());
-  ring_fill(std::integral_constant<int, 6>());
-  ring_fill(std::integral_constant<int, 7>());
-  ring_fill(std::integral_constant<int, 8>());
+  auto ring_rest = [&](auto self, auto q_c) -> void {
+    constexpr int q = decltype(q_c)::value;
+    if constexpr (q < kW) {
+      ring_fill(q_c);
+      self(self, std::integral_constant<int, q + 1>());
+    }
+  };
+  ring_rest(ring_rest, std::integral_constant<int, 3>());
   __builtin_amdgcn_sched_barrier(0);
 
   // ---- everything below needs the rest of the arguments ----
@@ -328,8 +335,8 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
   tile_outputs(tile);
 
   floatx16 acc[4];
-  // the first patch is older than the six fragments and the two scale / shift loads requested after it
-  __builtin_amdgcn_s_waitcnt(vmcnt_only(kRing - 1));
+  // the first patch is older than the kW - 3 fragments and the two scale / shift loads requested after it
+  __builtin_amdgcn_s_waitcnt(vmcnt_only(kW - 1));
   __syncthreads();
 
   int stage_no = 0;
@@ -340,7 +347,7 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
   for (;;) {
     const int next_tile = tile + tstep;
     for (int slab = 0; slab < nslab; ++slab) {
-      const bool last = slab + 1 == nslab;
+      const bool last = RES || slab + 1 == nslab;
       // The patch of the next stage goes into the other buffer.  After the last tile the same instructions
       // are issued with descriptors of no bytes (same count on every path; no memory traffic).
       // the cell offsets of the next tile's patch replace this tile's once its last slab has been requested
@@ -379,7 +386,7 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
           constexpr int PPS = (kLoadsPerWave + kPieceSteps - 1) / kPieceSteps;  // patch pieces per step: 1 or 2
           constexpr int nx = st + kRing, nt = nx / KPG, nk = nx % KPG;
           static_assert(nt < 18, "the ring reaches at most into the next stage");
-          const u32x4 wfrag = wring[st % kRing];
+          const u32x4 wfrag = wring[RES ? st : st % kRing];
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const bool rowlive = PG == 1 || j < nrows;  // a pixel group may hold fewer rows (uniform per wave)
@@ -417,7 +424,7 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
                 rv[j % NOWN][1] = __builtin_amdgcn_raw_buffer_load_b128(rs_res, obase[j % NOWN], 16, 0);
               }
             }
-            if (j == 3) {
+            if (j == 3 && !RES) {
               // refill this ring slot with the fragment kRing steps further down the stream
               if constexpr (nt < 9) {
                 wring[st % kRing] = wload_at(wo + nt * 4096 + nk * 1024);
@@ -497,6 +504,15 @@ __global__ __launch_bounds__(64 * PG * WF * WK) __attribute__((amdgpu_waves_per_
             }
           }
         }
+      }
+      if constexpr (RES) {
+        // Without refills nothing younger than the residual rows' loads is ever waited for: on the paths that do not
+        // read them (no residual -- the loads still go out, against a descriptor of no bytes -- or a slot group of
+        // another wave) they would stay pending in the compiler's books, and the next tile's first reuse of their
+        // registers would wait for everything in flight, this tile's stores included.  A use here settles them on
+        // every path.
+#pragma unroll
+        for (int o = 0; o < NOWN; ++o) asm volatile("" : "+v"(rv[o][0]), "+v"(rv[o][1]));
       }
       floatx4 sc4[4], sh4[4];
 #pragma unroll
@@ -663,7 +679,14 @@ bool stream_config(int N, int H, int W, int C, int F, bool act, int only_pg, Str
     const int per_cu = c.PG == 1 ? 2 : 1;
     // as many workgroups per filter block as the CUs hold, evened out so that all of them walk the same number of
     // tiles (896 tiles on 512 places: 448 workgroups of two tiles, not 384 of two and 128 of one)
-    const int places = std::max(1, 256 * per_cu / c.FB), rounds = (c.geo.n_tiles + places - 1) / places;
+    // A one-slab layer in the 64-filter form keeps its weights in registers (RES): the longer a workgroup lives, the
+    // fewer fragments cross the vector-memory path.  With passes in flight, where a launch need not fill the chip on
+    // its own, its tiles go to half the places (ResNet-18's layer1 at batch 32, four passes in flight, same box: 448
+    // workgroups of two tiles 207.5 k images/s, 299 of three 211.9 k, 224 of four 212.6 k, 180 of five 213.2 k,
+    // 128 of seven 193 k; one pass at a time the 224 cost 2 % of the pass).
+    const bool resident = C == 64 && c.WF == 2 && c.PG == 1 && !act;
+    const int per_cu_places = (resident && overlap_hint() >= 3) ? 128 * per_cu : 256 * per_cu;
+    const int places = std::max(1, per_cu_places / c.FB), rounds = (c.geo.n_tiles + places - 1) / places;
     c.Wpf = (c.geo.n_tiles + rounds - 1) / rounds;
     const long long wgs = (long long)c.FB * c.Wpf;
     const long long wg_per_cu = (wgs + 255) / 256;  // on the busiest CU
@@ -742,14 +765,16 @@ bool conv3x3_stream_applicable(const IgemmArgs& a, int in_dt, int out_dt) {
   const long long fine_wgs = (long long)c.geo.n_tiles * (a.F / 32);
   // With three or more passes in flight (overlap_hint) a ReLU layer whose filter count rules out the 128-filter form goes
   // to the patch kernel, whose 256-slot workgroups hold fewer slots for the same work than the 64-filter form here
-  // (ResNet-18's layer1 at batch 32, four passes in flight: 0.161 against 0.165 ms per pass).
-  if (!all && overlap_hint() >= 3 && a.relu <= kActRelu && c.WF != 4) return false;
+  // (ResNet-18's layer1 at batch 32, four passes in flight: 0.161 against 0.165 ms per pass) -- unless it is a one-slab
+  // layer, whose 64-filter form keeps the weights in registers (204.4 k images/s with layer1 on the patch kernel,
+  // 212.6 k here, same box).
+  if (!all && overlap_hint() >= 3 && a.relu <= kActRelu && c.WF != 4 && !(a.C == 64 && c.WF == 2 && c.PG == 1)) return false;
   return all || (fine_wgs >= 160 && c.geo.TH * a.W >= 96);
 }
 
-template <int PG, int WF, int WK, bool ACT>
+template <int PG, int WF, int WK, bool ACT, bool RES = false>
 static void launch_stream_cfg(const StreamArgs& a, int grid, double flops, double bytes, const char* tag, hipStream_t s) {
-  auto kern = conv3x3_f16_stream_kernel<PG, WF, WK, ACT>;
+  auto kern = conv3x3_f16_stream_kernel<PG, WF, WK, ACT, RES>;
   constexpr int NW = PG * WF * WK;
   constexpr int smem = 2 * patch_bytes(NW) + 2 * 32 * WF * 4;
   static const bool attr = [&] {
@@ -802,6 +827,7 @@ bool launch_conv3x3_stream(const IgemmArgs& g, hipStream_t s) {
     else launch_stream_cfg<1, 1, 4, false>(a, grid, flops, bytes, "conv3x3_stream<f16,1x1x4>", s);
   } else {
     if (act) launch_stream_cfg<1, 2, 2, true>(a, grid, flops, bytes, "conv3x3_stream<f16,1x2x2,act>", s);
+    else if (g.C == 64) launch_stream_cfg<1, 2, 2, false, true>(a, grid, flops, bytes, "conv3x3_stream<f16,1x2x2,res>", s);
     else launch_stream_cfg<1, 2, 2, false>(a, grid, flops, bytes, "conv3x3_stream<f16,1x2x2>", s);
   }
   NNCV_HIP_CHECK(hipGetLastError());

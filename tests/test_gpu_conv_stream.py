@@ -19,7 +19,9 @@ pytestmark = pytest.mark.gpu
 CASES = [
     (8, 28, 28, 128, 128, True, True, abi.ACT_RELU, "conv3x3_stream<f16,1x1x4>"),      # 56 tiles x 4 filter groups, two slabs
     (12, 14, 14, 256, 256, True, True, abi.ACT_RELU, "conv3x3_stream<f16,1x1x4>"),     # images one zero row apart, four slabs
-    (20, 56, 56, 64, 64, True, False, abi.ACT_RELU, "conv3x3_stream<f16,1x2x2>"),      # 560 tiles: workgroups walk two tiles
+    (20, 56, 56, 64, 64, True, False, abi.ACT_RELU, "conv3x3_stream<f16,1x2x2,res>"),  # 560 tiles: workgroups walk two tiles; one slab: weights stay in registers
+    (37, 56, 56, 64, 64, True, True, abi.ACT_RELU, "conv3x3_stream<f16,1x2x2,res>"),   # 1036 tiles: three tiles on the same fragments, residual
+    (16, 56, 56, 64, 64, False, True, abi.ACT_NONE, "conv3x3_stream<f16,1x2x2,res>"),  # one tile per workgroup, no BatchNorm
     (58, 28, 28, 64, 128, True, True, abi.ACT_RELU, "conv3x3_stream<f16,1x4x1>"),      # 406 workgroups of 128 filters, no K groups
     (10, 23, 17, 192, 160, False, True, abi.ACT_NONE, "conv3x3_stream<f16,1x1x4>"),    # oblong, 32-filter groups only, no BatchNorm
     (6, 40, 40, 128, 128, True, False, abi.ACT_SILU, "conv3x3_stream<f16,1x2x2,act>"),
@@ -45,7 +47,8 @@ OVERLAP_CASES = [
     (8, 28, 28, 128, 128, True, True, abi.ACT_RELU, "conv3x3_stream<f16,1x4x1>"),      # 56 workgroups, two slabs
     (12, 14, 14, 256, 256, True, True, abi.ACT_RELU, "conv3x3_stream<f16,1x4x1>"),     # 40 workgroups across image borders, four slabs
     (5, 97, 31, 64, 128, True, False, abi.ACT_RELU, "conv3x3_stream<f16,1x4x1>"),      # short last tile of an image
-    (20, 56, 56, 64, 64, True, False, abi.ACT_RELU, "conv3x3_patch<f16,4,1>"),         # 64 filters: the patch kernel's 256-slot form
+    (20, 56, 56, 64, 64, True, True, abi.ACT_RELU, "conv3x3_stream<f16,1x2x2,res>"),   # one slab: resident weights, 187 workgroups of three tiles
+    (20, 56, 56, 128, 64, True, False, abi.ACT_RELU, "conv3x3_patch<f16,2,2>"),        # 64 filters, two slabs: the patch kernel
     (6, 40, 40, 128, 128, True, True, abi.ACT_HARDSWISH, "conv3x3_stream<f16,1x2x2,act>"),  # other activations keep their form
 ]
 

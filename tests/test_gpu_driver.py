@@ -215,7 +215,7 @@ def test_two_handles_on_two_streams_run_concurrently_and_stay_exact(blob, dt):
 
 def test_overlap_hint_changes_the_launch_shapes_not_the_results(blob):
     """nncv_hip_set_overlap_hint(4): the planners switch to the forms meant for several passes in flight (128-filter stream
-    form on layer2 / layer3, layer1 on the patch kernel, average pool and FC as separate launches), the logits stay within
+    form on layer2 / layer3, layer1 on the form that keeps its weights in registers, average pool and FC as separate launches), the logits stay within
     the fp16 bar of the oracle with its top-1, four handles on four streams each reproduce the bits of a pass run alone,
     and hint 1 brings the usual shapes back."""
     import torch
@@ -247,7 +247,8 @@ def test_overlap_hint_changes_the_launch_shapes_not_the_results(blob):
         print("hint 4:", rep, flush=True)
         count = lambda r, prefix: sum(v for k, v in r.items() if k.startswith(prefix))
         assert rep.get("conv3x3_stream<f16,1x4x1>", 0) == 6            # layer2 and layer3
-        assert count(rep, "conv3x3_patch") == 7 and count(rep, "conv3x3_stream") == 6  # layer1 joins layer4 on the patch kernel
+        assert rep.get("conv3x3_stream<f16,1x2x2,res>", 0) == 4        # layer1: one channel slab, weights resident in registers
+        assert count(rep, "conv3x3_patch") == 3 and count(rep, "conv3x3_stream") == 10  # layer4 stays on the patch kernel
         assert count(rep, "conv3x3s2_patch") == 3 and count(rep, "igemm") == 1  # the FC of the split head
         assert "avgpool_fc" not in rep and rep.get("global_avgpool", 0) == 1
         want = oracle.resnet18_forward(xs[0][:4], hb)

@@ -82,7 +82,7 @@ DOMINANT_LAYER = {
 # script, scaled by the same counters' reading for a device copy of known size (factor 2.0 for
 # FETCH_SIZE, 1.0 for WRITE_SIZE on this part).
 DOMINANT_TRAFFIC = {  # profiles/resnet18_fp16_bs32_hbm_counters.txt, launches without a residual input
-    "conv3x3_stream<f16,1x2x2>": (8954 + 6272) * 1024,
+    "conv3x3_stream<f16,1x2x2>": (8772 + 6272) * 1024,
     "conv3x3_patch<f16,2,2>": (8746 + 6272) * 1024,
     "conv3x3_patch<f16,4,1>": (13341 + 12544) * 1024,
     "conv3x3_patch<f16,1,4>": (17301 + 1568) * 1024,
@@ -91,7 +91,7 @@ DOMINANT_TRAFFIC = {  # profiles/resnet18_fp16_bs32_hbm_counters.txt, launches w
 
 # the same for the launch plan of three or more passes in flight
 IN_FLIGHT_TRAFFIC = {  # profiles/resnet18_fp16_bs32_in_flight_plan_hbm_counters.txt, the layer alone, no residual input
-    "conv3x3_stream<f16,1x4x1>": (8980 + 6272) * 1024,
+    "conv3x3_stream<f16,1x4x1>": (8835 + 6272) * 1024,
 }
 
 

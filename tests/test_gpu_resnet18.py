@@ -131,6 +131,25 @@ def test_fp16_layers_take_the_kernels_they_are_measured_on(blob):
     assert rel_l2(got, oracle.resnet18_forward(x, hb)) < FP16_REL_L2
 
 
+def test_fp16_stage_outputs_at_a_batch_whose_shortcuts_ride_along(blob):
+    """Batch 20 at 224x224: the stride-2 launches carry their block's 1x1 shortcut inside the workgroups of the 3x3
+    convolution, behind its epilogue.  Every stage's
+    output against the oracle, so that a wrong shortcut shows where it enters and not only in the logits."""
+    hb = synth.round_fp16(blob)
+    x = synth.round_fp16(synth.uniform(4007, (20, 3, 224, 224), 0.0, 1.0))
+    m = Model(hb, abi.F16, abi.ALGO_IGEMM)
+    xd = dev(x, abi.F16)
+    for stage in (1, 2, 3, 4):
+        want_logits, want_tap = oracle.resnet18_forward(x, hb, tap_layer=stage)
+        logits, tap = m(xd, tap_stage=stage)
+        got = nchw(host(tap))
+        errs = [rel_l2(got[i], want_tap[i]) for i in range(20)]
+        print("stage", stage, "worst image rel_l2 %.2e" % max(errs), flush=True)
+        assert max(errs) < FP16_REL_L2
+    assert rel_l2(host(logits), want_logits) < FP16_REL_L2
+    m.close()
+
+
 def test_graph_replay_matches_eager_every_time(blob):
     """The device entry point captures the forward into a HIP graph on the second call with the
     same buffers and replays it afterwards: every replay must equal the eager result, also when the

@@ -61,6 +61,7 @@ struct PatchArgs {
   int ldo, pix;          // elements between pixels of out (and residual) / of in: F and C unless they are slices of wider tensors
   int txw;               // TW | NTX << 16.  NTX = 1 (TW = the full output width) unless a row is too wide for the loader
   int rw_log;            // patch loader: 2^rw_log >= patch columns per loader row
+  int rowx;              // stride 1: spare bytes behind the cells of a patch row (see the row pitch in the kernel)
   int OH, OW;            // output size (stride 2; stride 1: H, W)
   int xcd_by_filter;     // XCD <- filter block instead of XCD <- tile range
   unsigned in_bytes, wf_bytes;
@@ -391,6 +392,11 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   const int OH = ST == 1 ? a.H : a.OH, OW = ST == 1 ? a.W : a.OW;
   const int PH = ST == 1 ? a.TH + 2 : 2 * a.TH + 1, PW = ST == 1 ? TW + 2 : 2 * TW + 1;
   const int PWh = TW + 1;
+  // Stride 1: consecutive slots wrap from the end of one tile row to the start of the next, and a 16-byte LDS read of a
+  // wave is free of bank conflicts when the 16-byte units of the slots continue the sequence of a row (9 units per
+  // slot) across the wrap.  A patch row is TW + 2 cells, two more than the tile row: with 14 spare units behind it the
+  // row pitch is 9 * TW units mod 16.  (7x7 tiles: 40 % of the LDS cycles of a launch were conflict cycles without it.)
+  const int RP = PW * kPitch + (ST == 1 ? a.rowx : 0);  // bytes from one patch row to the next (stride 1)
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in an SGPR
@@ -448,8 +454,8 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
     for (int i = 0; i < kPasses; ++i) {
       const int q = i * (NT / 8) + p8;
       const int r = q >> a.rw_log, px = q & rwm;
-      const int cell = ST == 1 ? __umul24(r, PW) + px : __umul24(2 * r + (px & 1), PWh) + (px >> 1);
-      const int dst = (int)__umul24(cell, kPitch) + pc;
+      const int dst = (ST == 1 ? (int)__umul24(r, RP) + (int)__umul24(px, kPitch)
+                               : (int)__umul24(__umul24(2 * r + (px & 1), PWh) + (px >> 1), kPitch)) + pc;
       *reinterpret_cast<u32x4*>(patch + (((px < PW) & (r < prows)) ? dst : dump)) = pregs[i];
     }
   };
@@ -495,8 +501,9 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
     const int ty = fast_div(rem, TW, a.inv_w, &tx);
     const bool ok = (sl < nslots) & ((n0 + nl) < a.N) & ((y0 + ty) < OH) & ((x0 + tx) < OW);
     // slots beyond the tile read pixel 0 of the patch; their results are never stored
-    const int cell = ST == 1 ? __umul24(__umul24(nl, PH) + ty, PW) + tx : __umul24(__umul24(nl, PH) + 2 * ty, 2 * PWh) + tx;
-    sbase[j] = (ok ? (int)__umul24(cell, kPitch) : 0) + (lchunk + 2 * wk * KPG) * 16;
+    const int celloff = ST == 1 ? (int)__umul24(__umul24(nl, PH) + ty, RP) + (int)__umul24(tx, kPitch)
+                                : (int)__umul24(__umul24(__umul24(nl, PH) + 2 * ty, 2 * PWh) + tx, kPitch);
+    sbase[j] = (ok ? celloff : 0) + (lchunk + 2 * wk * KPG) * 16;
     obase[j] = ok ? (((n0 + nl) * OH + y0 + ty) * OW + x0 + tx) * a.ldo : -1;
   }
 
@@ -523,7 +530,7 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
 #pragma unroll
   for (int r = 0; r < 3; ++r)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) rowbase[r][j] = sbase[j] + r * (ST == 1 ? PW : 2 * PWh) * kPitch;
+    for (int j = 0; j < 2; ++j) rowbase[r][j] = sbase[j] + r * (ST == 1 ? RP : 2 * PWh * kPitch);
   const int odd_col = PWh * kPitch;  // stride 2: from an even column to the odd one right of it
   u32x4 ring[kDepth][2];
   auto ldp = [&](auto step_c) {
@@ -700,6 +707,7 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
 // most.  H, W: output size (= input size at stride 1).  Rows whose patch is wider than the loader
 // takes are cut into NTX column tiles of equal width.
 struct TilePlan { int TN, TH, TW, NTX, rw_log; };
+constexpr int kRowSpare = 14 * 16;  // (9 * TW - 9 * (TW + 2)) mod 16 units of 16 bytes
 static bool plan_tile_ntx(int st, int N, int H, int W_full, int ntx, int slots, int cap, int cover, TilePlan* t) {
   const int W = (W_full + ntx - 1) / ntx;
   const int PW = st == 1 ? W + 2 : 2 * W + 1;       // patch columns the loader walks
@@ -709,7 +717,10 @@ static bool plan_tile_ntx(int st, int N, int H, int W_full, int ntx, int slots, 
   while ((1 << lg) < PW) ++lg;
   if ((1 << lg) > 64 || W > slots) return false;
   const int max_rows = cover >> lg;  // patch rows the loader can cover
-  auto fits = [&](int tn, int th) { return tn * th * W <= slots && tn * prow(th) * cells <= cap && tn * prow(th) <= max_rows; };
+  // stride 1: every patch row carries kRowSpare spare bytes (the kernel's conflict-free row pitch)
+  auto fits = [&](int tn, int th) {
+    return tn * th * W <= slots && tn * prow(th) * (cells * kPitch + (st == 1 ? kRowSpare : 0)) <= cap * kPitch && tn * prow(th) <= max_rows;
+  };
   int thmax = 0;
   for (int th = 1; th <= H; ++th)
     if (fits(1, th)) thmax = th;
@@ -874,6 +885,7 @@ void launch_conv3x3_patch(const IgemmArgs& g, int in_dt, int out_dt, hipStream_t
   TilePlan tp;
   NNCV_REQUIRE(plan_patch(st, a.N, a.OH, a.OW, a.F, a.C * (int)dtype_size(in_dt) / 128, &ws, &tp), "conv3x3_patch: no tile fits");
   a.TN = tp.TN; a.TH = tp.TH; a.rw_log = tp.rw_log;
+  a.rowx = st == 1 ? kRowSpare : 0;
   a.txw = tp.TW | (tp.NTX << 16);
   a.tiles_y = ((a.OH + a.TH - 1) / a.TH) * tp.NTX;
   a.tiles = ((a.N + a.TN - 1) / a.TN) * a.tiles_y;

@@ -1,6 +1,8 @@
 // Bandwidth-bound helpers of the ResNet-18 path: pooling, layout packing and one-time parameter
 // preparation.  Activations are NHWC inside the library (channels contiguous), so every kernel
 // here maps lanes to the channel axis and moves 16 bytes per lane where the shape allows.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace nncv_hip {
@@ -299,47 +301,84 @@ void launch_global_avgpool_nhwc(const void* in, void* out, int dt, int N, int HW
 // ---------------------------------------------------------------------------------------------
 // Network head in one launch: global average pool (sum over the image, one divide,
 // tests/Nets/Res18.mlir:609-614) and the 512 -> F fully connected layer with bias (:615-628).
-// A workgroup = one image x a slice of the F outputs.  Phase 1: the 256 threads sum the image's
-// pixels, two channels each (one coalesced kilobyte per pixel), fp32, and leave the 512 means in
-// LDS; the pooled vector is never rounded to the storage type.  Phase 2: a wave takes one output
-// at a time, its 64 lanes each hold 8 of the 512 means and read 8 consecutive weights (the whole
-// filter row is one contiguous kilobyte), and a shuffle tree adds the 64 partial dot products.
-// Slices recompute the (cheap, L2-resident) pooling instead of synchronising across workgroups.
+// A workgroup = one image x a slice of the F outputs.  Phase 1: a wave sums every fourth pixel of the
+// image, a lane eight channels of it (16-byte loads: one kilobyte per instruction), fp32, in pixel
+// order; the four waves' sums meet in LDS and are added in wave order, one divide; the pooled vector
+// is never rounded to the storage type.  Phase 2: a wave takes eight outputs per trip, its 64 lanes
+// each hold 8 of the 512 means and read 8 consecutive weights of each filter (a filter row is one
+// contiguous kilobyte); the eight dot products are added over the lanes together (see below).
+// Slices recompute the pooling instead of synchronising across workgroups.
 // ---------------------------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void avgpool_fc_kernel(const T* __restrict__ in, const T* __restrict__ w,
-                                                         const float* __restrict__ bias, float* __restrict__ out, int HW,
+                                                         const float* __restrict__ bias, float* __restrict__ out, int N, int HW,
                                                          int F, int f_per_block) {
-  __shared__ float mean[512];
+  // images per workgroup.  More would read the filters less often (once per IG images); measured at batch 32 with slices
+  // of 64 outputs: 6.2 us with one, 6.7 with two, 9.0 with four (longer chains per workgroup, fewer workgroups).
+  constexpr int IG = 1;
+  typedef float floatx4 __attribute__((ext_vector_type(4)));
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+  __shared__ __align__(16) float part[IG][4][512];  // per image and wave: the sums over the wave's pixels
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n = blockIdx.y;
+  const int n0 = blockIdx.y * IG;
   {
-    typedef T V2 __attribute__((ext_vector_type(2)));
-    const V2* src = reinterpret_cast<const V2*>(in + (long long)n * HW * 512) + tid;
-    float s0 = 0.0f, s1 = 0.0f;
-    int p = 0;
-    for (; p + 16 <= HW; p += 16) {  // sixteen loads in flight; the additions stay in pixel order
-      V2 v[16];
+    // A wave takes every fourth pixel, a lane eight channels of it: one kilobyte (fp32: two) per load instruction.  (Two
+    // channels per lane, 4-byte loads, kept the vector-memory path busy for a quarter of the instructions' worth of
+    // data: 5.4 of the launch's 7.8 us at batch 32.)  Through buffer descriptors of exactly one image each (none for an
+    // image past N): what lies past the end reads as zeros, and a sum that started at +0 is the same with +0 added.
+    typedef T V8 __attribute__((ext_vector_type(8)));
+    constexpr int PB = 16 / IG;  // pixels per wave and trip
+    const unsigned pix_bytes = 512u * (unsigned)sizeof(T), img_bytes = (unsigned)HW * pix_bytes;
+    const unsigned loff = (unsigned)lane * 8u * (unsigned)sizeof(T);
+    __amdgpu_buffer_rsrc_t rs[IG];
+    float ps[IG][8];
 #pragma unroll
-      for (int u = 0; u < 16; ++u) v[u] = src[(long long)(p + u) * 256];
+    for (int g = 0; g < IG; ++g) {
+      const bool have = n0 + g < N;
+      rs[g] = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(in + (long long)(have ? n0 + g : 0) * HW * 512), 0, have ? img_bytes : 0u, 0x00020000);
 #pragma unroll
-      for (int u = 0; u < 16; ++u) {
-        s0 += (float)v[u][0];
-        s1 += (float)v[u][1];
-      }
+      for (int e = 0; e < 8; ++e) ps[g][e] = 0.0f;
     }
-    for (; p < HW; ++p) {
-      const V2 v = src[(long long)p * 256];
-      s0 += (float)v[0];
-      s1 += (float)v[1];
+    for (int p = wave; p < HW; p += 4 * PB) {  // the additions of a wave stay in pixel order
+      V8 v[IG][PB];
+#pragma unroll
+      for (int g = 0; g < IG; ++g)
+#pragma unroll
+        for (int u = 0; u < PB; ++u) {
+          const unsigned off = (unsigned)(p + 4 * u) * pix_bytes + loff;
+          if constexpr (sizeof(T) == 2) {
+            v[g][u] = __builtin_bit_cast(V8, __builtin_amdgcn_raw_buffer_load_b128(rs[g], off, 0, 0));
+          } else {
+            typedef unsigned u32x8 __attribute__((ext_vector_type(8)));
+            const u32x4 lo = __builtin_amdgcn_raw_buffer_load_b128(rs[g], off, 0, 0), hi = __builtin_amdgcn_raw_buffer_load_b128(rs[g], off + 16u, 0, 0);
+            v[g][u] = __builtin_bit_cast(V8, u32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]});
+          }
+        }
+#pragma unroll
+      for (int g = 0; g < IG; ++g)
+#pragma unroll
+        for (int u = 0; u < PB; ++u)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) ps[g][e] += (float)v[g][u][e];
     }
-    mean[2 * tid] = s0 / (float)HW;
-    mean[2 * tid + 1] = s1 / (float)HW;
+#pragma unroll
+    for (int g = 0; g < IG; ++g) {
+      *reinterpret_cast<floatx4*>(&part[g][wave][lane * 8]) = floatx4{ps[g][0], ps[g][1], ps[g][2], ps[g][3]};
+      *reinterpret_cast<floatx4*>(&part[g][wave][lane * 8 + 4]) = floatx4{ps[g][4], ps[g][5], ps[g][6], ps[g][7]};
+    }
   }
   __syncthreads();
-  float m[8];
+  float m[IG][8];  // the means of this lane's eight channels: the four waves' sums in wave order, one divide
 #pragma unroll
-  for (int e = 0; e < 8; ++e) m[e] = mean[lane * 8 + e];
+  for (int g = 0; g < IG; ++g)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      floatx4 a = *reinterpret_cast<const floatx4*>(&part[g][0][lane * 8 + 4 * h]);
+#pragma unroll
+      for (int k = 1; k < 4; ++k) a += *reinterpret_cast<const floatx4*>(&part[g][k][lane * 8 + 4 * h]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) m[g][4 * h + e] = a[e] / (float)HW;
+    }
   const int f_begin = blockIdx.x * f_per_block;
   const int f_end = f_begin + f_per_block < F ? f_begin + f_per_block : F;
   typedef T V8 __attribute__((ext_vector_type(8)));
@@ -350,16 +389,47 @@ __global__ __launch_bounds__(256) void avgpool_fc_kernel(const T* __restrict__ i
       const int f = f0 + 4 * u < f_end ? f0 + 4 * u : f0;
       wv[u] = *reinterpret_cast<const V8*>(w + (long long)f * 512 + lane * 8);
     }
+    // The V = 8 * IG dot products of a trip are added over the 64 lanes together: at distance 32 a lane keeps the lower or
+    // the upper half of the values (by its bit 5), hands the other half to its partner and adds what it receives, and so
+    // on at 16, 8 ...; V - 1 lane exchanges and a few more for the bits that are left, instead of six per value, and
+    // the same additions (own + partner's, the same pairs at the same distances: bit-identical to a tree per value).
+    // A lane ends with the sum of value (g, u) = (vi >> 3, vi & 7), vi read off its upper bits.
+    constexpr int V = 8 * IG;
+    int vi = 0, dd = 32;
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      float acc = 0.0f;
+    for (int n = V; n > 1; n >>= 1, dd >>= 1) vi += (lane & dd) ? n / 2 : 0;
+    const int gl = vi >> 3, fl = f0 + 4 * (vi & 7);
+    const bool writer = (lane & (2 * dd - 1)) == 0 && fl < f_end && n0 + gl < N;
+    const float bl = (bias && fl < f_end) ? bias[fl] : 0.0f;  // with the weights: fetched where it is added it is a trip to memory per output
+    float x[V];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc += m[e] * (float)wv[u][e];
+    for (int g = 0; g < IG; ++g)
 #pragma unroll
-      for (int d = 32; d >= 1; d >>= 1) acc += __shfl_xor(acc, d);
-      const int f = f0 + 4 * u;
-      if (lane == 0 && f < f_end) out[(long long)n * F + f] = acc + (bias ? bias[f] : 0.0f);
-    }
+      for (int u = 0; u < 8; ++u) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc += m[g][e] * (float)wv[u][e];
+        x[g * 8 + u] = acc;
+      }
+    // (compile-time recursion: as a loop over halving n the compiler kept x[] indexed at run time)
+    auto fold = [&](auto self, auto n_c, auto d_c) -> void {
+      constexpr int n = decltype(n_c)::value, d = decltype(d_c)::value;
+      if constexpr (n > 1) {
+        const bool hi = (lane & d) != 0;
+#pragma unroll
+        for (int v = 0; v < n / 2; ++v) {
+          const float keep = hi ? x[v + n / 2] : x[v];
+          const float send = hi ? x[v] : x[v + n / 2];
+          x[v] = keep + __shfl_xor(send, d);
+        }
+        self(self, std::integral_constant<int, n / 2>(), std::integral_constant<int, d / 2>());
+      } else if constexpr (d >= 1) {
+        x[0] += __shfl_xor(x[0], d);
+        self(self, n_c, std::integral_constant<int, d / 2>());
+      }
+    };
+    fold(fold, std::integral_constant<int, V>(), std::integral_constant<int, 32>());
+    if (writer) out[(long long)(n0 + gl) * F + fl] = x[0] + bl;
   }
 }
 
@@ -367,15 +437,17 @@ __global__ __launch_bounds__(256) void avgpool_fc_kernel(const T* __restrict__ i
 void launch_avgpool_fc(const void* in, const void* w, const float* bias, float* out, int dt, int N, int HW, int C, int F,
                        hipStream_t s) {
   NNCV_REQUIRE(C == 512, "avgpool_fc: the head is built for 512 channels");
-  NNCV_REQUIRE(N > 0 && N <= 65535 && HW > 0 && F > 0, "avgpool_fc: bad shape");
-  const int fpb = 32;  // one trip of eight filters per wave: the kernel is a chain of memory latencies, so keep it short
+  NNCV_REQUIRE(N > 0 && N <= 65535 && HW > 0 && F > 0 && (long long)HW * 512 * (long long)dtype_size(dt) < (1ll << 31), "avgpool_fc: bad shape");
+  // Slices of 64 outputs (two trips of eight filters per wave) once the images alone fill the CUs twice over, 32 (one
+  // trip: the kernel is a chain of memory latencies) below that.  Batch 32: 6.5 us with 32, 6.2 with 64, 7.5 with 128.
+  const int fpb = N >= 16 ? 64 : 32;
   dim3 grid((F + fpb - 1) / fpb, N);
   const double es = (double)dtype_size(dt);
   ProfScope prof("avgpool_fc", 2.0 * N * F * 512.0, es * ((double)N * HW * 512 + (double)F * 512) + 4.0 * N * F, s);
   if (dt == kF16)
-    hipLaunchKernelGGL((avgpool_fc_kernel<half_t>), grid, dim3(256), 0, s, (const half_t*)in, (const half_t*)w, bias, out, HW, F, fpb);
+    hipLaunchKernelGGL((avgpool_fc_kernel<half_t>), grid, dim3(256), 0, s, (const half_t*)in, (const half_t*)w, bias, out, N, HW, F, fpb);
   else
-    hipLaunchKernelGGL((avgpool_fc_kernel<float>), grid, dim3(256), 0, s, (const float*)in, (const float*)w, bias, out, HW, F, fpb);
+    hipLaunchKernelGGL((avgpool_fc_kernel<float>), grid, dim3(256), 0, s, (const float*)in, (const float*)w, bias, out, N, HW, F, fpb);
   NNCV_HIP_CHECK(hipGetLastError());
 }
 

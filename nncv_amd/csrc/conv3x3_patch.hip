@@ -495,16 +495,23 @@ __global__ __launch_bounds__(64 * WS * WK) __attribute__((amdgpu_waves_per_eu(2,
   int obase[2];  // element offset of the slot's output pixel row, or -1
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
-    const int sl = ws * 64 + j * 32 + lrow;
+    const int sl0 = ws * 64 + j * 32 + lrow;
+    // a slot beyond the tile reads with the slot 16, 32 ... before it (the same LDS banks as if it had a pixel: fifteen
+    // lanes on one cell were a bank conflict per read on 7x7 tiles); its results are never stored
+    int sl = sl0;
+    if (sl0 >= nslots) {
+      const int back = (((sl0 - nslots) >> 4) + 1) << 4;
+      sl = sl0 >= back ? sl0 - back : 0;
+    }
     int nl = 0, rem = sl, tx;
     if (a.TN > 1) nl = fast_div(sl, a.TH * TW, a.inv_thw, &rem);
     const int ty = fast_div(rem, TW, a.inv_w, &tx);
     const bool ok = (sl < nslots) & ((n0 + nl) < a.N) & ((y0 + ty) < OH) & ((x0 + tx) < OW);
-    // slots beyond the tile read pixel 0 of the patch; their results are never stored
+    // slots whose pixel lies outside the image read pixel 0 of the patch
     const int celloff = ST == 1 ? (int)__umul24(__umul24(nl, PH) + ty, RP) + (int)__umul24(tx, kPitch)
                                 : (int)__umul24(__umul24(__umul24(nl, PH) + 2 * ty, 2 * PWh) + tx, kPitch);
     sbase[j] = (ok ? celloff : 0) + (lchunk + 2 * wk * KPG) * 16;
-    obase[j] = ok ? (((n0 + nl) * OH + y0 + ty) * OW + x0 + tx) * a.ldo : -1;
+    obase[j] = (ok && sl0 < nslots) ? (((n0 + nl) * OH + y0 + ty) * OW + x0 + tx) * a.ldo : -1;
   }
 
   // [filter half][pixel half]; with NI = 1 only acc[0] is used.  The first step of the first slab starts the sums from a

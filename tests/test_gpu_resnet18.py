@@ -207,6 +207,24 @@ def test_fp16_fused_stem_and_pool(blob, shape):
     assert e_log < FP16_REL_L2
 
 
+@pytest.mark.parametrize("dt", [abi.F16, abi.F32])
+def test_head_on_a_final_image_of_many_pixels(blob, dt):
+    """416x480 in: the last stage is 13x15 = 195 pixels, so the head's pooling walks several trips of sixteen pixels per
+    wave with a ragged last one (at 224x224 it is 49 pixels, one trip)."""
+    b = synth.round_fp16(blob) if dt == abi.F16 else blob
+    x = synth.uniform(4400, (1, 3, 416, 480), 0.0, 1.0)
+    if dt == abi.F16:
+        x = synth.round_fp16(x)
+    want = oracle.resnet18_forward(x, b)
+    m = Model(b, dt)
+    got = host(m(dev(x, dt)))
+    err = rel_l2(got, want)
+    print("head on 13x15, dtype", dt, "logits rel_l2 %.2e" % err, flush=True)
+    assert err < (FP16_REL_L2 if dt == abi.F16 else 1e-4)
+    assert got.argmax(1) == want.argmax(1)
+    m.close()
+
+
 def test_fp16_fused_stem_propagates_nan(blob):
     """arith.maximumf keeps NaN: a NaN pixel poisons exactly the pooled outputs whose windows see it."""
     hb = synth.round_fp16(blob)
